@@ -1,0 +1,187 @@
+/*
+ * svox_hip.h -- C ABI of libsvox_hip.so: N^3-tree point queries and differentiable volume
+ * rendering on AMD gfx950 (MI355X).
+ *
+ * Every entry point below replaces one function of the reference's pybind11 module `svox.csrc`
+ * (svox/csrc/svox.cpp:63-122).  Where the reference passes torch::Tensor members, this ABI passes
+ * raw device pointers plus sizes; where the reference allocates and returns a tensor, the caller
+ * passes the output buffer.  Nothing here depends on torch or on HIP headers: `stream` is a
+ * hipStream_t carried as void* (NULL = the null stream).
+ *
+ * Conventions
+ *   - all pointers are device pointers valid on the current HIP device unless stated otherwise;
+ *   - all arrays are dense and row-major (the reference requires contiguous tensors,
+ *     svox/csrc/include/data_spec.hpp:37-42);
+ *   - `dtype` selects the scalar type of every `void*` array in the call: SVOX_F32 or SVOX_F64
+ *     (the reference dispatches with AT_DISPATCH_FLOATING_TYPES);
+ *   - every function returns SVOX_OK (0) or a negative SvoxStatus; svox_last_error() returns a
+ *     per-thread message for the last failing call.  Launches are asynchronous on `stream`;
+ *   - the library never allocates or frees device memory.
+ */
+#ifndef SVOX_HIP_H_
+#define SVOX_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SVOX_ABI_VERSION 1
+
+typedef enum SvoxStatus {
+    SVOX_OK = 0,
+    SVOX_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
+    SVOX_ERR_BAD_SHAPE = -2,      /* a size is negative / zero where it may not be, or inconsistent */
+    SVOX_ERR_BAD_DTYPE = -3,      /* dtype is neither SVOX_F32 nor SVOX_F64 */
+    SVOX_ERR_UNSUPPORTED = -4,    /* valid in the reference but outside what this build covers */
+    SVOX_ERR_LAUNCH = -5,         /* hipGetLastError() after the launch was not hipSuccess */
+    SVOX_ERR_NO_DEVICE = -6       /* no usable HIP device */
+} SvoxStatus;
+
+typedef enum SvoxDType { SVOX_F32 = 0, SVOX_F64 = 1 } SvoxDType;
+
+/* svox/csrc/include/data_spec.hpp:44-49 */
+typedef enum SvoxDataFormat {
+    SVOX_FORMAT_RGBA = 0,
+    SVOX_FORMAT_SH = 1,
+    SVOX_FORMAT_SG = 2,
+    SVOX_FORMAT_ASG = 3
+} SvoxDataFormat;
+
+#define SVOX_MAX_BASIS_DIM 25 /* size of the reference's basis_fn array, rt_kernel.cu:250 */
+#define SVOX_MAX_OUT_DIM 16   /* widest rendered colour vector this build accumulates */
+
+/* TreeSpec, svox/csrc/include/data_spec.hpp:65-89 */
+typedef struct SvoxTreeSpec {
+    void* data;                  /* (capacity, N, N, N, data_dim) scalar; leaf records, sigma last */
+    const int32_t* child;        /* (capacity, N, N, N) relative child offset, 0 = leaf */
+    const int32_t* parent_depth; /* (capacity, 2): packed parent cell, node depth */
+    const void* extra_data;      /* (extra_rows, extra_cols) scalar for SG/ASG, else NULL */
+    const void* offset;          /* 3 scalars on the device, NULL = (0,0,0) */
+    const void* scaling;         /* 3 scalars on the device, NULL = (1,1,1) */
+    void* weight_accum;          /* (capacity, N, N, N) scalar, or NULL */
+    int64_t capacity;            /* M = child.shape[0] */
+    int32_t N;                   /* branching factor */
+    int32_t data_dim;            /* K */
+    int32_t extra_rows;
+    int32_t extra_cols;
+    int32_t weight_accum_max;    /* nonzero: max-reduce into weight_accum, zero: sum */
+    int32_t dtype;               /* SvoxDType of data/extra_data/offset/scaling/weight_accum */
+} SvoxTreeSpec;
+
+/* RaysSpec, svox/csrc/include/data_spec.hpp:51-63 */
+typedef struct SvoxRaysSpec {
+    const void* origins; /* (n_rays, 3) scalar */
+    const void* dirs;    /* (n_rays, 3) scalar */
+    const void* vdirs;   /* (n_rays, 3) scalar */
+    int64_t n_rays;
+} SvoxRaysSpec;
+
+/* CameraSpec, svox/csrc/include/data_spec.hpp:91-104 */
+typedef struct SvoxCameraSpec {
+    const void* c2w; /* device pointer, (3 or 4, 4) scalar; only the first 3 rows are read */
+    float fx;
+    float fy;
+    int32_t width;
+    int32_t height;
+} SvoxCameraSpec;
+
+/* RenderOptions, svox/csrc/include/data_spec.hpp:107-126 (bool widened to int32_t) */
+typedef struct SvoxRenderOptions {
+    float step_size;
+    float background_brightness;
+    int32_t format;    /* SvoxDataFormat */
+    int32_t basis_dim; /* -1 for RGBA */
+    int32_t ndc_width; /* < 0 disables NDC */
+    int32_t ndc_height;
+    float ndc_focal;
+    int32_t min_comp;
+    int32_t max_comp;
+    float sigma_thresh;
+    float stop_thresh;
+    int32_t density_softplus;
+    float rgb_padding;
+} SvoxRenderOptions;
+
+/* Per-launch march statistics written by svox_volume_render_stats (no counterpart in the
+ * reference; used to price a launch in algorithmic bytes). */
+typedef struct SvoxMarchStats {
+    uint64_t rays;            /* rays traced */
+    uint64_t rays_hit;        /* rays whose segment intersects the unit cube */
+    uint64_t samples;         /* leaf visits of the forward march */
+    uint64_t samples_shaded;  /* leaf visits with sigma > sigma_thresh */
+    uint64_t samples_bwd;     /* leaf visits of one backward march (no early stop) */
+    uint64_t samples_bwd_pos; /* of those, visits with sigma > 0 */
+    uint64_t levels;          /* child-table entries read by a root-to-leaf walk, forward march */
+    uint64_t reserved;
+} SvoxMarchStats;
+
+int svox_abi_version(void);
+const char* svox_last_error(void);
+const char* svox_status_string(int status);
+
+/* Debugging aid without a counterpart in the reference.  Bit 0: route every call to the generic
+ * kernels (any N, any dtype) even where a specialised octree kernel exists. */
+void svox_set_debug_flags(int flags);
+
+/* query_vertical(TreeSpec&, Tensor indices) -> (values, node_ids); svox/csrc/svox_kernel.cu:120-143.
+ * indices (n_points,3) scalar; values_out (n_points, data_dim) scalar; node_ids_out (n_points) int64. */
+int svox_query_vertical(const SvoxTreeSpec* tree, const void* indices, int64_t n_points,
+                        void* values_out, int64_t* node_ids_out, void* stream);
+
+/* query_vertical_backward(TreeSpec&, indices, grad_output) -> grad_data; svox_kernel.cu:160-182.
+ * grad_output (n_points, grad_dim); grad_data_out (capacity, N, N, N, grad_dim).  The reference
+ * returns a fresh zero-filled tensor; here the library zero-fills grad_data_out first unless
+ * `accumulate` is nonzero. */
+int svox_query_vertical_backward(const SvoxTreeSpec* tree, const void* indices, int64_t n_points,
+                                 const void* grad_output, int32_t grad_dim, void* grad_data_out,
+                                 int32_t accumulate, void* stream);
+
+/* assign_vertical(TreeSpec&, indices, values); svox_kernel.cu:145-158.  values (n_points, value_dim),
+ * value_dim <= data_dim.  Two points in one leaf race; the last writer wins, as in the reference. */
+int svox_assign_vertical(const SvoxTreeSpec* tree, const void* indices, int64_t n_points,
+                         const void* values, int32_t value_dim, void* stream);
+
+/* calc_corners(TreeSpec&, indexer) -> (n,3); svox_kernel.cu:184-203.  indexer (n_leaves,4) int64
+ * rows [node, x, y, z]; corners_out (n_leaves,3) scalar of tree->dtype. */
+int svox_calc_corners(const SvoxTreeSpec* tree, const int64_t* indexer, int64_t n_leaves,
+                      void* corners_out, void* stream);
+
+/* volume_render(TreeSpec&, RaysSpec&, RenderOptions&) -> (n_rays, out_dim); rt_kernel.cu:1019-1036.
+ * out_dim = svox_out_data_dim(opt->format, opt->basis_dim, tree->data_dim). */
+int svox_volume_render(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                       const SvoxRenderOptions* opt, void* out, void* stream);
+
+/* volume_render_image(TreeSpec&, CameraSpec&, RenderOptions&) -> (H, W, out_dim);
+ * rt_kernel.cu:1038-1057. */
+int svox_volume_render_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                             const SvoxRenderOptions* opt, void* out, void* stream);
+
+/* volume_render_backward(TreeSpec&, RaysSpec&, RenderOptions&, grad_output) -> zeros_like(data) +
+ * scatter; rt_kernel.cu:1059-1083.  grad_output (n_rays, out_dim); grad_data_out has the shape of
+ * tree->data and is zero-filled first unless `accumulate` is nonzero. */
+int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                                const SvoxRenderOptions* opt, const void* grad_output,
+                                void* grad_data_out, int32_t accumulate, void* stream);
+
+/* volume_render_image_backward(TreeSpec&, CameraSpec&, RenderOptions&, grad_output);
+ * rt_kernel.cu:1085-1109.  grad_output (H, W, out_dim). */
+int svox_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                                      const SvoxRenderOptions* opt, const void* grad_output,
+                                      void* grad_data_out, int32_t accumulate, void* stream);
+
+/* get_out_data_dim, rt_kernel.cu:1009-1015.  Returns -1 for an invalid combination. */
+int svox_out_data_dim(int32_t format, int32_t basis_dim, int32_t data_dim);
+
+/* No counterpart in the reference.  Walks the same marches as svox_volume_render (rays != NULL) or
+ * svox_volume_render_image (cam != NULL) and adds the visit counts of the launch into *stats_out
+ * (device pointer to one SvoxMarchStats, which the caller zeroes). */
+int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                             const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
+                             SvoxMarchStats* stats_out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SVOX_HIP_H_ */

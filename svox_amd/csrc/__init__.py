@@ -1,0 +1,391 @@
+"""svox_amd.csrc -- the operator module the Python layer calls.
+
+It presents the names of the reference's extension module `svox.csrc`
+(svox/csrc/svox.cpp:63-122): the four spec classes with the same attributes and the free functions
+`query_vertical`, `query_vertical_backward`, `assign_vertical`, `calc_corners`, `volume_render`,
+`volume_render_image`, `volume_render_backward`, `volume_render_image_backward`.  Each function
+checks its tensors the way the reference's `check()` methods do (svox/csrc/include/data_spec.hpp),
+allocates the outputs with the reference's shapes / dtypes / devices and calls the matching
+extern "C" entry point of libsvox_hip.so on torch's current stream.
+
+There is no CPU implementation here: tensors that are not on a GPU raise, and a missing library
+raises at the first call.
+"""
+import ctypes
+
+import torch
+
+from . import _abi
+from ._abi import FORMAT_ASG, FORMAT_RGBA, FORMAT_SG, FORMAT_SH  # noqa: F401
+
+
+class RaysSpec:
+    """svox/csrc/include/data_spec.hpp:51-63"""
+
+    def __init__(self):
+        self.origins = None
+        self.dirs = None
+        self.vdirs = None
+
+
+class TreeSpec:
+    """svox/csrc/include/data_spec.hpp:65-89.  `offset` / `scaling` may be None (identity)."""
+
+    def __init__(self):
+        self.data = None
+        self.child = None
+        self.parent_depth = None
+        self.extra_data = None
+        self.offset = None
+        self.scaling = None
+        self._weight_accum = None
+        self._weight_accum_max = False
+
+
+class CameraSpec:
+    """svox/csrc/include/data_spec.hpp:91-104"""
+
+    def __init__(self):
+        self.c2w = None
+        self.fx = 0.0
+        self.fy = 0.0
+        self.width = 0
+        self.height = 0
+
+
+class RenderOptions:
+    """svox/csrc/include/data_spec.hpp:107-126"""
+
+    def __init__(self):
+        self.step_size = 1e-3
+        self.background_brightness = 1.0
+        self.format = FORMAT_RGBA
+        self.basis_dim = -1
+        self.ndc_width = -1
+        self.ndc_height = -1
+        self.ndc_focal = 1.0
+        self.min_comp = 0
+        self.max_comp = 0
+        self.sigma_thresh = 0.0
+        self.stop_thresh = 0.0
+        self.density_softplus = False
+        self.rgb_padding = 0.0
+
+    def _pack(self):
+        return _abi.RenderOptionsC(
+            float(self.step_size), float(self.background_brightness), int(self.format),
+            int(self.basis_dim), int(self.ndc_width), int(self.ndc_height), float(self.ndc_focal),
+            int(self.min_comp), int(self.max_comp), float(self.sigma_thresh),
+            float(self.stop_thresh), int(bool(self.density_softplus)), float(self.rgb_padding))
+
+
+# --------------------------------------------------------------------------------------------
+# checks (CHECK_INPUT and friends, data_spec.hpp:37-42)
+# --------------------------------------------------------------------------------------------
+def _check_input(x, name):
+    if not isinstance(x, torch.Tensor):
+        raise RuntimeError(f"{name} must be a tensor")
+    if not x.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not x.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _numel(x):
+    return 0 if x is None else x.numel()
+
+
+def _dtype_code(dtype, name):
+    if dtype == torch.float32:
+        return _abi.SVOX_F32
+    if dtype == torch.float64:
+        return _abi.SVOX_F64
+    raise RuntimeError(f"{name} must be a float32 or float64 tensor, got {dtype}")
+
+
+def _same_dtype(x, dtype, name):
+    if x.dtype != dtype:
+        raise RuntimeError(f"expected scalar type {dtype} for {name} but found {x.dtype}")
+
+
+def _check_tree(tree):
+    """TreeSpec::check, data_spec.hpp:75-88, plus the shape facts the kernels rely on."""
+    _check_input(tree.data, "data")
+    _check_input(tree.child, "child")
+    _check_input(tree.parent_depth, "parent_depth")
+    if _numel(tree.extra_data):
+        _check_input(tree.extra_data, "extra_data")
+    if tree.offset is not None:
+        _check_input(tree.offset, "offset")
+    if tree.scaling is not None:
+        _check_input(tree.scaling, "scaling")
+    if _numel(tree._weight_accum):
+        _check_input(tree._weight_accum, "_weight_accum")
+    if tree.data.dim() != 5 or tree.child.dim() != 4 or tree.parent_depth.dim() != 2:
+        raise RuntimeError("data must be 5-D, child 4-D and parent_depth 2-D")
+    if tree.child.dtype != torch.int32 or tree.parent_depth.dtype != torch.int32:
+        raise RuntimeError("child and parent_depth must be int32 tensors")
+    if tuple(tree.data.shape[:4]) != tuple(tree.child.shape):
+        raise RuntimeError("data and child disagree on (capacity, N, N, N)")
+
+
+def _pack_tree(tree, dtype=None, need_data=True):
+    _check_tree(tree)
+    dt = tree.data.dtype if dtype is None else dtype
+    code = _dtype_code(dt, "data")
+    if need_data:
+        _same_dtype(tree.data, dt, "data")
+    spec = _abi.TreeSpecC()
+    spec.data = tree.data.data_ptr()
+    spec.child = tree.child.data_ptr()
+    spec.parent_depth = tree.parent_depth.data_ptr()
+    extra = tree.extra_data if _numel(tree.extra_data) else None
+    if extra is not None:
+        _same_dtype(extra, dt, "extra_data")
+        if extra.dim() != 2:
+            raise RuntimeError("extra_data must be 2-D")
+        spec.extra_data = extra.data_ptr()
+        spec.extra_rows, spec.extra_cols = int(extra.shape[0]), int(extra.shape[1])
+    else:
+        spec.extra_data = None
+        spec.extra_rows = spec.extra_cols = 0
+    for attr in ("offset", "scaling"):
+        t = getattr(tree, attr)
+        if t is not None:
+            _same_dtype(t, dt, attr)
+            if t.numel() != 3:
+                raise RuntimeError(f"{attr} must have 3 elements")
+            setattr(spec, attr, t.data_ptr())
+        else:
+            setattr(spec, attr, None)
+    wa = tree._weight_accum if _numel(tree._weight_accum) else None
+    if wa is not None:
+        _same_dtype(wa, dt, "_weight_accum")
+        if wa.numel() != tree.child.numel():
+            raise RuntimeError("_weight_accum must have one entry per cell of child")
+        spec.weight_accum = wa.data_ptr()
+    else:
+        spec.weight_accum = None
+    spec.weight_accum_max = int(bool(tree._weight_accum_max))
+    spec.capacity = int(tree.child.shape[0])
+    spec.N = int(tree.child.shape[1])
+    spec.data_dim = int(tree.data.shape[4])
+    spec.dtype = code
+    return spec
+
+
+def _check_indices(indices, name="indices"):
+    """check_indices, svox_kernel.cu:34-38"""
+    _check_input(indices, name)
+    if indices.dim() != 2:
+        raise RuntimeError(f"{name} must be 2-D")
+    if not indices.is_floating_point():
+        raise RuntimeError(f"{name} must be a floating point tensor")
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _call(name, *args):
+    lib = _abi.load_library()
+    rc = getattr(lib, name)(*args)
+    if rc != _abi.SVOX_OK:
+        msg = lib.svox_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"svox.{name[5:]}: {msg} ({lib.svox_status_string(rc).decode()})")
+
+
+def out_data_dim(fmt, basis_dim, data_dim):
+    """get_out_data_dim, rt_kernel.cu:1009-1015"""
+    if fmt != FORMAT_RGBA:
+        return (data_dim - 1) // basis_dim
+    return data_dim - 1
+
+
+# --------------------------------------------------------------------------------------------
+# queries
+# --------------------------------------------------------------------------------------------
+def query_vertical(tree, indices):
+    """(values (Q, K) like indices, node_ids (Q,) int64 on child's device); svox_kernel.cu:120-143"""
+    _check_indices(indices)
+    spec = _pack_tree(tree, indices.dtype)
+    if indices.shape[1] != 3:
+        raise RuntimeError("indices must be (Q, 3)")
+    Q, K = indices.shape[0], spec.data_dim
+    values = torch.empty((Q, K), dtype=indices.dtype, device=indices.device)
+    node_ids = torch.empty((Q,), dtype=torch.int64, device=tree.child.device)
+    with torch.cuda.device(indices.device):
+        _call("svox_query_vertical", ctypes.byref(spec), indices.data_ptr(), Q, values.data_ptr(),
+              node_ids.data_ptr(), _stream(indices.device))
+    return values, node_ids
+
+
+def query_vertical_backward(tree, indices, grad_output):
+    """zeros (M, N, N, N, grad_output.shape[1]) + scatter-add; svox_kernel.cu:160-182"""
+    _check_indices(indices)
+    _check_indices(grad_output, "grad_output")
+    _same_dtype(grad_output, indices.dtype, "grad_output")
+    spec = _pack_tree(tree, indices.dtype, need_data=False)
+    Q, Kg = indices.shape[0], int(grad_output.shape[1])
+    if grad_output.shape[0] != Q:
+        raise RuntimeError("grad_output must have one row per point")
+    N = spec.N
+    grad_data = torch.empty((spec.capacity, N, N, N, Kg), dtype=grad_output.dtype,
+                            device=grad_output.device)
+    with torch.cuda.device(indices.device):
+        _call("svox_query_vertical_backward", ctypes.byref(spec), indices.data_ptr(), Q,
+              grad_output.data_ptr(), Kg, grad_data.data_ptr(), 0, _stream(indices.device))
+    return grad_data
+
+
+def assign_vertical(tree, indices, values):
+    """store values into the leaves of the points; svox_kernel.cu:145-158"""
+    _check_indices(indices)
+    _check_indices(values, "values")
+    _same_dtype(values, indices.dtype, "values")
+    spec = _pack_tree(tree, indices.dtype)
+    if values.shape[0] != indices.shape[0]:
+        raise RuntimeError("values must have one row per point")
+    with torch.cuda.device(indices.device):
+        _call("svox_assign_vertical", ctypes.byref(spec), indices.data_ptr(), indices.shape[0],
+              values.data_ptr(), int(values.shape[1]), _stream(indices.device))
+
+
+def calc_corners(tree, indexer):
+    """(Q, 3) lower corners of the leaves [node, x, y, z]; svox_kernel.cu:184-203"""
+    spec = _pack_tree(tree, need_data=False)
+    _check_input(indexer, "indexer")
+    if indexer.dtype != torch.int64 or indexer.dim() != 2 or indexer.shape[1] != 4:
+        raise RuntimeError("indexer must be an int64 (Q, 4) tensor")
+    Q = indexer.shape[0]
+    out = torch.empty((Q, 3), dtype=tree.data.dtype, device=tree.data.device)
+    with torch.cuda.device(indexer.device):
+        _call("svox_calc_corners", ctypes.byref(spec), indexer.data_ptr(), Q, out.data_ptr(),
+              _stream(indexer.device))
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# rendering
+# --------------------------------------------------------------------------------------------
+def _pack_rays(rays, dtype):
+    """RaysSpec::check, data_spec.hpp:56-63"""
+    for name in ("origins", "dirs", "vdirs"):
+        t = getattr(rays, name)
+        _check_input(t, name)
+        if not t.is_floating_point():
+            raise RuntimeError(f"{name} must be a floating point tensor")
+        _same_dtype(t, dtype, name)
+        if t.dim() != 2 or t.shape[1] != 3:
+            raise RuntimeError(f"{name} must be (B, 3)")
+    B = rays.origins.shape[0]
+    if rays.dirs.shape[0] != B or rays.vdirs.shape[0] != B:
+        raise RuntimeError("origins, dirs and vdirs must have the same number of rays")
+    return _abi.RaysSpecC(rays.origins.data_ptr(), rays.dirs.data_ptr(), rays.vdirs.data_ptr(), B)
+
+
+def _pack_camera(cam, dtype):
+    """CameraSpec::check, data_spec.hpp:98-103"""
+    _check_input(cam.c2w, "c2w")
+    if not cam.c2w.is_floating_point():
+        raise RuntimeError("c2w must be a floating point tensor")
+    if cam.c2w.dim() != 2 or cam.c2w.shape[1] != 4 or cam.c2w.shape[0] < 3:
+        raise RuntimeError("c2w must be (3, 4) or (4, 4)")
+    _same_dtype(cam.c2w, dtype, "c2w")
+    return _abi.CameraSpecC(cam.c2w.data_ptr(), float(cam.fx), float(cam.fy), int(cam.width),
+                            int(cam.height))
+
+
+def _render_out_dim(spec, opt):
+    lib = _abi.load_library()
+    od = lib.svox_out_data_dim(int(opt.format), int(opt.basis_dim), spec.data_dim)
+    if od < 0:
+        raise RuntimeError("invalid data format / basis_dim for this tree")
+    return od
+
+
+def volume_render(tree, rays, opt):
+    """(B, out_dim) like rays.origins; rt_kernel.cu:1019-1036"""
+    spec = _pack_tree(tree, rays.origins.dtype if isinstance(rays.origins, torch.Tensor) else None)
+    rspec = _pack_rays(rays, tree.data.dtype)
+    od = _render_out_dim(spec, opt)
+    out = torch.empty((rspec.n_rays, od), dtype=rays.origins.dtype, device=rays.origins.device)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),
+              out.data_ptr(), _stream(tree.data.device))
+    return out
+
+
+def volume_render_image(tree, cam, opt):
+    """(H, W, out_dim) like tree.data; rt_kernel.cu:1038-1057"""
+    spec = _pack_tree(tree)
+    cspec = _pack_camera(cam, tree.data.dtype)
+    od = _render_out_dim(spec, opt)
+    out = torch.empty((cspec.height, cspec.width, od), dtype=tree.data.dtype, device=tree.data.device)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_image", ctypes.byref(spec), ctypes.byref(cspec),
+              ctypes.byref(copt), out.data_ptr(), _stream(tree.data.device))
+    return out
+
+
+def _check_grad(grad_output, shape, dtype):
+    _check_input(grad_output, "grad_output")
+    _same_dtype(grad_output, dtype, "grad_output")
+    if tuple(grad_output.shape) != tuple(shape):
+        raise RuntimeError(f"grad_output must have shape {tuple(shape)}, got {tuple(grad_output.shape)}")
+
+
+def volume_render_backward(tree, rays, opt, grad_output):
+    """zeros_like(tree.data) + scatter; rt_kernel.cu:1059-1083"""
+    spec = _pack_tree(tree)
+    rspec = _pack_rays(rays, tree.data.dtype)
+    od = _render_out_dim(spec, opt)
+    _check_grad(grad_output, (rspec.n_rays, od), tree.data.dtype)
+    grad = torch.empty_like(tree.data)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_backward", ctypes.byref(spec), ctypes.byref(rspec),
+              ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
+              _stream(tree.data.device))
+    return grad
+
+
+def volume_render_image_backward(tree, cam, opt, grad_output):
+    """zeros_like(tree.data) + scatter; rt_kernel.cu:1085-1109"""
+    spec = _pack_tree(tree)
+    cspec = _pack_camera(cam, tree.data.dtype)
+    od = _render_out_dim(spec, opt)
+    _check_grad(grad_output, (cspec.height, cspec.width, od), tree.data.dtype)
+    grad = torch.empty_like(tree.data)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_image_backward", ctypes.byref(spec), ctypes.byref(cspec),
+              ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
+              _stream(tree.data.device))
+    return grad
+
+
+def volume_render_stats(tree, rays_or_cam, opt):
+    """Visit counts of one launch (dict); `rays_or_cam` is a RaysSpec or a CameraSpec."""
+    spec = _pack_tree(tree)
+    copt = opt._pack()
+    counters = torch.zeros(8, dtype=torch.int64, device=tree.data.device)
+    with torch.cuda.device(tree.data.device):
+        if isinstance(rays_or_cam, RaysSpec):
+            rspec = _pack_rays(rays_or_cam, tree.data.dtype)
+            _call("svox_volume_render_stats", ctypes.byref(spec), ctypes.byref(rspec), None,
+                  ctypes.byref(copt), counters.data_ptr(), _stream(tree.data.device))
+        else:
+            cspec = _pack_camera(rays_or_cam, tree.data.dtype)
+            _call("svox_volume_render_stats", ctypes.byref(spec), None, ctypes.byref(cspec),
+                  ctypes.byref(copt), counters.data_ptr(), _stream(tree.data.device))
+    vals = counters.cpu().tolist()
+    names = [f[0] for f in _abi.MarchStatsC._fields_]
+    return {n: int(v) for n, v in zip(names, vals) if n != "reserved"}
+
+
+def set_debug_flags(flags):
+    """bit 0: route every call to the generic kernels"""
+    _abi.load_library().svox_set_debug_flags(int(flags))

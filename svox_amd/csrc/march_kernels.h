@@ -1,0 +1,699 @@
+// march_kernels.h -- ray marching through the leaves of the N^3 tree: forward rendering, its
+// backward pass and the visit counters (reference: svox/csrc/rt_kernel.cu:189-477, 717-844).
+//
+// Every kernel exists in two flavours that compute the same numbers:
+//   GenericPolicy<T>   any branching factor, scalar type, data format, component range, softplus,
+//                      weight accumulation; the reference's floating-point walk from the root for
+//                      every sample.
+//   OctreePolicy<FMT,D> fp32 octree with the default options (SH with D in {1,4,9,16,25}, or RGBA
+//                      with 3 colours): integer-coordinate walk restarted from the previous path
+//                      (OctreeCursor), record length and basis size known at compile time so the
+//                      basis, the colour accumulators and the dot products live in registers.
+#pragma once
+
+#include "basis.h"
+#include "tree_walk.h"
+
+namespace svox {
+
+constexpr int kMarchThreads = 256;
+constexpr int kTile = 16;  // image kernels: a block covers a 16x16 pixel tile, a wavefront 8x8
+
+// ------------------------------------------------------------------------------------------------
+// ray sources
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+struct RayBatch {
+    const T* origins;
+    const T* dirs;
+    const T* vdirs;
+    int64_t n_rays;
+};
+
+template <typename T>
+struct Camera {
+    const T* c2w;
+    float fx, fy;
+    int width, height;
+};
+
+// _dda_unit, rt_kernel.cu:203-220: the segment of the ray inside the unit cube
+template <typename T>
+__device__ __forceinline__ void dda_unit(const T* cen, const T* invdir, T* tmin, T* tmax) {
+    T lo = T(0), hi = T(1e9f);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        const T t1 = -cen[i] * invdir[i];
+        const T t2 = t1 + invdir[i];
+        lo = max_(lo, min_(t1, t2));
+        hi = min_(hi, max_(t1, t2));
+    }
+    *tmin = lo;
+    *tmax = hi;
+}
+
+// cam2world_ray, rt_kernel.cu:758-772: pixel corner (no half-pixel offset), camera looking down
+// -z with +y up.  x and y are formed in double and rounded; the radicand is widened for `+ 1.0`.
+template <typename T>
+__device__ __forceinline__ void cam2world_ray(int ix, int iy, const Camera<T>& cam, T* dir, T* origin) {
+    T x = (T)(((double)ix - 0.5 * (double)cam.width) / (double)cam.fx);
+    T y = (T)(-((double)iy - 0.5 * (double)cam.height) / (double)cam.fy);
+    T z = (T)__builtin_sqrtf((float)((double)fma_(x, x, y * y) + 1.0));
+    x /= z;
+    y /= z;
+    z = (T)(-1.0f / z);
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        const T* row = cam.c2w + r * 4;
+        dir[r] = fma_(row[2], z, fma_(row[0], x, row[1] * y));
+        origin[r] = row[3];
+    }
+}
+
+// maybe_world2ndc, rt_kernel.cu:775-796 with near = 1
+template <typename T>
+__device__ __forceinline__ void maybe_world2ndc(const SvoxRenderOptions& opt, T* dir, T* cen) {
+    if (opt.ndc_width < 0) return;
+    const T near = T(1);
+    const T t = -(near + cen[2]) / dir[2];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) cen[i] = fma_(t, dir[i], cen[i]);
+    const float two_f = 2 * opt.ndc_focal;
+    const T kx = (T)(two_f / (float)opt.ndc_width);
+    const T ky = (T)(two_f / (float)opt.ndc_height);
+    dir[0] = -kx * (dir[0] / dir[2] - cen[0] / cen[2]);
+    dir[1] = -ky * (dir[1] / dir[2] - cen[1] / cen[2]);
+    dir[2] = T(-2) * near / cen[2];
+    cen[0] = -kx * (cen[0] / cen[2]);
+    cen[1] = -ky * (cen[1] / cen[2]);
+    cen[2] = T(1) + T(2) * near / cen[2];
+    const T n = norm3(dir);
+    dir[0] /= n;
+    dir[1] /= n;
+    dir[2] /= n;
+}
+
+// Which ray a thread traces.  Batch: thread i takes ray i.  Image: blocks are 16x16 pixel tiles
+// and each wavefront an 8x8 sub-tile, so the 64 rays of a wavefront stay close in the tree; tiles
+// are dealt to blocks so that the blocks one XCD receives (block ids congruent mod 8) form one
+// contiguous band of the image and share that XCD's L2.
+template <typename T>
+struct BatchSource {
+    RayBatch<T> rays;
+    __device__ __forceinline__ int64_t count() const { return rays.n_rays; }
+    // returns the output slot (ray index) or -1
+    __device__ __forceinline__ int64_t fetch(const TreeDev<T>&, const SvoxRenderOptions&, const T* offset,
+                                             const T* scaling, T* origin, T* dir, T* vdir) const {
+        const int64_t r = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
+        if (r >= rays.n_rays) return -1;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            origin[i] = rays.origins[r * 3 + i];
+            dir[i] = rays.dirs[r * 3 + i];
+            vdir[i] = rays.vdirs[r * 3 + i];
+        }
+        transform_coord(origin, offset, scaling);
+        return r;
+    }
+};
+
+__host__ __device__ inline int tiles_of(int extent) { return (extent + kTile - 1) / kTile; }
+
+template <typename T>
+struct ImageSource {
+    Camera<T> cam;
+    int chunk;  // tiles per XCD band = ceil(n_tiles / 8)
+    __device__ __forceinline__ int64_t count() const { return (int64_t)cam.width * cam.height; }
+    __device__ __forceinline__ int64_t fetch(const TreeDev<T>&, const SvoxRenderOptions& opt, const T* offset,
+                                             const T* scaling, T* origin, T* dir, T* vdir) const {
+        const int ntx = tiles_of(cam.width), nty = tiles_of(cam.height);
+        const int tile = (int)(blockIdx.x & 7u) * chunk + (int)(blockIdx.x >> 3);
+        if (tile >= ntx * nty) return -1;
+        const int ty = tile / ntx, tx = tile - ty * ntx;
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        const int ix = tx * kTile + (wave & 1) * 8 + (lane & 7);
+        const int iy = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
+        if (ix >= cam.width || iy >= cam.height) return -1;
+        cam2world_ray(ix, iy, cam, dir, origin);
+#pragma unroll
+        for (int i = 0; i < 3; ++i) vdir[i] = dir[i];
+        maybe_world2ndc(opt, dir, origin);
+        transform_coord(origin, offset, scaling);
+        return (int64_t)iy * cam.width + ix;
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+// per-ray march state
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+struct RayState {
+    T o[3], d[3], inv[3];
+    T t, tmax, dscale;
+};
+
+// rt_kernel.cu:228-247: scale and normalise the direction, reciprocal in double, clip to the cube
+template <typename T>
+__device__ __forceinline__ bool setup_ray(RayState<T>& r, const T* origin, const T* dir, const T* scaling) {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        r.o[i] = origin[i];
+        r.d[i] = dir[i] * scaling[i];
+    }
+    const T s = T(1) / norm3(r.d);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        r.d[i] *= s;
+        r.inv[i] = (T)(1.0 / ((double)r.d[i] + 1e-9));
+    }
+    r.dscale = s;
+    T tmin, tmax;
+    dda_unit(r.o, r.inv, &tmin, &tmax);
+    r.t = tmin;
+    r.tmax = tmax;
+    return !(tmax < T(0) || tmin > tmax);
+}
+
+struct Visit {
+    int64_t leaf;  // cell index node*N^3 + cell, -1 ends the ray (malformed tree)
+    int levels;
+};
+
+// One sample with the reference's walk: position, leaf, step length.  rt_kernel.cu:262-275.
+template <typename T>
+__device__ __forceinline__ Visit step_generic(const TreeDev<T>& tr, const RayState<T>& r, T step_size,
+                                              T* delta_t) {
+    T pos[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) pos[j] = fma_(r.t, r.d[j], r.o[j]);
+    T cube;
+    Visit v;
+    v.leaf = descend_generic<T>(tr.child, tr.capacity, tr.N, pos, &cube, &v.levels);
+    T s0, s1;
+    dda_unit(pos, r.inv, &s0, &s1);
+    *delta_t = (s1 - s0) / cube + step_size;
+    return v;
+}
+
+// The same sample for an fp32 octree: integer walk resumed from the previous path.
+__device__ __forceinline__ Visit step_octree(const TreeDev<float>& tr, const RayState<float>& r,
+                                             OctreeCursor& cur, float step_size, float* delta_t,
+                                             int* reads) {
+    float pc[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) pc[j] = clamp01(fma_(r.t, r.d[j], r.o[j]));
+    Visit v;
+    const int32_t leaf = cur.seek(tr.child, tr.capacity, cell_coord(pc[0]), cell_coord(pc[1]),
+                                  cell_coord(pc[2]), reads);
+    float inv_cube;  // 2^-levels: dividing by the power of two 2^levels is this multiplication
+    float local[3];
+    if (leaf >= 0) {
+        v.leaf = leaf;
+        v.levels = cur.levels;
+        const float cube = __uint_as_float((uint32_t)(127 + cur.levels) << 23);
+        inv_cube = __uint_as_float((uint32_t)(127 - cur.levels) << 23);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) local[j] = leaf_local(pc[j], cube);
+    } else {
+        // more levels than the integer coordinates hold (or a broken tree): floating-point walk
+        float cube;
+#pragma unroll
+        for (int j = 0; j < 3; ++j) local[j] = pc[j];
+        v.leaf = descend_generic<float>(tr.child, tr.capacity, 2, local, &cube, &v.levels);
+        *reads += v.levels;
+        inv_cube = 1.0f / cube;
+    }
+    float s0, s1;
+    dda_unit(local, r.inv, &s0, &s1);
+    *delta_t = (s1 - s0) * inv_cube + step_size;
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------------
+// policies
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+struct GenericPolicy {
+    using scalar = T;
+    static constexpr bool kOctree = false;
+};
+
+template <int FMT, int D>
+struct OctreePolicy {
+    using scalar = float;
+    static constexpr bool kOctree = true;
+    static constexpr int kFormat = FMT;
+    static constexpr int kBasis = D;                                   // 0 for RGBA
+    static constexpr int kRecord = (FMT == SVOX_FORMAT_RGBA) ? 4 : 3 * D + 1;
+};
+
+// atomicMax of the reference (common.cuh:152-172): compare-and-swap loop around fmaxf
+__device__ __forceinline__ void atomic_max_float(float* addr, float value) {
+    unsigned* a = (unsigned*)addr;
+    unsigned old = *a, assumed;
+    do {
+        assumed = old;
+        old = atomicCAS(a, assumed, __float_as_uint(max_(value, __uint_as_float(assumed))));
+    } while (old != assumed);
+}
+__device__ __forceinline__ void atomic_max_float(double* addr, double value) {
+    unsigned long long* a = (unsigned long long*)addr;
+    unsigned long long old = *a, assumed;
+    do {
+        assumed = old;
+        const double m = (double)max_((float)value, (float)__longlong_as_double((long long)assumed));
+        old = atomicCAS(a, assumed, (unsigned long long)__double_as_longlong(m));
+    } while (old != assumed);
+}
+
+// ------------------------------------------------------------------------------------------------
+// forward
+// ------------------------------------------------------------------------------------------------
+// trace_ray, rt_kernel.cu:222-321, generic flavour
+template <typename T>
+__device__ void trace_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt, const T* origin,
+                              const T* dir, const T* vdir, const T* scaling, int out_dim, T* out) {
+    RayState<T> r;
+    T acc[SVOX_MAX_OUT_DIM];
+    if (!setup_ray(r, origin, dir, scaling)) {
+        for (int j = 0; j < out_dim; ++j) out[j] = (T)opt.background_brightness;
+        return;
+    }
+    for (int j = 0; j < out_dim; ++j) acc[j] = T(0);
+    T basis[SVOX_MAX_BASIS_DIM];
+    precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
+    T light = T(1);
+    const T pad = (T)opt.rgb_padding;
+    const T d_rgb_pad = (T)(1 + 2 * opt.rgb_padding);
+    bool stopped = false;
+    while (r.t < r.tmax) {
+        T delta_t;
+        const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+        if (v.leaf < 0) break;
+        const T* val = tr.data + v.leaf * tr.K;
+        T sigma = val[tr.K - 1];
+        if (opt.density_softplus) sigma = softplus_m1(sigma);
+        if (sigma > (T)opt.sigma_thresh) {
+            const T att = exp_sp<T>(-delta_t * r.dscale * sigma);
+            const T weight = light * (T(1) - att);
+            if (opt.format != SVOX_FORMAT_RGBA) {
+                for (int c = 0; c < out_dim; ++c) {
+                    const int off = c * opt.basis_dim;
+                    T tmp = T(0);
+                    for (int i = opt.min_comp; i <= opt.max_comp; ++i) tmp = fma_(basis[i], val[off + i], tmp);
+                    acc[c] = fma_(weight, fma_(sigmoid_(tmp), d_rgb_pad, -pad), acc[c]);
+                }
+            } else {
+                for (int c = 0; c < out_dim; ++c)
+                    acc[c] = fma_(weight, fma_(sigmoid_(val[c]), d_rgb_pad, -pad), acc[c]);
+            }
+            light *= att;
+            if (tr.weight_accum) {
+                if (tr.weight_accum_max)
+                    atomic_max_float(tr.weight_accum + v.leaf, weight);
+                else
+                    atomicAdd(tr.weight_accum + v.leaf, weight);
+            }
+            if (light <= (T)opt.stop_thresh) {
+                const T scale = (T)(1.0 / (1.0 - (double)light));
+                for (int j = 0; j < out_dim; ++j) acc[j] *= scale;
+                stopped = true;
+                break;
+            }
+        }
+        r.t += delta_t;
+    }
+    if (!stopped)
+        for (int j = 0; j < out_dim; ++j) acc[j] = fma_(light, (T)opt.background_brightness, acc[j]);
+    for (int j = 0; j < out_dim; ++j) out[j] = acc[j];
+}
+
+// colour of one leaf record for the octree flavour: 3 sigmoids of basis . coefficients
+template <class P>
+__device__ __forceinline__ void leaf_colour(const float* __restrict__ rec, const float* basis, float* s) {
+    if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+#pragma unroll
+        for (int c = 0; c < 3; ++c) s[c] = sigmoid_(rec[c]);
+    } else {
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            float tmp = 0.0f;
+#pragma unroll
+            for (int i = 0; i < P::kBasis; ++i) tmp = fma_(basis[i], rec[c * P::kBasis + i], tmp);
+            s[c] = sigmoid_(tmp);
+        }
+    }
+}
+
+// trace_ray, octree flavour
+template <class P>
+__device__ __forceinline__ void trace_octree(const TreeDev<float>& tr, const SvoxRenderOptions& opt,
+                                             const float* origin, const float* dir, const float* vdir,
+                                             const float* scaling, OctreeCursor& cur, float* out) {
+    RayState<float> r;
+    const float bg = opt.background_brightness;
+    if (!setup_ray(r, origin, dir, scaling)) {
+        out[0] = bg;
+        out[1] = bg;
+        out[2] = bg;
+        return;
+    }
+    float basis[P::kBasis > 0 ? P::kBasis : 1];
+    if constexpr (P::kFormat == SVOX_FORMAT_SH) sh_basis<float>(P::kBasis, vdir, basis);
+    float acc[3] = {0.f, 0.f, 0.f};
+    float light = 1.0f;
+    const float pad = opt.rgb_padding;
+    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
+    const float step = opt.step_size, sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
+    bool stopped = false;
+    int reads = 0;
+    while (r.t < r.tmax) {
+        float delta_t;
+        const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
+        if (v.leaf < 0) break;
+        const float* rec = tr.data + v.leaf * P::kRecord;
+        const float sigma = rec[P::kRecord - 1];
+        if (sigma > sigma_thresh) {
+            const float att = expf_fixed(-delta_t * r.dscale * sigma);
+            const float weight = light * (1.0f - att);
+            float s[3];
+            leaf_colour<P>(rec, basis, s);
+#pragma unroll
+            for (int c = 0; c < 3; ++c) acc[c] = fma_(weight, fma_(s[c], d_rgb_pad, -pad), acc[c]);
+            light *= att;
+            if (light <= stop_thresh) {
+                const float scale = (float)(1.0 / (1.0 - (double)light));
+#pragma unroll
+                for (int c = 0; c < 3; ++c) acc[c] *= scale;
+                stopped = true;
+                break;
+            }
+        }
+        r.t += delta_t;
+    }
+    if (!stopped) {
+#pragma unroll
+        for (int c = 0; c < 3; ++c) acc[c] = fma_(light, bg, acc[c]);
+    }
+    out[0] = acc[0];
+    out[1] = acc[1];
+    out[2] = acc[2];
+}
+
+template <class P, class Source>
+__global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<typename P::scalar> tr,
+                                                                       Source src, SvoxRenderOptions opt,
+                                                                       int out_dim,
+                                                                       typename P::scalar* __restrict__ out) {
+    using T = typename P::scalar;
+    __shared__ int32_t path[P::kOctree ? kPathLevels * kMarchThreads : 1];
+    T offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    T origin[3], dir[3], vdir[3];
+    const int64_t slot = src.fetch(tr, opt, offset, scaling, origin, dir, vdir);
+    if (slot < 0) return;
+    if constexpr (P::kOctree) {
+        OctreeCursor cur;
+        cur.reset(path + threadIdx.x, kMarchThreads);
+        trace_octree<P>(tr, opt, origin, dir, vdir, scaling, cur, out + slot * 3);
+    } else {
+        trace_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, out + slot * out_dim);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// backward
+// ------------------------------------------------------------------------------------------------
+// trace_ray_backward, rt_kernel.cu:323-477, generic flavour: two marches, the colour gradients in
+// the first, the density gradient in the second; both test sigma > 0 and never stop early.
+template <typename T>
+__device__ void trace_backward_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt, const T* origin,
+                                       const T* dir, const T* vdir, const T* scaling, int out_dim,
+                                       const T* grad_out, T* grad_data) {
+    RayState<T> r;
+    if (!setup_ray(r, origin, dir, scaling)) return;
+    T basis[SVOX_MAX_BASIS_DIM];
+    precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
+    T go[SVOX_MAX_OUT_DIM];
+    for (int j = 0; j < out_dim; ++j) go[j] = grad_out[j];
+    const T pad = (T)opt.rgb_padding;
+    const T d_rgb_pad = (T)(1 + 2 * opt.rgb_padding);
+    const T tmin = r.t;
+    T accum = T(0);
+    {
+        T light = T(1);
+        while (r.t < r.tmax) {
+            T delta_t;
+            const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+            if (v.leaf < 0) return;
+            const int64_t base = v.leaf * tr.K;
+            const T* val = tr.data + base;
+            T sigma = val[tr.K - 1];
+            if (opt.density_softplus) sigma = softplus_m1(sigma);
+            if (sigma > T(0)) {
+                const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
+                const T weight = light * (T(1) - att);
+                T total_color = T(0);
+                if (opt.format != SVOX_FORMAT_RGBA) {
+                    for (int c = 0; c < out_dim; ++c) {
+                        const int off = c * opt.basis_dim;
+                        T tmp = T(0);
+                        for (int i = opt.min_comp; i <= opt.max_comp; ++i)
+                            tmp = fma_(basis[i], val[off + i], tmp);
+                        const T sg = sigmoid_(tmp);
+                        const T tmp2 = (T)((double)(weight * sg) * (1.0 - (double)sg) * (double)go[c] *
+                                           (double)d_rgb_pad);
+                        for (int i = opt.min_comp; i <= opt.max_comp; ++i)
+                            atomicAdd(grad_data + base + off + i, basis[i] * tmp2);
+                        total_color = fma_(fma_(sg, d_rgb_pad, -pad), go[c], total_color);
+                    }
+                } else {
+                    for (int c = 0; c < out_dim; ++c) {
+                        const T sg = sigmoid_(val[c]);
+                        atomicAdd(grad_data + base + c, weight * sg * (T(1) - sg) * go[c] * d_rgb_pad);
+                        total_color = fma_(fma_(sg, d_rgb_pad, -pad), go[c], total_color);
+                    }
+                }
+                light *= att;
+                accum = fma_(weight, total_color, accum);
+            }
+            r.t += delta_t;
+        }
+        T total_grad = T(0);
+        for (int j = 0; j < out_dim; ++j) total_grad += go[j];
+        accum = fma_(light * (T)opt.background_brightness, total_grad, accum);
+    }
+    {
+        T light = T(1);
+        r.t = tmin;
+        while (r.t < r.tmax) {
+            T delta_t;
+            const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+            if (v.leaf < 0) return;
+            const int64_t base = v.leaf * tr.K;
+            const T* val = tr.data + base;
+            T sigma = val[tr.K - 1];
+            const T raw_sigma = sigma;
+            if (opt.density_softplus) sigma = softplus_m1(sigma);
+            if (sigma > T(0)) {
+                const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
+                const T weight = light * (T(1) - att);
+                T total_color = T(0);
+                if (opt.format != SVOX_FORMAT_RGBA) {
+                    for (int c = 0; c < out_dim; ++c) {
+                        const int off = c * opt.basis_dim;
+                        T tmp = T(0);
+                        for (int i = opt.min_comp; i <= opt.max_comp; ++i)
+                            tmp = fma_(basis[i], val[off + i], tmp);
+                        total_color = fma_(fma_(sigmoid_(tmp), d_rgb_pad, -pad), go[c], total_color);
+                    }
+                } else {
+                    for (int c = 0; c < out_dim; ++c)
+                        total_color = fma_(fma_(sigmoid_(val[c]), d_rgb_pad, -pad), go[c], total_color);
+                }
+                light *= att;
+                accum = fma_(-weight, total_color, accum);
+                const T chain = opt.density_softplus ? sigmoid_(raw_sigma - T(1)) : T(1);
+                atomicAdd(grad_data + base + tr.K - 1,
+                          delta_t * r.dscale * fma_(total_color, light, -accum) * chain);
+            }
+            r.t += delta_t;
+        }
+    }
+}
+
+// trace_ray_backward, octree flavour.  The first march only accumulates <render, grad_out>
+// (no memory writes); the second replays it and issues every atomic add: colour gradients with the
+// reference's per-sample values, then the density gradient.
+template <class P>
+__device__ __forceinline__ void trace_backward_octree(const TreeDev<float>& tr, const SvoxRenderOptions& opt,
+                                                      const float* origin, const float* dir,
+                                                      const float* vdir, const float* scaling,
+                                                      OctreeCursor& cur, const float* grad_out,
+                                                      float* __restrict__ grad_data) {
+    RayState<float> r;
+    if (!setup_ray(r, origin, dir, scaling)) return;
+    float basis[P::kBasis > 0 ? P::kBasis : 1];
+    if constexpr (P::kFormat == SVOX_FORMAT_SH) sh_basis<float>(P::kBasis, vdir, basis);
+    const float go[3] = {grad_out[0], grad_out[1], grad_out[2]};
+    const float pad = opt.rgb_padding;
+    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
+    const float step = opt.step_size;
+    const float tmin = r.t;
+    float accum = 0.0f;
+    int reads = 0;
+    {
+        float light = 1.0f;
+        while (r.t < r.tmax) {
+            float delta_t;
+            const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
+            if (v.leaf < 0) return;
+            const float* rec = tr.data + v.leaf * P::kRecord;
+            const float sigma = rec[P::kRecord - 1];
+            if (sigma > 0.0f) {
+                const float att = expf_fixed(-delta_t * sigma * r.dscale);
+                const float weight = light * (1.0f - att);
+                float s[3];
+                leaf_colour<P>(rec, basis, s);
+                float total_color = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 3; ++c) total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+                light *= att;
+                accum = fma_(weight, total_color, accum);
+            }
+            r.t += delta_t;
+        }
+        const float total_grad = (go[0] + go[1]) + go[2];
+        accum = fma_(light * opt.background_brightness, total_grad, accum);
+    }
+    {
+        float light = 1.0f;
+        r.t = tmin;
+        while (r.t < r.tmax) {
+            float delta_t;
+            const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
+            if (v.leaf < 0) return;
+            const int64_t base = v.leaf * P::kRecord;
+            const float* rec = tr.data + base;
+            const float sigma = rec[P::kRecord - 1];
+            if (sigma > 0.0f) {
+                const float att = expf_fixed(-delta_t * sigma * r.dscale);
+                const float weight = light * (1.0f - att);
+                float s[3];
+                leaf_colour<P>(rec, basis, s);
+                float total_color = 0.0f;
+                float* g = grad_data + base;
+#pragma unroll
+                for (int c = 0; c < 3; ++c) {
+                    if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                        atomicAdd(g + c, weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad);
+                    } else {
+                        const float tmp2 = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) *
+                                                   (double)go[c] * (double)d_rgb_pad);
+#pragma unroll
+                        for (int i = 0; i < P::kBasis; ++i) atomicAdd(g + c * P::kBasis + i, basis[i] * tmp2);
+                    }
+                    total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+                }
+                light *= att;
+                accum = fma_(-weight, total_color, accum);
+                atomicAdd(g + P::kRecord - 1, delta_t * r.dscale * fma_(total_color, light, -accum));
+            }
+            r.t += delta_t;
+        }
+    }
+}
+
+template <class P, class Source>
+__global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(
+    TreeDev<typename P::scalar> tr, Source src, SvoxRenderOptions opt, int out_dim,
+    const typename P::scalar* __restrict__ grad_out, typename P::scalar* __restrict__ grad_data) {
+    using T = typename P::scalar;
+    __shared__ int32_t path[P::kOctree ? kPathLevels * kMarchThreads : 1];
+    T offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    T origin[3], dir[3], vdir[3];
+    const int64_t slot = src.fetch(tr, opt, offset, scaling, origin, dir, vdir);
+    if (slot < 0) return;
+    if constexpr (P::kOctree) {
+        OctreeCursor cur;
+        cur.reset(path + threadIdx.x, kMarchThreads);
+        trace_backward_octree<P>(tr, opt, origin, dir, vdir, scaling, cur, grad_out + slot * 3, grad_data);
+    } else {
+        trace_backward_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, grad_out + slot * out_dim,
+                                  grad_data);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// visit counters
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ unsigned long long wave_sum(unsigned long long v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const unsigned lo = __shfl_down((unsigned)(v & 0xffffffffull), off);
+        const unsigned hi = __shfl_down((unsigned)(v >> 32), off);
+        v += ((unsigned long long)hi << 32) | lo;
+    }
+    return v;
+}
+
+// Counts, with the reference's walk, what the forward march (thresholds, early stop) and one
+// backward march (sigma > 0, no stop) of every ray visit.
+template <typename T, class Source>
+__global__ __launch_bounds__(kMarchThreads) void render_stats_kernel(TreeDev<T> tr, Source src,
+                                                                     SvoxRenderOptions opt,
+                                                                     unsigned long long* __restrict__ stats) {
+    T offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    T origin[3], dir[3], vdir[3];
+    const int64_t slot = src.fetch(tr, opt, offset, scaling, origin, dir, vdir);
+    unsigned long long c_rays = 0, c_hit = 0, c_samples = 0, c_shaded = 0, c_bwd = 0, c_bwd_pos = 0, c_levels = 0;
+    if (slot >= 0) {
+        c_rays = 1;
+        RayState<T> r;
+        if (setup_ray(r, origin, dir, scaling)) {
+            c_hit = 1;
+            T light = T(1);
+            bool fwd_live = true;
+            while (r.t < r.tmax) {
+                T delta_t;
+                const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+                if (v.leaf < 0) break;
+                T sigma = tr.data[v.leaf * tr.K + tr.K - 1];
+                if (opt.density_softplus) sigma = softplus_m1(sigma);
+                c_bwd += 1;
+                if (sigma > T(0)) c_bwd_pos += 1;
+                if (fwd_live) {
+                    c_samples += 1;
+                    c_levels += (unsigned)v.levels;
+                    if (sigma > (T)opt.sigma_thresh) {
+                        c_shaded += 1;
+                        light *= exp_sp<T>(-delta_t * r.dscale * sigma);
+                        if (light <= (T)opt.stop_thresh) fwd_live = false;
+                    }
+                }
+                r.t += delta_t;
+            }
+        }
+    }
+    // every lane reaches the reductions
+    c_rays = wave_sum(c_rays);
+    c_hit = wave_sum(c_hit);
+    c_samples = wave_sum(c_samples);
+    c_shaded = wave_sum(c_shaded);
+    c_bwd = wave_sum(c_bwd);
+    c_bwd_pos = wave_sum(c_bwd_pos);
+    c_levels = wave_sum(c_levels);
+    if ((threadIdx.x & 63) == 0) {
+        atomicAdd(stats + 0, c_rays);
+        atomicAdd(stats + 1, c_hit);
+        atomicAdd(stats + 2, c_samples);
+        atomicAdd(stats + 3, c_shaded);
+        atomicAdd(stats + 4, c_bwd);
+        atomicAdd(stats + 5, c_bwd_pos);
+        atomicAdd(stats + 6, c_levels);
+    }
+}
+
+}  // namespace svox

@@ -1,0 +1,482 @@
+// svox_hip.hip -- the extern "C" entry points of libsvox_hip.so (declared in include/svox_hip.h):
+// argument validation, kernel selection and launches.  Each entry point stands where one function
+// of the reference's extension module stood (svox/csrc/svox.cpp:106-121; host launchers
+// svox/csrc/svox_kernel.cu:120-203 and svox/csrc/rt_kernel.cu:1009-1109).
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/svox_hip.h"
+#include "march_kernels.h"
+#include "query_kernels.h"
+
+namespace {
+
+using namespace svox;
+
+thread_local char g_error[512] = "";
+int g_debug_flags = 0;  // bit 0: always take the generic kernels
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char* what) {
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return fail(SVOX_ERR_LAUNCH, "svox.%s: %s", what, hipGetErrorString(err));
+    return SVOX_OK;
+}
+
+int check_tree(const SvoxTreeSpec* t, bool need_data) {
+    if (!t) return fail(SVOX_ERR_NULL_POINTER, "tree spec is NULL");
+    if (need_data && !t->data) return fail(SVOX_ERR_NULL_POINTER, "tree.data is NULL");
+    if (!t->child) return fail(SVOX_ERR_NULL_POINTER, "tree.child is NULL");
+    if (!t->parent_depth) return fail(SVOX_ERR_NULL_POINTER, "tree.parent_depth is NULL");
+    if (t->dtype != SVOX_F32 && t->dtype != SVOX_F64)
+        return fail(SVOX_ERR_BAD_DTYPE, "tree.dtype must be SVOX_F32 or SVOX_F64, got %d", t->dtype);
+    if (t->capacity < 1) return fail(SVOX_ERR_BAD_SHAPE, "tree.capacity must be >= 1, got %lld", (long long)t->capacity);
+    if (t->N < 2) return fail(SVOX_ERR_BAD_SHAPE, "tree.N must be >= 2, got %d", t->N);
+    if (t->data_dim < 1) return fail(SVOX_ERR_BAD_SHAPE, "tree.data_dim must be >= 1, got %d", t->data_dim);
+    const double cells = (double)t->capacity * t->N * t->N * t->N;
+    if (cells >= 9.0e18 / (double)(t->data_dim > 0 ? t->data_dim : 1))
+        return fail(SVOX_ERR_BAD_SHAPE, "tree is too large to index");
+    if (t->capacity > 0x7fffffffll)
+        return fail(SVOX_ERR_BAD_SHAPE, "tree.capacity exceeds the int32 node ids of the child table");
+    return SVOX_OK;
+}
+
+template <typename T>
+TreeDev<T> make_tree(const SvoxTreeSpec* t) {
+    TreeDev<T> d;
+    d.data = (T*)t->data;
+    d.child = t->child;
+    d.parent_depth = t->parent_depth;
+    d.extra = (const T*)t->extra_data;
+    d.offset = (const T*)t->offset;
+    d.scaling = (const T*)t->scaling;
+    d.weight_accum = (T*)t->weight_accum;
+    d.capacity = t->capacity;
+    d.N = t->N;
+    d.K = t->data_dim;
+    d.extra_cols = t->extra_cols;
+    d.weight_accum_max = t->weight_accum_max;
+    return d;
+}
+
+// cell indices fit int32 and the tree is an fp32 octree
+bool octree_fast_ok(const SvoxTreeSpec* t) {
+    return !(g_debug_flags & 1) && t->dtype == SVOX_F32 && t->N == 2 && t->capacity < (1ll << 28);
+}
+
+int zero_fill(void* ptr, int64_t bytes, hipStream_t stream) {
+    if (bytes <= 0) return SVOX_OK;
+    if (((uintptr_t)ptr & 15u) != 0 || (bytes & 3) != 0)
+        return fail(SVOX_ERR_BAD_SHAPE, "gradient buffer must be 16-byte aligned and a multiple of 4 bytes");
+    const int64_t n16 = bytes / 16;
+    const int n_tail = (int)((bytes - n16 * 16) / 4);
+    int64_t blocks = (n16 + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint4*)ptr, n16,
+                       (uint32_t*)((char*)ptr + n16 * 16), n_tail);
+    return check_launch("zero_fill");
+}
+
+// ---------------------------------------------------------------------------------------------
+// queries
+// ---------------------------------------------------------------------------------------------
+constexpr int kLdsNodesMax = 584;  // child rows kept in LDS per block: 584 * 32 B = 18.25 KiB
+
+template <typename T, int MODE>
+int launch_query(const SvoxTreeSpec* tree, const void* points, int64_t n, void* values, void* target,
+                 int64_t* ids, int32_t Kx, hipStream_t stream, const char* what) {
+    if (n == 0) return SVOX_OK;
+    const TreeDev<T> tr = make_tree<T>(tree);
+    const int64_t tiles = (n + kQueryThreads - 1) / kQueryThreads;
+    const int64_t blocks = tiles < 256 * 8 ? tiles : 256 * 8;
+    if constexpr (sizeof(T) == 4) {
+        if (octree_fast_ok(tree)) {
+            const int32_t lds_nodes = tree->capacity < kLdsNodesMax ? (int32_t)tree->capacity : kLdsNodesMax;
+            hipLaunchKernelGGL((query_kernel<T, MODE, true>), dim3((unsigned)blocks), dim3(kQueryThreads),
+                               (size_t)lds_nodes * 32, stream, tr, (const T*)points, n, (T*)values,
+                               (T*)target, ids, Kx, lds_nodes);
+            return check_launch(what);
+        }
+    }
+    hipLaunchKernelGGL((query_kernel<T, MODE, false>), dim3((unsigned)blocks), dim3(kQueryThreads), 0, stream,
+                       tr, (const T*)points, n, (T*)values, (T*)target, ids, Kx, 0);
+    return check_launch(what);
+}
+
+// ---------------------------------------------------------------------------------------------
+// rendering
+// ---------------------------------------------------------------------------------------------
+int check_render(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, int* out_dim) {
+    int rc = check_tree(tree, true);
+    if (rc) return rc;
+    if (!opt) return fail(SVOX_ERR_NULL_POINTER, "render options are NULL");
+    if (opt->format < SVOX_FORMAT_RGBA || opt->format > SVOX_FORMAT_ASG)
+        return fail(SVOX_ERR_BAD_SHAPE, "unknown data format %d", opt->format);
+    const int od = svox_out_data_dim(opt->format, opt->basis_dim, tree->data_dim);
+    if (od < 0)
+        return fail(SVOX_ERR_BAD_SHAPE, "basis_dim %d is invalid for format %d", opt->basis_dim, opt->format);
+    if (od > SVOX_MAX_OUT_DIM)
+        return fail(SVOX_ERR_UNSUPPORTED, "rendered colour dimension %d exceeds %d", od, SVOX_MAX_OUT_DIM);
+    if (opt->format != SVOX_FORMAT_RGBA) {
+        if (opt->basis_dim > SVOX_MAX_BASIS_DIM)
+            return fail(SVOX_ERR_UNSUPPORTED, "basis_dim %d exceeds %d", opt->basis_dim, SVOX_MAX_BASIS_DIM);
+        if (opt->min_comp < 0 || opt->max_comp >= opt->basis_dim)
+            return fail(SVOX_ERR_BAD_SHAPE, "component range [%d, %d] outside [0, %d)", opt->min_comp,
+                        opt->max_comp, opt->basis_dim);
+        if (opt->format == SVOX_FORMAT_SG || opt->format == SVOX_FORMAT_ASG) {
+            const int need = opt->format == SVOX_FORMAT_SG ? 4 : 11;
+            if (!tree->extra_data || tree->extra_rows < opt->basis_dim || tree->extra_cols < need)
+                return fail(SVOX_ERR_BAD_SHAPE, "extra_data must be (%d, >=%d) for this format", opt->basis_dim, need);
+        }
+    }
+    *out_dim = od;
+    return SVOX_OK;
+}
+
+int check_camera(const SvoxCameraSpec* cam) {
+    if (!cam) return fail(SVOX_ERR_NULL_POINTER, "camera spec is NULL");
+    if (!cam->c2w) return fail(SVOX_ERR_NULL_POINTER, "cam.c2w is NULL");
+    if (cam->width < 0 || cam->height < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative image size");
+    return SVOX_OK;
+}
+
+int check_rays(const SvoxRaysSpec* rays) {
+    if (!rays) return fail(SVOX_ERR_NULL_POINTER, "rays spec is NULL");
+    if (rays->n_rays < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative ray count");
+    if (rays->n_rays > 0 && (!rays->origins || !rays->dirs || !rays->vdirs))
+        return fail(SVOX_ERR_NULL_POINTER, "rays.origins / dirs / vdirs is NULL");
+    return SVOX_OK;
+}
+
+// default options on an fp32 octree whose record matches the format: the specialised kernels
+int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
+    if (!octree_fast_ok(tree) || tree->weight_accum || opt->density_softplus) return -1;
+    if (opt->format == SVOX_FORMAT_RGBA) return tree->data_dim == 4 ? 0 : -1;
+    if (opt->format != SVOX_FORMAT_SH) return -1;
+    const int D = opt->basis_dim;
+    if (D != 1 && D != 4 && D != 9 && D != 16 && D != 25) return -1;
+    if (tree->data_dim != 3 * D + 1 || opt->min_comp != 0 || opt->max_comp != D - 1) return -1;
+    return D;
+}
+
+template <typename T>
+BatchSource<T> batch_source(const SvoxRaysSpec* rays) {
+    BatchSource<T> s;
+    s.rays.origins = (const T*)rays->origins;
+    s.rays.dirs = (const T*)rays->dirs;
+    s.rays.vdirs = (const T*)rays->vdirs;
+    s.rays.n_rays = rays->n_rays;
+    return s;
+}
+
+template <typename T>
+ImageSource<T> image_source(const SvoxCameraSpec* cam, unsigned* blocks) {
+    ImageSource<T> s;
+    s.cam.c2w = (const T*)cam->c2w;
+    s.cam.fx = cam->fx;
+    s.cam.fy = cam->fy;
+    s.cam.width = cam->width;
+    s.cam.height = cam->height;
+    const int n_tiles = tiles_of(cam->width) * tiles_of(cam->height);
+    s.chunk = (n_tiles + 7) / 8;
+    *blocks = (unsigned)s.chunk * 8u;
+    return s;
+}
+
+#define SVOX_DISPATCH_OCTREE(D, ...)                                         \
+    switch (D) {                                                             \
+        case 0: { using P = OctreePolicy<SVOX_FORMAT_RGBA, 0>; __VA_ARGS__; } break; \
+        case 1: { using P = OctreePolicy<SVOX_FORMAT_SH, 1>; __VA_ARGS__; } break;   \
+        case 4: { using P = OctreePolicy<SVOX_FORMAT_SH, 4>; __VA_ARGS__; } break;   \
+        case 9: { using P = OctreePolicy<SVOX_FORMAT_SH, 9>; __VA_ARGS__; } break;   \
+        case 16: { using P = OctreePolicy<SVOX_FORMAT_SH, 16>; __VA_ARGS__; } break; \
+        default: { using P = OctreePolicy<SVOX_FORMAT_SH, 25>; __VA_ARGS__; } break; \
+    }
+
+template <class Source, typename T>
+void launch_forward(const SvoxTreeSpec* tree, const Source& src, unsigned blocks, const SvoxRenderOptions* opt,
+                    int out_dim, void* out, hipStream_t stream) {
+    if constexpr (sizeof(T) == 4) {
+        const int D = fast_basis(tree, opt);
+        if (D >= 0) {
+            SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source>), dim3(blocks),
+                                                       dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                       src, *opt, out_dim, (float*)out));
+            return;
+        }
+    }
+    hipLaunchKernelGGL((render_forward_kernel<GenericPolicy<T>, Source>), dim3(blocks), dim3(kMarchThreads), 0,
+                       stream, make_tree<T>(tree), src, *opt, out_dim, (T*)out);
+}
+
+template <class Source, typename T>
+void launch_backward(const SvoxTreeSpec* tree, const Source& src, unsigned blocks, const SvoxRenderOptions* opt,
+                     int out_dim, const void* grad_out, void* grad_data, hipStream_t stream) {
+    if constexpr (sizeof(T) == 4) {
+        const int D = fast_basis(tree, opt);
+        if (D >= 0) {
+            SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source>), dim3(blocks),
+                                                       dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                       src, *opt, out_dim, (const float*)grad_out,
+                                                       (float*)grad_data));
+            return;
+        }
+    }
+    hipLaunchKernelGGL((render_backward_kernel<GenericPolicy<T>, Source>), dim3(blocks), dim3(kMarchThreads), 0,
+                       stream, make_tree<T>(tree), src, *opt, out_dim, (const T*)grad_out, (T*)grad_data);
+}
+
+unsigned batch_blocks(int64_t n) { return (unsigned)((n + kMarchThreads - 1) / kMarchThreads); }
+
+int64_t data_bytes(const SvoxTreeSpec* t) {
+    const int64_t esz = t->dtype == SVOX_F32 ? 4 : 8;
+    return t->capacity * t->N * t->N * t->N * t->data_dim * esz;
+}
+
+}  // namespace
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+int svox_abi_version(void) { return SVOX_ABI_VERSION; }
+
+const char* svox_last_error(void) { return g_error; }
+
+const char* svox_status_string(int status) {
+    switch (status) {
+        case SVOX_OK: return "ok";
+        case SVOX_ERR_NULL_POINTER: return "null pointer";
+        case SVOX_ERR_BAD_SHAPE: return "bad shape";
+        case SVOX_ERR_BAD_DTYPE: return "bad dtype";
+        case SVOX_ERR_UNSUPPORTED: return "unsupported";
+        case SVOX_ERR_LAUNCH: return "kernel launch failed";
+        case SVOX_ERR_NO_DEVICE: return "no device";
+        default: return "unknown status";
+    }
+}
+
+// Debugging aid: bit 0 routes every call to the generic kernels.
+void svox_set_debug_flags(int flags) { g_debug_flags = flags; }
+
+int svox_out_data_dim(int32_t format, int32_t basis_dim, int32_t data_dim) {
+    if (data_dim < 1) return -1;
+    if (format != SVOX_FORMAT_RGBA) {
+        if (basis_dim <= 0) return -1;
+        return (data_dim - 1) / basis_dim;
+    }
+    return data_dim - 1;
+}
+
+int svox_query_vertical(const SvoxTreeSpec* tree, const void* indices, int64_t n_points, void* values_out,
+                        int64_t* node_ids_out, void* stream) {
+    int rc = check_tree(tree, true);
+    if (rc) return rc;
+    if (n_points < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative point count");
+    if (n_points == 0) return SVOX_OK;
+    if (!indices || !values_out || !node_ids_out) return fail(SVOX_ERR_NULL_POINTER, "indices / values_out / node_ids_out is NULL");
+    if (tree->dtype == SVOX_F32)
+        return launch_query<float, kQueryGather>(tree, indices, n_points, values_out, nullptr, node_ids_out,
+                                                 tree->data_dim, (hipStream_t)stream, "query_vertical");
+    return launch_query<double, kQueryGather>(tree, indices, n_points, values_out, nullptr, node_ids_out,
+                                              tree->data_dim, (hipStream_t)stream, "query_vertical");
+}
+
+int svox_query_vertical_backward(const SvoxTreeSpec* tree, const void* indices, int64_t n_points,
+                                 const void* grad_output, int32_t grad_dim, void* grad_data_out,
+                                 int32_t accumulate, void* stream) {
+    int rc = check_tree(tree, false);
+    if (rc) return rc;
+    if (n_points < 0 || grad_dim < 1) return fail(SVOX_ERR_BAD_SHAPE, "negative point count or grad_dim < 1");
+    if (!grad_data_out) return fail(SVOX_ERR_NULL_POINTER, "grad_data_out is NULL");
+    const int64_t esz = tree->dtype == SVOX_F32 ? 4 : 8;
+    if (!accumulate) {
+        rc = zero_fill(grad_data_out, tree->capacity * tree->N * tree->N * tree->N * grad_dim * esz,
+                       (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    if (n_points == 0) return SVOX_OK;
+    if (!indices || !grad_output) return fail(SVOX_ERR_NULL_POINTER, "indices / grad_output is NULL");
+    if (tree->dtype == SVOX_F32)
+        return launch_query<float, kQueryScatterAdd>(tree, indices, n_points, (void*)grad_output, grad_data_out,
+                                                     nullptr, grad_dim, (hipStream_t)stream,
+                                                     "query_vertical_backward");
+    return launch_query<double, kQueryScatterAdd>(tree, indices, n_points, (void*)grad_output, grad_data_out,
+                                                  nullptr, grad_dim, (hipStream_t)stream,
+                                                  "query_vertical_backward");
+}
+
+int svox_assign_vertical(const SvoxTreeSpec* tree, const void* indices, int64_t n_points, const void* values,
+                         int32_t value_dim, void* stream) {
+    int rc = check_tree(tree, true);
+    if (rc) return rc;
+    if (n_points < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative point count");
+    if (value_dim < 1 || value_dim > tree->data_dim)
+        return fail(SVOX_ERR_BAD_SHAPE, "value_dim %d outside [1, data_dim=%d]", value_dim, tree->data_dim);
+    if (n_points == 0) return SVOX_OK;
+    if (!indices || !values) return fail(SVOX_ERR_NULL_POINTER, "indices / values is NULL");
+    if (tree->dtype == SVOX_F32)
+        return launch_query<float, kQueryAssign>(tree, indices, n_points, (void*)values, nullptr, nullptr,
+                                                 value_dim, (hipStream_t)stream, "assign_vertical");
+    return launch_query<double, kQueryAssign>(tree, indices, n_points, (void*)values, nullptr, nullptr, value_dim,
+                                              (hipStream_t)stream, "assign_vertical");
+}
+
+int svox_calc_corners(const SvoxTreeSpec* tree, const int64_t* indexer, int64_t n_leaves, void* corners_out,
+                      void* stream) {
+    int rc = check_tree(tree, false);
+    if (rc) return rc;
+    if (n_leaves < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative leaf count");
+    if (n_leaves == 0) return SVOX_OK;
+    if (!indexer || !corners_out) return fail(SVOX_ERR_NULL_POINTER, "indexer / corners_out is NULL");
+    const unsigned blocks = (unsigned)((n_leaves + kQueryThreads - 1) / kQueryThreads);
+    if (tree->dtype == SVOX_F32)
+        hipLaunchKernelGGL((corners_kernel<float>), dim3(blocks), dim3(kQueryThreads), 0, (hipStream_t)stream,
+                           tree->parent_depth, tree->N, tree->capacity, indexer, n_leaves, (float*)corners_out);
+    else
+        hipLaunchKernelGGL((corners_kernel<double>), dim3(blocks), dim3(kQueryThreads), 0, (hipStream_t)stream,
+                           tree->parent_depth, tree->N, tree->capacity, indexer, n_leaves, (double*)corners_out);
+    return check_launch("calc_corners");
+}
+
+int svox_volume_render(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt, void* out,
+                       void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    rc = check_rays(rays);
+    if (rc) return rc;
+    if (rays->n_rays == 0) return SVOX_OK;
+    if (!out) return fail(SVOX_ERR_NULL_POINTER, "out is NULL");
+    const unsigned blocks = batch_blocks(rays->n_rays);
+    if (tree->dtype == SVOX_F32)
+        launch_forward<BatchSource<float>, float>(tree, batch_source<float>(rays), blocks, opt, od, out,
+                                                  (hipStream_t)stream);
+    else
+        launch_forward<BatchSource<double>, double>(tree, batch_source<double>(rays), blocks, opt, od, out,
+                                                    (hipStream_t)stream);
+    return check_launch("volume_render");
+}
+
+int svox_volume_render_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
+                             void* out, void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    rc = check_camera(cam);
+    if (rc) return rc;
+    if (cam->width == 0 || cam->height == 0) return SVOX_OK;
+    if (!out) return fail(SVOX_ERR_NULL_POINTER, "out is NULL");
+    unsigned blocks;
+    if (tree->dtype == SVOX_F32) {
+        const auto src = image_source<float>(cam, &blocks);
+        launch_forward<ImageSource<float>, float>(tree, src, blocks, opt, od, out, (hipStream_t)stream);
+    } else {
+        const auto src = image_source<double>(cam, &blocks);
+        launch_forward<ImageSource<double>, double>(tree, src, blocks, opt, od, out, (hipStream_t)stream);
+    }
+    return check_launch("volume_render_image");
+}
+
+int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
+                                const void* grad_output, void* grad_data_out, int32_t accumulate, void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    rc = check_rays(rays);
+    if (rc) return rc;
+    if (!grad_data_out) return fail(SVOX_ERR_NULL_POINTER, "grad_data_out is NULL");
+    if (!accumulate) {
+        rc = zero_fill(grad_data_out, data_bytes(tree), (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    if (rays->n_rays == 0) return SVOX_OK;
+    if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
+    const unsigned blocks = batch_blocks(rays->n_rays);
+    if (tree->dtype == SVOX_F32)
+        launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays), blocks, opt, od, grad_output,
+                                                   grad_data_out, (hipStream_t)stream);
+    else
+        launch_backward<BatchSource<double>, double>(tree, batch_source<double>(rays), blocks, opt, od,
+                                                     grad_output, grad_data_out, (hipStream_t)stream);
+    return check_launch("volume_render_backward");
+}
+
+int svox_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                                      const SvoxRenderOptions* opt, const void* grad_output, void* grad_data_out,
+                                      int32_t accumulate, void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    rc = check_camera(cam);
+    if (rc) return rc;
+    if (!grad_data_out) return fail(SVOX_ERR_NULL_POINTER, "grad_data_out is NULL");
+    if (!accumulate) {
+        rc = zero_fill(grad_data_out, data_bytes(tree), (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    if (cam->width == 0 || cam->height == 0) return SVOX_OK;
+    if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
+    unsigned blocks;
+    if (tree->dtype == SVOX_F32) {
+        const auto src = image_source<float>(cam, &blocks);
+        launch_backward<ImageSource<float>, float>(tree, src, blocks, opt, od, grad_output, grad_data_out,
+                                                   (hipStream_t)stream);
+    } else {
+        const auto src = image_source<double>(cam, &blocks);
+        launch_backward<ImageSource<double>, double>(tree, src, blocks, opt, od, grad_output, grad_data_out,
+                                                     (hipStream_t)stream);
+    }
+    return check_launch("volume_render_image_backward");
+}
+
+int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCameraSpec* cam,
+                             const SvoxRenderOptions* opt, SvoxMarchStats* stats_out, void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    if (!stats_out) return fail(SVOX_ERR_NULL_POINTER, "stats_out is NULL");
+    if ((rays != nullptr) == (cam != nullptr))
+        return fail(SVOX_ERR_BAD_SHAPE, "exactly one of rays and cam must be given");
+    unsigned long long* st = (unsigned long long*)stats_out;
+    if (rays) {
+        rc = check_rays(rays);
+        if (rc) return rc;
+        if (rays->n_rays == 0) return SVOX_OK;
+        const unsigned blocks = batch_blocks(rays->n_rays);
+        if (tree->dtype == SVOX_F32)
+            hipLaunchKernelGGL((render_stats_kernel<float, BatchSource<float>>), dim3(blocks), dim3(kMarchThreads), 0,
+                               (hipStream_t)stream, make_tree<float>(tree), batch_source<float>(rays), *opt, st);
+        else
+            hipLaunchKernelGGL((render_stats_kernel<double, BatchSource<double>>), dim3(blocks), dim3(kMarchThreads),
+                               0, (hipStream_t)stream, make_tree<double>(tree), batch_source<double>(rays), *opt, st);
+    } else {
+        rc = check_camera(cam);
+        if (rc) return rc;
+        if (cam->width == 0 || cam->height == 0) return SVOX_OK;
+        unsigned blocks;
+        if (tree->dtype == SVOX_F32) {
+            const auto src = image_source<float>(cam, &blocks);
+            hipLaunchKernelGGL((render_stats_kernel<float, ImageSource<float>>), dim3(blocks), dim3(kMarchThreads), 0,
+                               (hipStream_t)stream, make_tree<float>(tree), src, *opt, st);
+        } else {
+            const auto src = image_source<double>(cam, &blocks);
+            hipLaunchKernelGGL((render_stats_kernel<double, ImageSource<double>>), dim3(blocks), dim3(kMarchThreads),
+                               0, (hipStream_t)stream, make_tree<double>(tree), src, *opt, st);
+        }
+    }
+    return check_launch("volume_render_stats");
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

@@ -1,0 +1,183 @@
+// tree_walk.h -- root-to-leaf descent of the N^3 tree (reference: query_single_from_root,
+// svox/csrc/include/common.cuh:52-90).
+//
+// Two formulations that return the same leaf and the same leaf-local position:
+//
+//   descend_generic<T>   the reference's floating-point walk (multiply by N, floor, subtract) for
+//                        any branching factor and scalar type.
+//
+//   OctreeCursor         N == 2, fp32.  Multiplying by 2, taking the floor and subtracting it are
+//                        exact in binary floating point, so the cell chosen at level l is bit
+//                        (24 - l) of trunc(p * 2^24) and the leaf-local position at depth L is
+//                        frac(p * 2^L).  The walk therefore runs on integers, and because a ray's
+//                        next sample is close to the previous one, it restarts from the deepest
+//                        node whose cell still contains the new point instead of from the root:
+//                        the node ids of the previous path are kept in LDS, one column per lane.
+#pragma once
+
+#include "fpmath.h"
+
+namespace svox {
+
+constexpr int kMaxWalkLevels = 64;   // a deeper (malformed) tree ends the walk with leaf -1
+constexpr int kCoordBits = 24;       // integer cell coordinates hold 24 levels of an octree
+constexpr int kPathLevels = 12;      // levels of the previous path remembered per lane
+
+template <typename T>
+struct TreeDev {
+    T* data;
+    const int32_t* child;
+    const int32_t* parent_depth;
+    const T* extra;
+    const T* offset;   // may be null: zero
+    const T* scaling;  // may be null: one
+    T* weight_accum;
+    int64_t capacity;
+    int32_t N;
+    int32_t K;
+    int32_t extra_cols;
+    int32_t weight_accum_max;
+};
+
+template <typename T>
+__device__ __forceinline__ void load_transform(const TreeDev<T>& tr, T* offset, T* scaling) {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        offset[i] = tr.offset ? tr.offset[i] : T(0);
+        scaling[i] = tr.scaling ? tr.scaling[i] : T(1);
+    }
+}
+
+// transform_coord, common.cuh:43-50
+template <typename T>
+__device__ __forceinline__ void transform_coord(T* q, const T* offset, const T* scaling) {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) q[i] = fma_(scaling[i], q[i], offset[i]);
+}
+
+// The reference's walk.  xyz: in = point in tree coordinates, out = position inside the leaf.
+// Returns the packed leaf id node*N^3 + u*N^2 + v*N + w, or -1 for a malformed tree.
+template <typename T>
+__device__ __forceinline__ int64_t descend_generic(const int32_t* __restrict__ child,
+                                                   int64_t capacity, int32_t Ni, T* xyz,
+                                                   T* cube_sz, int* levels) {
+    const T N = (T)Ni;
+    xyz[0] = clamp01(xyz[0]);
+    xyz[1] = clamp01(xyz[1]);
+    xyz[2] = clamp01(xyz[2]);
+    int64_t node = 0;
+    *cube_sz = N;
+    for (int level = 1; level <= kMaxWalkLevels; ++level) {
+        xyz[0] *= N;
+        xyz[1] *= N;
+        xyz[2] *= N;
+        const int32_t u = (int32_t)floor_(xyz[0]);
+        const int32_t v = (int32_t)floor_(xyz[1]);
+        const int32_t w = (int32_t)floor_(xyz[2]);
+        xyz[0] -= (T)u;
+        xyz[1] -= (T)v;
+        xyz[2] -= (T)w;
+        const int64_t cell = ((node * Ni + u) * Ni + v) * Ni + w;
+        const int32_t skip = child[cell];
+        if (skip == 0) {
+            *levels = level;
+            return cell;
+        }
+        *cube_sz *= N;
+        node += skip;
+        if (node < 0 || node >= capacity) return -1;
+    }
+    return -1;
+}
+
+// Integer cell coordinates of a clamped point: trunc(p * 2^24), exact.
+__device__ __forceinline__ uint32_t cell_coord(float pc) { return (uint32_t)(pc * 16777216.0f); }
+
+__device__ __forceinline__ int cell_at(uint32_t ix, uint32_t iy, uint32_t iz, int level) {
+    const int s = kCoordBits - level;
+    return (int)((((ix >> s) & 1u) << 2) | (((iy >> s) & 1u) << 1) | ((iz >> s) & 1u));
+}
+
+// Octree walk over integer coordinates with no path memory (point queries).
+// `lds_child` holds the child rows of nodes [0, lds_nodes); deeper nodes are read from memory.
+// Returns the leaf cell index node*8 + cell (or -1) and the number of levels visited.
+__device__ __forceinline__ int32_t descend_octree(const int32_t* __restrict__ child,
+                                                  const int32_t* lds_child, int32_t lds_nodes,
+                                                  int64_t capacity, uint32_t ix, uint32_t iy,
+                                                  uint32_t iz, int* levels) {
+    int32_t node = 0;
+    for (int level = 1; level <= kCoordBits; ++level) {
+        const int32_t cell = node * 8 + cell_at(ix, iy, iz, level);
+        const int32_t skip = node < lds_nodes ? lds_child[cell] : child[cell];
+        if (skip == 0) {
+            *levels = level;
+            return cell;
+        }
+        node += skip;
+        if (node < 0 || node >= capacity) return -1;
+    }
+    return -1;  // deeper than the integer coordinates resolve; the host routes such trees elsewhere
+}
+
+// leaf-local position frac(pc * 2^levels) and the reciprocal cell count 2^-levels
+__device__ __forceinline__ float leaf_local(float pc, float cube_sz) {
+    const float s = pc * cube_sz;
+    return s - floor_(s);
+}
+
+// Per-lane cursor that remembers the previous descent.  `path` points at this lane's column of an
+// LDS array laid out [kPathLevels][block threads]: path[l * stride] is the node whose child row is
+// indexed at level l + 1 (path[0] is the root, node 0).
+struct OctreeCursor {
+    int32_t* path;
+    int stride;
+    uint32_t ix, iy, iz;  // coordinates of the previous query
+    int levels;           // levels of the previous leaf, 0 = no previous query
+    int32_t leaf;         // its cell index
+
+    __device__ __forceinline__ void reset(int32_t* lane_path, int lane_stride) {
+        path = lane_path;
+        stride = lane_stride;
+        levels = 0;
+        leaf = -1;
+        ix = iy = iz = 0;
+    }
+
+    // Finds the leaf of the point with integer coordinates (nx, ny, nz).  Returns the leaf cell
+    // index (or -1); `levels` is updated.  `reads` is incremented per child entry read.
+    __device__ __forceinline__ int32_t seek(const int32_t* __restrict__ child, int64_t capacity,
+                                            uint32_t nx, uint32_t ny, uint32_t nz, int* reads) {
+        int level = 1;
+        int32_t node = 0;
+        if (levels > 0) {
+            const uint32_t diff = (ix ^ nx) | (iy ^ ny) | (iz ^ nz);
+            // first level at which the two points fall into different cells
+            const int first_diff = diff ? (kCoordBits - 31 + __builtin_clz(diff)) : kCoordBits + 1;
+            if (first_diff > levels) {
+                ix = nx; iy = ny; iz = nz;
+                return leaf;  // still inside the previous leaf
+            }
+            level = first_diff < kPathLevels ? first_diff : kPathLevels;
+            node = path[(level - 1) * stride];
+        }
+        ix = nx; iy = ny; iz = nz;
+        for (; level <= kCoordBits; ++level) {
+            if (level <= kPathLevels) path[(level - 1) * stride] = node;
+            const int32_t cell = node * 8 + cell_at(nx, ny, nz, level);
+            const int32_t skip = child[cell];
+            *reads += 1;
+            if (skip == 0) {
+                levels = level;
+                leaf = cell;
+                return cell;
+            }
+            node += skip;
+            if (node < 0 || node >= capacity) break;
+        }
+        levels = 0;
+        leaf = -1;
+        return -1;
+    }
+};
+
+}  // namespace svox

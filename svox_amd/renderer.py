@@ -1,0 +1,188 @@
+"""VolumeRenderer: differentiable volume rendering of an N3Tree on the GPU.
+
+Mirrors `svox.VolumeRenderer` (svox/renderer.py:114-469): same constructor arguments, `forward(rays)`
+for ray batches, `render_persp(c2w, ...)` for pinhole images, `persp_rays`, the `fast` switch and
+the `sigma_thresh` / `stop_thresh` attribute overrides.  Rendering runs in the HIP kernels behind
+`svox_amd.csrc`; gradients flow to `tree.data` only.
+"""
+from warnings import warn
+
+import torch
+from torch import nn
+
+from . import csrc as _C
+from .formats import DataFormat, NDCConfig, Rays  # noqa: F401
+
+
+def _rays_spec_from_rays(rays):
+    spec = _C.RaysSpec()
+    spec.origins = rays.origins
+    spec.dirs = rays.dirs
+    spec.vdirs = rays.viewdirs
+    return spec
+
+
+def _make_camera_spec(c2w, width, height, fx, fy):
+    spec = _C.CameraSpec()
+    spec.c2w = c2w
+    spec.width = width
+    spec.height = height
+    spec.fx = fx
+    spec.fy = fy
+    return spec
+
+
+class _VolumeRenderFunction(torch.autograd.Function):
+    """svox/renderer.py:57-72.  The specs are kept on ctx as plain attributes, so the backward
+    pass sees the tree as it is when backward runs."""
+
+    @staticmethod
+    def forward(ctx, data, tree, rays, opt):
+        out = _C.volume_render(tree, rays, opt)
+        ctx.tree, ctx.rays, ctx.opt = tree, rays, opt
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        if not ctx.needs_input_grad[0]:
+            return None, None, None, None
+        grad = _C.volume_render_backward(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous())
+        return grad, None, None, None
+
+
+class _VolumeRenderImageFunction(torch.autograd.Function):
+    """svox/renderer.py:74-89"""
+
+    @staticmethod
+    def forward(ctx, data, tree, cam, opt):
+        out = _C.volume_render_image(tree, cam, opt)
+        ctx.tree, ctx.cam, ctx.opt = tree, cam, opt
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        if not ctx.needs_input_grad[0]:
+            return None, None, None, None
+        grad = _C.volume_render_image_backward(ctx.tree, ctx.cam, ctx.opt, grad_out.contiguous())
+        return grad, None, None, None
+
+
+def convert_to_ndc(origins, directions, focal, w, h, near=1.0):
+    """Rays in normalised device coordinates of a forward-facing scene (svox/renderer.py:92-112).
+    The image kernels apply the same map themselves and then normalise the direction; ray batches
+    passed to `VolumeRenderer.forward` must be converted by the caller."""
+    t = -(near + origins[..., 2]) / directions[..., 2]
+    origins = origins + t[..., None] * directions
+    ox, oy, oz = origins.unbind(-1)
+    dx, dy, dz = directions.unbind(-1)
+    sx, sy = -(2.0 * focal) / w, -(2.0 * focal) / h
+    new_o = torch.stack([sx * (ox / oz), sy * (oy / oz), 1.0 + 2.0 * near / oz], -1)
+    new_d = torch.stack([sx * (dx / dz - ox / oz), sy * (dy / dz - oy / oz), -2.0 * near / oz], -1)
+    return new_o, new_d
+
+
+class VolumeRenderer(nn.Module):
+    """Stores rendering options for one tree; holds no tensors of its own.
+
+    :param tree: N3Tree to render
+    :param step_size: epsilon added to every leaf crossing
+    :param background_brightness: 1.0 = white
+    :param ndc: NDCConfig(width, height, focal) or None
+    :param min_comp, max_comp: range of basis components to render (-1 = last);
+           min_comp > max_comp renders 0.5 grey
+    :param density_softplus: apply log(1 + exp(sigma - 1)) to the stored density
+    :param rgb_padding: colours become sigmoid * (1 + 2 p) - p
+    """
+
+    def __init__(self, tree, step_size=1e-3, background_brightness=1.0, ndc=None, min_comp=0,
+                 max_comp=-1, density_softplus=False, rgb_padding=0.0):
+        super().__init__()
+        self.tree = tree
+        self.step_size = step_size
+        self.background_brightness = background_brightness
+        self.ndc_config = ndc
+        self.min_comp = min_comp
+        self.max_comp = max_comp
+        self.density_softplus = density_softplus
+        self.rgb_padding = rgb_padding
+        if isinstance(tree.data_format, DataFormat):
+            self._data_format = None
+        else:
+            warn("Legacy N3Tree (pre 0.2.18) without data_format, auto-infering SH deg")
+            ddim = tree.data_dim
+            self._data_format = DataFormat("" if ddim == 4 else f"SH{(ddim - 1) // 3}")
+        self.tree._weight_accum = None
+
+    @property
+    def data_format(self):
+        return self._data_format or self.tree.data_format
+
+    def _require_gpu(self, cuda, what):
+        if not cuda or not self.tree.data.is_cuda:
+            raise RuntimeError(
+                f"{what}: this build has only the HIP path (tree on a GPU, cuda=True); the "
+                "reference's PyTorch fallback renderer is not included")
+
+    def forward(self, rays, cuda=True, fast=False):
+        """Render a batch of rays -> (B, rgb_dim).  `fast` sets sigma_thresh = stop_thresh = 1e-2."""
+        self._require_gpu(cuda, "VolumeRenderer.forward")
+        return _VolumeRenderFunction.apply(self.tree.data, self.tree._spec(),
+                                           _rays_spec_from_rays(rays), self._get_options(fast))
+
+    def render_persp(self, c2w, width=800, height=800, fx=1111.111, fy=None, cuda=True, fast=False):
+        """Render a pinhole image -> (height, width, rgb_dim).  c2w is (3, 4) or (4, 4), OpenGL
+        convention (camera looks down -z, +y up); pixel (ix, iy) looks through its corner."""
+        self._require_gpu(cuda, "VolumeRenderer.render_persp")
+        if fy is None:
+            fy = fx
+        cam = _make_camera_spec(c2w.to(dtype=self.tree.data.dtype, device=self.tree.data.device).contiguous(),
+                                width, height, fx, fy)
+        return _VolumeRenderImageFunction.apply(self.tree.data, self.tree._spec(), cam,
+                                                self._get_options(fast))
+
+    def se_grad(self, rays, colors):
+        raise NotImplementedError("se_grad is not part of this build")
+
+    def se_grad_persp(self, c2w, colors, width=800, height=800, fx=1111.111, fy=None):
+        raise NotImplementedError("se_grad_persp is not part of this build")
+
+    @staticmethod
+    def persp_rays(c2w, width=800, height=800, fx=1111.111, fy=None):
+        """Row-major pinhole rays usable with forward() (svox/renderer.py:387-426; no NDC)."""
+        if fy is None:
+            fy = fx
+        dev = c2w.device
+        origins = c2w[None, :3, 3].expand(height * width, -1).contiguous()
+        ys = torch.arange(height, dtype=torch.float64, device=dev)
+        xs = torch.arange(width, dtype=torch.float64, device=dev)
+        yy, xx = torch.meshgrid(ys, xs, indexing="ij")
+        cam = torch.stack(((xx - width * 0.5) / float(fx), -(yy - height * 0.5) / float(fy),
+                           -torch.ones_like(xx)), dim=-1)
+        cam = cam / torch.norm(cam, dim=-1, keepdim=True)
+        dirs = (cam.reshape(-1, 3) @ c2w[:3, :3].double().T).float().contiguous()
+        return Rays(origins=origins, dirs=dirs, viewdirs=dirs)
+
+    def _get_options(self, fast=False):
+        """RenderOptions for one call (svox/renderer.py:432-469)."""
+        fmt = self.data_format
+        opts = _C.RenderOptions()
+        opts.step_size = self.step_size
+        opts.background_brightness = self.background_brightness
+        opts.format = fmt.format
+        opts.basis_dim = fmt.basis_dim
+        opts.min_comp = self.min_comp
+        opts.max_comp = self.max_comp + fmt.basis_dim if self.max_comp < 0 else self.max_comp
+        opts.density_softplus = self.density_softplus
+        opts.rgb_padding = self.rgb_padding
+        if self.ndc_config is not None:
+            opts.ndc_width = self.ndc_config.width
+            opts.ndc_height = self.ndc_config.height
+            opts.ndc_focal = self.ndc_config.focal
+        else:
+            opts.ndc_width = -1
+        opts.sigma_thresh = opts.stop_thresh = 1e-2 if fast else 0.0
+        if hasattr(self, "sigma_thresh"):
+            opts.sigma_thresh = self.sigma_thresh
+        if hasattr(self, "stop_thresh"):
+            opts.stop_thresh = self.stop_thresh
+        return opts

