@@ -80,50 +80,84 @@ def dense_tree(levels, data_format="RGBA", seed=0, device="cpu", zero_fraction=0
 
 
 def _sdf_spheres(p, centers, radii):
+    """Distance to the surface of the union of spheres (exact outside, a lower bound inside)."""
     d = (p[:, None, :] - centers[None]).norm(dim=-1) - radii[None]
     return d.min(dim=1).values
 
 
-def shell_tree(depth=9, n_spheres=24, data_format="SH16", seed=0, device="cpu", shell_voxels=2.0,
-               coeff_std=0.3, sigma_range=(20.0, 200.0), geometry="spheres", chunk=1 << 20):
-    """Sparse octree refined to `depth` levels (leaf grid 2^depth per axis at the finest level) only
-    near a surface; leaves of the finest level within `shell_voxels` voxels of the surface get
-    sigma ~ U(sigma_range), every other leaf sigma 0; colour coefficients ~ N(0, coeff_std).
+def _sphere_geometry(gen, n_spheres, shell, dev):
+    centers = (0.2 + 0.6 * torch.rand(n_spheres, 3, generator=gen)).to(dev)
+    radii = (0.05 + 0.15 * torch.rand(n_spheres, generator=gen)).to(dev)
 
-    geometry "spheres": surface of a union of seeded spheres (centres U(.2,.8)^3, radii U(.05,.2)).
-    geometry "noise":   level set of seeded trilinear value noise plus a slab (forward-facing scene).
-    Built on `device` with torch ops (refine() level by level, selecting the cells whose centre is
-    within half a cell diagonal plus the shell width of the surface).
+    def may_touch(cen, size):
+        return _sdf_spheres(cen, centers, radii).abs() <= (math.sqrt(3.0) / 2.0) * size + shell
+
+    def occupied(cen):
+        return _sdf_spheres(cen, centers, radii).abs() <= shell
+
+    return may_touch, occupied
+
+
+def _noise_geometry(gen, dev, threshold=0.80, lattice=17, slab_z=0.25, slab_half=0.004):
+    """Blobs where seeded trilinear value noise exceeds `threshold`, plus a thin slab z ~ slab_z."""
+    R = lattice
+    grid = torch.rand(R, R, R, generator=gen).to(dev)
+
+    def noise(p):
+        q = p.clamp(0, 1) * (R - 1)
+        i0 = q.floor().clamp(max=R - 2).long()
+        fx, fy, fz = (q - i0).unbind(-1)
+        x0, y0, z0 = i0.unbind(-1)
+
+        def c(a, b, e):
+            return grid[x0 + a, y0 + b, z0 + e]
+
+        lo = (c(0, 0, 0) * (1 - fx) + c(1, 0, 0) * fx) * (1 - fy) + (c(0, 1, 0) * (1 - fx) + c(1, 1, 0) * fx) * fy
+        hi = (c(0, 0, 1) * (1 - fx) + c(1, 0, 1) * fx) * (1 - fy) + (c(0, 1, 1) * (1 - fx) + c(1, 1, 1) * fx) * fy
+        return lo * (1 - fz) + hi * fz
+
+    def may_touch(cen, size):
+        # the interpolant is multilinear inside a lattice cell, so over a tree cell that lies inside
+        # one (size <= 1/(R-1), aligned because R-1 is a power of two) its maximum is at a corner
+        blob = size > 1.0 / (R - 1) - 1e-9
+        half = 0.5 * size[:, None]
+        for dx in (-1.0, 1.0):
+            for dy in (-1.0, 1.0):
+                for dz in (-1.0, 1.0):
+                    corner = cen + half * torch.tensor([dx, dy, dz], device=cen.device)
+                    blob = blob | (noise(corner) > threshold)
+        slab = (cen[:, 2] - slab_z).abs() <= slab_half + 0.5 * size
+        return blob | slab
+
+    def occupied(cen):
+        return (noise(cen) > threshold) | ((cen[:, 2] - slab_z).abs() <= slab_half)
+
+    return may_touch, occupied
+
+
+def shell_tree(depth=9, n_spheres=24, data_format="SH16", seed=0, device="cpu", shell_voxels=2.0,
+               coeff_std=0.3, sigma_range=(20.0, 200.0), geometry="spheres", chunk=1 << 20,
+               noise_threshold=0.80):
+    """Sparse octree refined down to a 2^depth grid only where the geometry is; finest-level leaves
+    inside the geometry get sigma ~ U(sigma_range), every other leaf sigma 0; colour coefficients
+    ~ N(0, coeff_std).
+
+    geometry "spheres": shell of `shell_voxels` finest voxels around the surface of a union of seeded
+                        spheres (centres U(.2,.8)^3, radii U(.05,.2)).
+    geometry "noise":   blobs where seeded value noise exceeds `noise_threshold`, plus a thin slab
+                        (a forward-facing scene).
+    Built on `device` with torch ops: refine() level by level on the cells that may touch the
+    geometry (conservative test on the cell centre and size).
     """
     g = _gen(seed)
     dev = torch.device(device)
+    voxel = 2.0 ** (-depth)
     if geometry == "spheres":
-        centers = (0.2 + 0.6 * torch.rand(n_spheres, 3, generator=g)).to(dev)
-        radii = (0.05 + 0.15 * torch.rand(n_spheres, generator=g)).to(dev)
-
-        def sdf(p):
-            return _sdf_spheres(p, centers, radii)
+        may_touch, occupied_fn = _sphere_geometry(g, n_spheres, shell_voxels * voxel, dev)
     else:
-        R = 17
-        lattice = torch.rand(R, R, R, generator=g).to(dev)
-
-        def sdf(p):
-            # trilinear value noise in [0,1], thresholded at 0.62, plus a slab around z = 0.25;
-            # scaled so that |sdf| is a conservative distance bound (noise gradient <= (R-1)*sqrt(3))
-            q = p.clamp(0, 1) * (R - 1)
-            i0 = q.floor().clamp(max=R - 2).long()
-            f = q - i0
-            x0, y0, z0 = i0.unbind(-1)
-            fx, fy, fz = f.unbind(-1)
-            c = lambda a, b, c_: lattice[x0 + a, y0 + b, z0 + c_]  # noqa: E731
-            v = (((c(0, 0, 0) * (1 - fx) + c(1, 0, 0) * fx) * (1 - fy) + (c(0, 1, 0) * (1 - fx) + c(1, 1, 0) * fx) * fy) * (1 - fz)
-                 + ((c(0, 0, 1) * (1 - fx) + c(1, 0, 1) * fx) * (1 - fy) + (c(0, 1, 1) * (1 - fx) + c(1, 1, 1) * fx) * fy) * fz)
-            clutter = (0.70 - v) / ((R - 1) * math.sqrt(3.0))
-            slab = (p[:, 2] - 0.25).abs() - 0.01
-            return torch.minimum(clutter, slab)
+        may_touch, occupied_fn = _noise_geometry(g, dev, threshold=noise_threshold)
 
     tree = N3Tree(N=2, data_format=data_format, depth_limit=depth - 1, device=device)
-    voxel = 2.0 ** (-depth)
     for level in range(1, depth):
         leaves = tree._all_leaves().to(dev)
         corners = _leaf_corners(tree, leaves)
@@ -131,8 +165,7 @@ def shell_tree(depth=9, n_spheres=24, data_format="SH16", seed=0, device="cpu", 
         pick = torch.zeros(leaves.shape[0], dtype=torch.bool, device=dev)
         for s in range(0, leaves.shape[0], chunk):
             cen = corners[s:s + chunk] + 0.5 * size[s:s + chunk, None]
-            dist = sdf(cen).abs()
-            pick[s:s + chunk] = dist <= (math.sqrt(3.0) / 2.0) * size[s:s + chunk] + shell_voxels * voxel
+            pick[s:s + chunk] = may_touch(cen, size[s:s + chunk])
         sel = tuple(leaves[pick].T)
         if sel[0].numel() == 0:
             break
@@ -149,7 +182,7 @@ def shell_tree(depth=9, n_spheres=24, data_format="SH16", seed=0, device="cpu", 
     occupied = torch.zeros(leaves.shape[0], dtype=torch.bool, device=dev)
     for s in range(0, leaves.shape[0], chunk):
         cen = corners[s:s + chunk] + 0.5 * size[s:s + chunk, None]
-        occupied[s:s + chunk] = (sdf(cen).abs() <= shell_voxels * voxel) & (depth_of[s:s + chunk] == depth - 1)
+        occupied[s:s + chunk] = occupied_fn(cen) & (depth_of[s:s + chunk] == depth - 1)
     sig = torch.zeros(tree.child.shape, dtype=torch.float32, device=dev)
     lo, hi = sigma_range
     vals = lo + (hi - lo) * torch.rand(int(occupied.sum().item()), generator=gd, device=dev)

@@ -7,6 +7,7 @@ import torch
 import svox_amd as svox
 from svox_amd import csrc as C
 from svox_amd import synth
+from util import on_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -39,7 +40,7 @@ def test_query_vertical_matches_oracle(gpu, oracle_mod, name, tree, generic):
     pts = torch.cat([torch.rand(20000, 3, generator=g) * 1.2 - 0.1, edge_points()]).contiguous()
     ot = oracle_mod.Tree.from_n3tree(tree)
     ref_vals, ref_ids = oracle_mod.query_vertical(ot, pts)
-    dev_tree = tree.to(gpu)
+    dev_tree = on_gpu(tree, gpu)
     C.set_debug_flags(generic)
     try:
         vals, ids = dev_tree(pts.to(gpu), want_node_ids=True)
@@ -56,7 +57,7 @@ def test_query_local_coordinates_and_empty(gpu, oracle_mod):
     pts = torch.rand(1000, 3, generator=torch.Generator().manual_seed(1))
     ot = oracle_mod.Tree.from_n3tree(tree, world=False)
     ref_vals, ref_ids = oracle_mod.query_vertical(ot, pts)
-    dev_tree = tree.to(gpu)
+    dev_tree = on_gpu(tree, gpu)
     vals, ids = dev_tree(pts.to(gpu), want_node_ids=True, world=False)
     assert np.array_equal(ids.cpu().numpy(), ref_ids)
     assert np.array_equal(vals.detach().cpu().numpy(), ref_vals)
@@ -72,7 +73,7 @@ def test_query_backward_matches_oracle_and_index_add(gpu, oracle_mod, generic):
     go = torch.randn(50000, tree.data_dim, generator=g)
     ot = oracle_mod.Tree.from_n3tree(tree)
     ref = oracle_mod.query_vertical_backward(ot, pts, go)
-    dev_tree = tree.to(gpu)
+    dev_tree = on_gpu(tree, gpu)
     C.set_debug_flags(generic)
     try:
         vals = dev_tree(pts.to(gpu))
@@ -102,7 +103,7 @@ def test_assign_vertical(gpu, oracle_mod):
     vals = torch.randn(200, tree.data_dim, generator=torch.Generator().manual_seed(4))
     ref_tree = oracle_mod.Tree(tree.data.data.clone(), tree.child, tree.parent_depth, tree.offset, tree.invradius)
     oracle_mod.assign_vertical(ref_tree, pts, vals)
-    dev_tree = tree.to(gpu)
+    dev_tree = on_gpu(tree, gpu)
     dev_tree.set(pts.to(gpu), vals.to(gpu))
     assert np.array_equal(dev_tree.data.data.cpu().numpy(), ref_tree.data)
     # partial rows through the view API: tree[P, :3] = x
@@ -116,7 +117,7 @@ def test_calc_corners_matches_oracle(gpu, oracle_mod, name, tree):
     leaves = tree._all_leaves()
     ot = oracle_mod.Tree.from_n3tree(tree)
     ref = oracle_mod.calc_corners(ot, leaves)
-    dev_tree = tree.to(gpu)
+    dev_tree = on_gpu(tree, gpu)
     got = dev_tree._calc_corners(leaves.to(gpu))
     assert np.array_equal(got.cpu().numpy(), ref)
     if tree.N == 2:
@@ -134,13 +135,13 @@ def test_double_precision_query(gpu, oracle_mod):
     pts = torch.rand(5000, 3, dtype=torch.float64, generator=torch.Generator().manual_seed(5))
     ot = oracle_mod.Tree.from_n3tree(tree)
     ref_vals, ref_ids = oracle_mod.query_vertical(ot, pts)
-    vals, ids = tree.to(gpu)(pts.to(gpu), want_node_ids=True)
+    vals, ids = on_gpu(tree, gpu)(pts.to(gpu), want_node_ids=True)
     assert np.array_equal(ids.cpu().numpy(), ref_ids)
     assert np.array_equal(vals.detach().cpu().numpy(), ref_vals)
 
 
 def test_errors_mirror_reference_checks(gpu):
-    tree = synth.dense_tree(1, "RGBA", seed=0).to(gpu)
+    tree = on_gpu(synth.dense_tree(1, "RGBA", seed=0), gpu)
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
         C.query_vertical(tree._spec(), torch.rand(4, 3))
     with pytest.raises(RuntimeError, match="must be contiguous"):

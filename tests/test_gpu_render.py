@@ -14,7 +14,7 @@ import torch
 import svox_amd as svox
 from svox_amd import csrc as C
 from svox_amd import synth
-from util import cam_spec, grad_close, options, rays_spec
+from util import cam_spec, grad_close, on_gpu, options, rays_spec
 
 pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -23,7 +23,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 def render_both(gpu, oracle_mod, tree, rays, opt, generic=0):
     ot = oracle_mod.Tree.from_n3tree(tree)
     ref, ref_stats = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt, want_stats=True)
-    dev = tree.to(gpu)
+    dev = on_gpu(tree, gpu)
     C.set_debug_flags(generic)
     try:
         out = C.volume_render(dev._spec(), rays_spec(rays, gpu), opt)
@@ -102,7 +102,7 @@ def test_image_render_and_backward(gpu, oracle_mod, ndc):
     opt = options(tree, step_size=1e-3, **kw)
     ot = oracle_mod.Tree.from_n3tree(tree)
     ref, ref_stats = oracle_mod.volume_render_image(ot, c2w, fx, fx, W, H, opt, want_stats=True)
-    dev = tree.to(gpu)
+    dev = on_gpu(tree, gpu)
     cam = cam_spec(c2w, W, H, fx, device=gpu)
     out = C.volume_render_image(dev._spec(), cam, opt)
     assert out.shape == (H, W, 3)
@@ -169,7 +169,7 @@ def test_weight_accumulation(gpu, oracle_mod):
         ot.weight_accum = np.zeros(tree.child.shape, dtype=np.float32)
         ot.weight_accum_max = op == "max"
         oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
-        dev = tree.to(gpu)
+        dev = on_gpu(tree, gpu)
         renderer = svox.VolumeRenderer(dev)
         with dev.accumulate_weights(op=op) as accum:
             renderer(svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu)))
@@ -214,7 +214,7 @@ def test_toy_example_through_python_api(gpu):
 
 
 def test_render_persp_autograd_and_empty(gpu, oracle_mod):
-    tree = synth.dense_tree(2, "SH4", seed=2, sigma="lognormal").to(gpu)
+    tree = on_gpu(synth.dense_tree(2, "SH4", seed=2, sigma="lognormal"), gpu)
     r = svox.VolumeRenderer(tree, step_size=1e-3)
     c2w = synth.orbit_poses(1, seed=1, radius=3.0)[0].to(gpu)
     img = r.render_persp(c2w, width=40, height=30, fx=50.0, fast=True)

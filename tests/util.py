@@ -1,4 +1,6 @@
 """Helpers shared by the tests."""
+import copy
+
 import numpy as np
 import torch
 
@@ -52,3 +54,8 @@ def grad_close(got, ref, rel=1e-4):
     floor = np.abs(ref).max() * 1e-3
     err = np.abs(got - ref) / np.maximum(np.abs(ref), floor if floor > 0 else 1.0)
     return float(err.max()), err.max() <= rel
+
+
+def on_gpu(tree, device):
+    """A copy of `tree` on `device`; the original stays on the CPU (nn.Module.to moves in place)."""
+    return copy.deepcopy(tree).to(device)
