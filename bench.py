@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Benchmark of the octree rendering hot path on one MI355X.
+
+Workload "sparse512_sh16" (BASELINE.json configs[2] and [3]): a seeded sparse octree with a 512^3
+finest grid refined only near the surface of a union of spheres, SH16 leaf records (49 floats).
+  forward  : one step renders 8 poses of 800x800 pixels with step_size 5e-4 and
+             sigma_thresh = stop_thresh = 1e-2 through VolumeRenderer.render_persp;
+  fwd+bwd  : one step renders 1M rays drawn from those 8 poses, back-propagates a random
+             grad_output ~ N(0, 1e-2) into d(data) and applies one SGD update to tree.data.
+`value` is forward Mrays/s with everything resident in HBM; the fwd+bwd figure, the roofline of the
+dominant kernel and a CPU baseline measured on this host ride along in the same JSON line.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def forward_bytes(stats, n_rays, K, ray_io_bytes):
+    """Algorithmic bytes of one forward launch: per ray its input/output, per visited leaf one
+    child-table entry and sigma, per shaded leaf the K-1 colour coefficients."""
+    return n_rays * ray_io_bytes + stats["samples"] * 8 + stats["samples_shaded"] * 4 * (K - 1)
+
+
+def backward_bytes(stats, n_rays, K, ray_io_bytes, data_bytes):
+    """Two marches that read what the forward reads (without thresholds), an atomic read-modify-
+    write of the K gradients of every leaf with sigma > 0, and the zero-fill of d(data)."""
+    per_march = stats["samples_bwd"] * 8 + stats["samples_bwd_pos"] * 4 * (K - 1)
+    return n_rays * ray_io_bytes + 2 * per_march + stats["samples_bwd_pos"] * 8 * K + data_bytes
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--depth", type=int, default=9, help="finest grid is 2^depth per axis")
+    ap.add_argument("--size", type=int, default=800, help="image width and height")
+    ap.add_argument("--poses", type=int, default=8)
+    ap.add_argument("--train-rays", type=int, default=1 << 20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-bwd", action="store_true", help="skip the forward+backward leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (rays would shard "
+              "trivially; see DESIGN.md), run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import svox_amd as svox
+    from svox_amd import csrc as C
+    from svox_amd import synth
+    from svox_amd.renderer import _make_camera_spec, _rays_spec_from_rays
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    C._abi.load_library()
+
+    # ---------------------------------------------------------------- workload
+    t0 = time.time()
+    tree = synth.shell_tree(depth=args.depth, n_spheres=24, data_format="SH16", seed=0, device=dev)
+    torch.cuda.synchronize()
+    K = tree.data_dim
+    data_bytes = tree.data.numel() * 4
+    log(f"[bench] tree built in {time.time() - t0:.1f}s: {tree.info}, data {data_bytes / 2**30:.2f} GiB")
+    W = H = args.size
+    fx = 1111.111 * W / 800.0
+    poses = [p.to(dev) for p in synth.orbit_poses(args.poses, seed=1, radius=4.0)]
+    renderer = svox.VolumeRenderer(tree, step_size=5e-4)
+    opt = renderer._get_options(True)  # fast: sigma_thresh = stop_thresh = 1e-2
+    n_rays_step = args.poses * W * H
+
+    # visit counts per pose from the library's counter kernel (outside the timed region)
+    spec = tree._spec()
+    pose_stats = [C.volume_render_stats(spec, _make_camera_spec(p, W, H, fx, fx), opt) for p in poses]
+    fwd_bytes = [forward_bytes(s, W * H, K, 12) for s in pose_stats]
+
+    def forward_step(events=None):
+        with torch.no_grad():
+            for i, p in enumerate(poses):
+                if events is not None:
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a.record()
+                img = renderer.render_persp(p, width=W, height=H, fx=fx, fast=True)
+                if events is not None:
+                    b.record()
+                    events.append((i, a, b))
+        return img
+
+    for _ in range(args.warmup):
+        forward_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        forward_step()
+    torch.cuda.synchronize()
+    fwd_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    fwd_mrays = n_rays_step / (fwd_ms * 1e-3) / 1e6
+
+    # per-launch duration of the dominant kernel with events on the launching stream
+    events = []
+    for _ in range(max(2, args.steps)):
+        forward_step(events)
+    torch.cuda.synchronize()
+    durs = np.array([a.elapsed_time(b) for (_, a, b) in events])  # ms
+    launch_bytes = np.array([fwd_bytes[i] for (i, _, _) in events], dtype=np.float64)
+    achieved = launch_bytes.mean() / (durs.mean() * 1e-3) / 1e9
+
+    # copy ceiling of this device (read + write of 1 GiB)
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(5):
+        dst.copy_(src)
+    b.record()
+    torch.cuda.synchronize()
+    copy_gbs = 5 * 2 * src.numel() * 4 / (a.elapsed_time(b) * 1e-3) / 1e9
+    del src, dst
+
+    roofline = {
+        "bound": "hbm", "kernel": "render_forward_kernel<OctreePolicy<SH,16>, ImageSource>",
+        "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+        "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": None,
+        "algorithmic_bytes_per_launch": int(launch_bytes.mean()),
+        "avg_launch_ms": round(float(durs.mean()), 4),
+        "copy_ceiling_gbs": round(copy_gbs, 1),
+        "samples_per_ray": round(sum(s["samples"] for s in pose_stats) / n_rays_step, 2),
+        "shaded_per_ray": round(sum(s["samples_shaded"] for s in pose_stats) / n_rays_step, 2),
+    }
+    log(f"[bench] forward {fwd_ms:.2f} ms/step, {fwd_mrays:.1f} Mrays/s, roofline {roofline}")
+
+    # ---------------------------------------------------------------- forward + backward + SGD
+    fwd_bwd = None
+    if not args.no_bwd:
+        g = torch.Generator().manual_seed(7)
+        B = args.train_rays
+        per_pose = [svox.VolumeRenderer.persp_rays(p, W, H, fx) for p in poses]
+        pick = torch.randint(0, n_rays_step, (B,), generator=g).to(dev)
+        all_o = torch.cat([r.origins for r in per_pose])
+        all_d = torch.cat([r.dirs for r in per_pose])
+        rays = svox.Rays(all_o[pick].contiguous(), all_d[pick].contiguous(), all_d[pick].contiguous())
+        del all_o, all_d, per_pose
+        grad_out = (torch.randn(B, 3, generator=g) * 1e-2).to(dev)
+        lr = 1e-3
+        train_stats = C.volume_render_stats(spec, _rays_spec_from_rays(rays), opt)
+        ev = []
+
+        def train_step(record=False):
+            tree.data.grad = None
+            out = renderer(rays, fast=True)
+            if record:
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+            out.backward(grad_out)
+            if record:
+                b.record()
+                ev.append((a, b))
+            with torch.no_grad():
+                tree.data.data.add_(tree.data.grad, alpha=-lr)
+
+        for _ in range(args.warmup):
+            train_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            train_step()
+        torch.cuda.synchronize()
+        tb_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        for _ in range(2):
+            train_step(record=True)
+        torch.cuda.synchronize()
+        bwd_ms = float(np.mean([a.elapsed_time(b) for a, b in ev]))
+        bbytes = backward_bytes(train_stats, B, K, 36 + 12, data_bytes)
+        fwd_bwd = {
+            "value": round(B / (tb_ms * 1e-3) / 1e6, 3), "unit": "Mrays/s", "rays": B,
+            "ms_per_step": round(tb_ms, 3), "includes": "forward + backward (zero-fill, 2 marches, atomics) + SGD update",
+            "backward_ms": round(bwd_ms, 3),
+            "backward_algorithmic_gbs": round(bbytes / (bwd_ms * 1e-3) / 1e9, 2),
+            "backward_frac_of_peak": round(bbytes / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 5),
+            "samples_per_ray": round(train_stats["samples_bwd"] / B, 2),
+            "positive_per_ray": round(train_stats["samples_bwd_pos"] / B, 2),
+        }
+        tree.data.grad = None
+        log(f"[bench] fwd+bwd {fwd_bwd}")
+
+    # ---------------------------------------------------------------- CPU baseline (this host)
+    cpu = None
+    if not args.no_cpu:
+        from oracle import oracle, torch_fallback
+
+        n_threads = os.cpu_count() or 1
+        n_threads = min(n_threads, 16)
+        torch.set_num_threads(n_threads)
+        # a strided sample of pose 0's pixels, as a ray batch
+        rays0 = svox.VolumeRenderer.persp_rays(poses[0].cpu(), W, H, fx)
+        n_oracle = 1 << 16
+        sel = torch.linspace(0, W * H - 1, n_oracle).long()
+        o_s, d_s = rays0.origins[sel].contiguous(), rays0.dirs[sel].contiguous()
+        host = {k: getattr(tree, k).detach().cpu() for k in ("data", "child", "parent_depth", "invradius", "offset")}
+        ot = oracle.Tree(host["data"], host["child"], host["parent_depth"], host["offset"], host["invradius"])
+        t0 = time.perf_counter()
+        ref = oracle.volume_render(ot, o_s, d_s, d_s, opt, n_threads=n_threads)
+        t_oracle = time.perf_counter() - t0
+        # the GPU result on the same rays, for the record
+        with torch.no_grad():
+            got = renderer(svox.Rays(o_s.to(dev), d_s.to(dev), d_s.to(dev)), fast=True).cpu().numpy()
+        check = float(np.abs(got - ref).max())
+        # the reference's CPU path: its PyTorch fallback (restated), no thresholds, fewer rays
+        n_fb = 2048
+        sel2 = torch.linspace(0, W * H - 1, n_fb).long()
+        o_f, d_f = rays0.origins[sel2].contiguous(), rays0.dirs[sel2].contiguous()
+        t0 = time.perf_counter()
+        with torch.no_grad():
+            torch_fallback.render(host["data"], host["child"], host["parent_depth"], host["invradius"],
+                                  host["offset"], o_f, d_f, d_f, 16, step_size=5e-4)
+        t_fb = time.perf_counter() - t0
+        cpu = {
+            "value": round(n_fb / t_fb / 1e6, 6), "unit": "Mrays/s", "cores": n_threads, "kind": "port",
+            "sample": f"{n_fb} rays strided over pose 0, PyTorch restatement of the reference's fallback "
+                      f"renderer (no thresholds), {t_fb:.1f}s",
+            "scalar_oracle": {"value": round(n_oracle / t_oracle / 1e6, 4), "unit": "Mrays/s",
+                              "cores": n_threads, "sample": f"{n_oracle} rays strided over pose 0, OpenMP "
+                              f"C++ oracle with the benchmark's thresholds, {t_oracle:.1f}s"},
+            "gpu_vs_oracle_max_abs_err": check,
+            "host": f"{os.cpu_count()} logical cpus",
+        }
+        log(f"[bench] cpu baseline {cpu}")
+
+    line = {
+        "metric": "Mrays/s fwd, 512^3 sparse SH16 tree",
+        "value": round(fwd_mrays, 3), "unit": "Mrays/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(fwd_ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "sparse512_sh16: 8 poses x 800x800, step 5e-4, sigma/stop thresh 1e-2",
+                   "depth": args.depth, "image": [W, H], "poses": args.poses, "nodes": tree.info["nodes"],
+                   "leaves": tree.info["leaves"], "occupancy": round(tree.info["occupancy"], 5),
+                   "data_gib": round(data_bytes / 2**30, 3)},
+        "roofline": roofline,
+        "fwd_bwd": fwd_bwd,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
