@@ -1,0 +1,219 @@
+"""Host-side Python layer: tree construction and bookkeeping, views, option packing, argument
+checks.  No GPU and no kernels."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import svox_amd as svox
+from svox_amd import csrc as C
+from svox_amd import synth
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def test_quick_start_transcript():
+    """docs/source/quick.rst:70-85 of the reference."""
+    gold = json.load(open(os.path.join(HERE, "golden", "quick_view.json")))
+    tree = svox.N3Tree()
+    assert list(tree.shape) == gold["shape"]
+    tree[0] += 1
+    assert tree[:, :3].values.tolist() == gold["after_add_one_to_leaf0_cols0to3"]
+    tree[:, -1:] = -1
+    assert tree[:2].values.tolist() == gold["after_set_last_col_minus1_first2"]
+    assert "N3TreeView(tensor(" in repr(tree[:2])
+    assert len(tree) == 8 and tree.numel() == 32 and tree.size(1) == 4 and tree.ndim == 2
+
+
+@pytest.mark.parametrize("N,levels", [(2, 3), (3, 2), (2, 0)])
+def test_uniform_refinement_counts_and_order(N, levels):
+    tree = svox.N3Tree(N=N, init_refine=levels)
+    nodes = sum(N ** (3 * i) for i in range(levels + 1))
+    assert tree.capacity == nodes and tree.n_internal == nodes
+    assert tree.n_leaves == N ** (3 * (levels + 1))
+    assert tree.check_integrity()
+    assert tree.max_depth == levels
+    # children are created in lexicographic (node, x, y, z) order of the leaves they split
+    if levels > 0:
+        root_links = tree.child[0].reshape(-1)
+        assert root_links.tolist() == list(range(1, N ** 3 + 1))
+        first_child = 1
+        pd = tree.parent_depth
+        assert pd[first_child].tolist() == [0, 1]
+        assert pd[N ** 3].tolist() == [N ** 3 - 1, 1]
+    assert tree.child.dtype == torch.int32 and tree.parent_depth.dtype == torch.int32
+    assert tree.data.shape == (nodes, N, N, N, 4)
+
+
+def test_refine_selected_leaves_and_depth_limit():
+    tree = svox.N3Tree(depth_limit=1)
+    tree.data.data[0, 1, 0, 1] = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    resized = tree.refine(sel=(torch.tensor([0]), torch.tensor([1]), torch.tensor([0]), torch.tensor([1])))
+    assert resized and tree.n_internal == 2 and tree.n_leaves == 15
+    assert tree.child[0, 1, 0, 1] == 1 and tree.parent_depth[1].tolist() == [5, 1]
+    # children start as copies of the split leaf, which keeps its own record
+    assert torch.equal(tree.data.data[1], torch.tensor([1.0, 2.0, 3.0, 4.0]).expand(2, 2, 2, 4))
+    assert tree.data.data[0, 1, 0, 1].tolist() == [1.0, 2.0, 3.0, 4.0]
+    tree.refine()       # depth 0 leaves split, depth 1 leaves are at the limit
+    assert tree.n_internal == 2 + 7 and tree.check_integrity()
+    assert not tree.refine()  # everything is at the limit now
+    assert tree.max_depth == 1
+    tree._refine_at(0, (0, 0, 0))      # already refined: no-op
+    assert tree.n_internal == 9
+
+
+def test_refine_at_zeroes_the_parent_record():
+    tree = svox.N3Tree()
+    tree.data.data[0, 0, 1, 1] = 5.0
+    tree._refine_at(0, (0, 1, 1))
+    assert tree.n_internal == 2 and torch.all(tree.data.data[1] == 5.0)
+    assert torch.all(tree.data.data[0, 0, 1, 1] == 0.0)
+
+
+def test_pack_unpack_round_trip_and_all_leaves_order():
+    tree = svox.N3Tree(N=3, init_refine=1)
+    leaves = tree._all_leaves()
+    assert leaves.shape == (729, 4)
+    assert torch.equal(tree._unpack_index(tree._pack_index(leaves)), leaves)
+    packed = tree._pack_index(leaves)
+    assert torch.all(packed[1:] > packed[:-1])
+
+
+def test_views_by_index_mask_and_channel():
+    tree = svox.N3Tree(init_refine=1, data_format="SH1")
+    tree.data.data.copy_(torch.arange(tree.data.numel(), dtype=torch.float32).reshape(tree.data.shape))
+    leaves = tree._all_leaves()
+    v = tree[5]
+    assert v.values.shape == (4,) and torch.equal(v.values.detach(), tree.data.data[tuple(leaves[5])])
+    assert tree[3:9].values.shape == (6, 4)
+    mask = torch.zeros(64, dtype=torch.bool)
+    mask[[1, 7]] = True
+    assert tree[mask].shape == (2, 4)
+    assert tree[:, -1].values.shape == (64,)
+    sub = tree[:, torch.tensor([0, 3])]
+    assert sub.values.shape == (64, 2)
+    tree[:, torch.tensor([0, 3])] = 9.0
+    assert torch.all(tree[:, 0].values == 9.0) and torch.all(tree[:, 1].values != 9.0)
+    assert tree.depths.tolist() == [1] * 64
+    assert torch.allclose(tree.lengths_local, torch.full((64,), 0.25))
+    assert (tree[:2] + 1).shape == (2, 4) and float((tree[0] * 0).sum().detach()) == 0.0
+    tree += 1.0
+    tree *= 2.0
+    assert float(tree[:1, 0].values[0].detach()) == 20.0
+
+
+def test_view_goes_stale_and_tree_can_be_locked():
+    tree = svox.N3Tree()
+    view = tree[:]
+    tree.refine()
+    with pytest.raises(RuntimeError, match="invalidated"):
+        _ = view.values
+    with tree.accumulate_weights() as acc:
+        assert acc.value.shape == tree.child.shape
+        with pytest.raises(RuntimeError, match="locked"):
+            tree.refine()
+    tree.refine()
+
+
+def test_expand_and_shrink_move_coefficients():
+    tree = svox.N3Tree(data_format="SH1")
+    tree.data.data[..., :] = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    tree.expand("SH4")
+    assert tree.data_dim == 13 and repr(tree.data_format) == "SH4"
+    row = tree.data.data[0, 0, 0, 0].tolist()
+    assert row == [1, 0, 0, 0, 2, 0, 0, 0, 3, 0, 0, 0, 4]
+    tree.shrink("SH1")
+    assert tree.data.data[0, 0, 0, 0].tolist() == [1, 2, 3, 4]
+    rgba = svox.N3Tree()
+    rgba.data.data[..., :] = torch.tensor([1.0, 2.0, 3.0, 4.0])
+    rgba.expand("RGBA", data_dim=6)
+    assert rgba.data.data[0, 0, 0, 0].tolist() == [1, 2, 3, 0, 0, 4]
+
+
+def test_data_format_parsing():
+    f = svox.DataFormat("SH16")
+    assert (f.format, f.basis_dim, f.data_dim) == (1, 16, 49) and repr(f) == "SH16"
+    f = svox.DataFormat("RGBA")
+    assert (f.format, f.basis_dim, f.data_dim) == (0, -1, None) and repr(f) == "RGBA"
+    assert svox.DataFormat("").format == 0
+    assert (svox.DataFormat("SG7").format, svox.DataFormat("ASG3").format) == (2, 3)
+    with pytest.raises(AssertionError):
+        svox.DataFormat("SH5")
+    with pytest.raises(AssertionError):
+        svox.DataFormat("SH36")
+    assert svox.N3Tree(data_format="SH9").data_dim == 28 and svox.N3Tree().data_dim == 4
+    with pytest.raises(AssertionError):
+        svox.N3Tree(data_format="SH9", data_dim=5)
+
+
+def test_render_options_packing():
+    tree = svox.N3Tree(data_format="SH9")
+    r = svox.VolumeRenderer(tree, step_size=2e-3, background_brightness=0.5, rgb_padding=0.01)
+    o = r._get_options(False)
+    assert (o.format, o.basis_dim, o.min_comp, o.max_comp) == (1, 9, 0, 8)
+    assert (o.sigma_thresh, o.stop_thresh, o.ndc_width) == (0.0, 0.0, -1)
+    o = r._get_options(True)
+    assert (o.sigma_thresh, o.stop_thresh) == (1e-2, 1e-2)
+    r.sigma_thresh = 0.5
+    assert r._get_options(True).sigma_thresh == 0.5 and r._get_options(True).stop_thresh == 1e-2
+    r2 = svox.VolumeRenderer(tree, ndc=svox.NDCConfig(100, 50, 80.0), min_comp=2, max_comp=4)
+    o = r2._get_options()
+    assert (o.ndc_width, o.ndc_height, o.ndc_focal, o.min_comp, o.max_comp) == (100, 50, 80.0, 2, 4)
+    packed = o._pack()
+    assert packed.basis_dim == 9 and abs(packed.step_size - 1e-3) < 1e-9 and packed.density_softplus == 0
+    rgba = svox.VolumeRenderer(svox.N3Tree())._get_options()
+    assert (rgba.format, rgba.basis_dim, rgba.max_comp) == (0, -1, -2)
+    assert C.out_data_dim(0, -1, 4) == 3 and C.out_data_dim(1, 9, 28) == 3
+
+
+def test_persp_rays_geometry():
+    c2w = synth.look_at_pose([3.0, 0.5, 0.5])
+    rays = svox.VolumeRenderer.persp_rays(c2w, 8, 6, 10.0)
+    assert rays.origins.shape == (48, 3) and torch.allclose(rays.origins[0], torch.tensor([3.0, 0.5, 0.5]))
+    assert torch.allclose(rays.dirs.norm(dim=1), torch.ones(48), atol=1e-6)
+    centre = rays.dirs.reshape(6, 8, 3)[3, 4]       # pixel (ix = W/2, iy = H/2) looks along -back
+    assert torch.allclose(centre, torch.tensor([-1.0, 0.0, 0.0]), atol=1e-6)
+
+
+def test_no_cpu_fallback_and_argument_checks():
+    tree = synth.dense_tree(1, "RGBA", seed=0)
+    with pytest.raises(RuntimeError, match="only the HIP path"):
+        tree(torch.rand(3, 3))
+    with pytest.raises(RuntimeError, match="only the HIP path"):
+        tree.set(torch.rand(3, 3), torch.rand(3, 4))
+    with pytest.raises(RuntimeError, match="only the HIP path"):
+        svox.VolumeRenderer(tree)(synth.sphere_rays(4))
+    with pytest.raises(RuntimeError, match="only the HIP path"):
+        svox.VolumeRenderer(tree).render_persp(synth.look_at_pose([2.0, 2, 2]))
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        C.query_vertical(tree._spec(), torch.rand(3, 3))
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        C.calc_corners(tree._spec(), torch.zeros(2, 4, dtype=torch.long))
+    with pytest.raises(AssertionError):
+        tree(torch.rand(3, 3, requires_grad=True))
+
+
+def test_save_load_round_trip(tmp_path):
+    tree = synth.shell_tree(depth=4, n_spheres=2, data_format="SH4", seed=3)
+    path = str(tmp_path / "tree.npz")
+    tree.save(path)
+    back = svox.N3Tree.load(path)
+    assert torch.equal(back.child, tree.child) and torch.equal(back.parent_depth, tree.parent_depth)
+    assert back.n_internal == tree.n_internal and repr(back.data_format) == "SH4"
+    assert torch.allclose(back.data.data, tree.data.data.half().float())      # stored as float16
+    assert torch.equal(back.invradius, tree.invradius) and back.check_integrity()
+
+
+def test_generators_are_seeded():
+    a = synth.shell_tree(depth=5, n_spheres=3, data_format="SH1", seed=5)
+    b = synth.shell_tree(depth=5, n_spheres=3, data_format="SH1", seed=5)
+    c = synth.shell_tree(depth=5, n_spheres=3, data_format="SH1", seed=6)
+    assert torch.equal(a.child, b.child) and torch.equal(a.data.data, b.data.data)
+    assert a.child.shape != c.child.shape or not torch.equal(a.child, c.child)
+    assert a.check_integrity() and 0 < a.info["occupancy"] < 0.5
+    r1, r2 = synth.sphere_rays(10, seed=1), synth.sphere_rays(10, seed=1)
+    assert torch.equal(r1.origins, r2.origins) and torch.allclose((r1.origins - 0.5).norm(dim=1), torch.full((10,), 2.0))
+    noise = synth.shell_tree(depth=6, data_format="SH1", seed=2, geometry="noise")
+    assert noise.check_integrity() and noise.info["occupied_leaves"] > 0
