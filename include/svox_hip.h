@@ -158,6 +158,21 @@ int svox_volume_render(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
 int svox_volume_render_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
                              const SvoxRenderOptions* opt, void* out, void* stream);
 
+/* No counterpart in the reference (its extension renders one image per call): n_images pinhole
+ * images of one size, focal length and option set in ONE launch, so that the tiles of several
+ * poses fill the GPU together.  cam->c2w points at the first pose; pose i starts pose_stride
+ * scalars after pose i-1 (12 for packed (3,4) poses, 16 for (4,4)).  out is (n_images, H, W, out_dim).
+ * With n_images == 1 this is svox_volume_render_image. */
+int svox_volume_render_images(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
+                              int64_t pose_stride, const SvoxRenderOptions* opt, void* out,
+                              void* stream);
+
+/* Backward of svox_volume_render_images; grad_output is (n_images, H, W, out_dim). */
+int svox_volume_render_images_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                                       int32_t n_images, int64_t pose_stride,
+                                       const SvoxRenderOptions* opt, const void* grad_output,
+                                       void* grad_data_out, int32_t accumulate, void* stream);
+
 /* volume_render_backward(TreeSpec&, RaysSpec&, RenderOptions&, grad_output) -> zeros_like(data) +
  * scatter; rt_kernel.cu:1059-1083.  grad_output (n_rays, out_dim); grad_data_out has the shape of
  * tree->data and is zero-filled first unless `accumulate` is nonzero. */

@@ -284,13 +284,14 @@ def _pack_rays(rays, dtype):
     return _abi.RaysSpecC(rays.origins.data_ptr(), rays.dirs.data_ptr(), rays.vdirs.data_ptr(), B)
 
 
-def _pack_camera(cam, dtype):
-    """CameraSpec::check, data_spec.hpp:98-103"""
+def _pack_camera(cam, dtype, batched=False):
+    """CameraSpec::check, data_spec.hpp:98-103.  batched: c2w is (n, 3 or 4, 4)."""
     _check_input(cam.c2w, "c2w")
     if not cam.c2w.is_floating_point():
         raise RuntimeError("c2w must be a floating point tensor")
-    if cam.c2w.dim() != 2 or cam.c2w.shape[1] != 4 or cam.c2w.shape[0] < 3:
-        raise RuntimeError("c2w must be (3, 4) or (4, 4)")
+    want = 3 if batched else 2
+    if cam.c2w.dim() != want or cam.c2w.shape[-1] != 4 or cam.c2w.shape[-2] not in (3, 4):
+        raise RuntimeError("c2w must be (n, 3, 4) or (n, 4, 4)" if batched else "c2w must be (3, 4) or (4, 4)")
     _same_dtype(cam.c2w, dtype, "c2w")
     return _abi.CameraSpecC(cam.c2w.data_ptr(), float(cam.fx), float(cam.fy), int(cam.width),
                             int(cam.height))
@@ -328,6 +329,36 @@ def volume_render_image(tree, cam, opt):
         _call("svox_volume_render_image", ctypes.byref(spec), ctypes.byref(cspec),
               ctypes.byref(copt), out.data_ptr(), _stream(tree.data.device))
     return out
+
+
+def volume_render_images(tree, cam, opt):
+    """(n, H, W, out_dim): n images in one launch; cam.c2w is (n, 3, 4) or (n, 4, 4).
+    No counterpart in the reference, whose extension renders one image per call."""
+    spec = _pack_tree(tree)
+    cspec = _pack_camera(cam, tree.data.dtype, batched=True)
+    n, stride = int(cam.c2w.shape[0]), int(cam.c2w.shape[1]) * 4
+    od = _render_out_dim(spec, opt)
+    out = torch.empty((n, cspec.height, cspec.width, od), dtype=tree.data.dtype, device=tree.data.device)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_images", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
+              ctypes.byref(copt), out.data_ptr(), _stream(tree.data.device))
+    return out
+
+
+def volume_render_images_backward(tree, cam, opt, grad_output):
+    """zeros_like(tree.data) + scatter for volume_render_images."""
+    spec = _pack_tree(tree)
+    cspec = _pack_camera(cam, tree.data.dtype, batched=True)
+    n, stride = int(cam.c2w.shape[0]), int(cam.c2w.shape[1]) * 4
+    od = _render_out_dim(spec, opt)
+    _check_grad(grad_output, (n, cspec.height, cspec.width, od), tree.data.dtype)
+    grad = torch.empty_like(tree.data)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_images_backward", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
+              ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0, _stream(tree.data.device))
+    return grad
 
 
 def _check_grad(grad_output, shape, dtype):

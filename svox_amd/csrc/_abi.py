@@ -110,6 +110,11 @@ SIGNATURES = {
     "svox_volume_render": (ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p]),
     "svox_volume_render_image": (
         ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p]),
+    "svox_volume_render_images": (
+        ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), c_int32, c_int64, P(RenderOptionsC), c_void_p, c_void_p]),
+    "svox_volume_render_images_backward": (
+        ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), c_int32, c_int64, P(RenderOptionsC), c_void_p, c_void_p,
+                       c_int32, c_void_p]),
     "svox_volume_render_backward": (
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int32, c_void_p]),
     "svox_volume_render_image_backward": (

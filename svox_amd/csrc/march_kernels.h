@@ -16,8 +16,8 @@
 
 namespace svox {
 
-constexpr int kMarchThreads = 256;
-constexpr int kTile = 16;  // image kernels: a block covers a 16x16 pixel tile, a wavefront 8x8
+constexpr int kMarchThreads = 64;  // one wavefront per block: finished tiles free their slot at once
+constexpr int kTile = 8;           // image kernels: a block (wavefront) covers an 8x8 pixel tile
 
 // ------------------------------------------------------------------------------------------------
 // ray sources
@@ -93,10 +93,10 @@ __device__ __forceinline__ void maybe_world2ndc(const SvoxRenderOptions& opt, T*
     dir[2] /= n;
 }
 
-// Which ray a thread traces.  Batch: thread i takes ray i.  Image: blocks are 16x16 pixel tiles
-// and each wavefront an 8x8 sub-tile, so the 64 rays of a wavefront stay close in the tree; tiles
-// are dealt to blocks so that the blocks one XCD receives (block ids congruent mod 8) form one
-// contiguous band of the image and share that XCD's L2.
+// Which ray a thread traces.  Batch: thread i takes ray i.  Image: each block (one wavefront) is
+// an 8x8 pixel tile, so its 64 rays stay close in the tree.  Several images of the same size can
+// share a launch; blocks are numbered image by image, so the dispatcher starts the next image's
+// tiles as the previous image's last tiles drain.
 template <typename T>
 struct BatchSource {
     RayBatch<T> rays;
@@ -121,25 +121,30 @@ __host__ __device__ inline int tiles_of(int extent) { return (extent + kTile - 1
 
 template <typename T>
 struct ImageSource {
-    Camera<T> cam;
-    int chunk;  // tiles per XCD band = ceil(n_tiles / 8)
-    __device__ __forceinline__ int64_t count() const { return (int64_t)cam.width * cam.height; }
+    Camera<T> cam;          // cam.c2w: pose of image 0
+    int n_images;
+    int64_t pose_stride;    // scalars between consecutive poses
+    __device__ __forceinline__ int64_t count() const { return (int64_t)n_images * cam.width * cam.height; }
     __device__ __forceinline__ int64_t fetch(const TreeDev<T>&, const SvoxRenderOptions& opt, const T* offset,
                                              const T* scaling, T* origin, T* dir, T* vdir) const {
         const int ntx = tiles_of(cam.width), nty = tiles_of(cam.height);
-        const int tile = (int)(blockIdx.x & 7u) * chunk + (int)(blockIdx.x >> 3);
-        if (tile >= ntx * nty) return -1;
+        const int per_image = ntx * nty;
+        const int image = (int)(blockIdx.x / (unsigned)per_image);
+        const int tile = (int)(blockIdx.x - (unsigned)image * (unsigned)per_image);
+        if (image >= n_images) return -1;
         const int ty = tile / ntx, tx = tile - ty * ntx;
-        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-        const int ix = tx * kTile + (wave & 1) * 8 + (lane & 7);
-        const int iy = ty * kTile + (wave >> 1) * 8 + (lane >> 3);
+        const int lane = threadIdx.x & 63;
+        const int ix = tx * kTile + (lane & 7);
+        const int iy = ty * kTile + (lane >> 3);
         if (ix >= cam.width || iy >= cam.height) return -1;
-        cam2world_ray(ix, iy, cam, dir, origin);
+        Camera<T> c = cam;
+        c.c2w = cam.c2w + (int64_t)image * pose_stride;
+        cam2world_ray(ix, iy, c, dir, origin);
 #pragma unroll
         for (int i = 0; i < 3; ++i) vdir[i] = dir[i];
         maybe_world2ndc(opt, dir, origin);
         transform_coord(origin, offset, scaling);
-        return (int64_t)iy * cam.width + ix;
+        return ((int64_t)image * cam.height + iy) * cam.width + ix;
     }
 };
 

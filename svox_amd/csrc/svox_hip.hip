@@ -144,10 +144,14 @@ int check_render(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, int* ou
     return SVOX_OK;
 }
 
-int check_camera(const SvoxCameraSpec* cam) {
+int check_camera(const SvoxCameraSpec* cam, int n_images = 1, int64_t pose_stride = 12) {
     if (!cam) return fail(SVOX_ERR_NULL_POINTER, "camera spec is NULL");
     if (!cam->c2w) return fail(SVOX_ERR_NULL_POINTER, "cam.c2w is NULL");
     if (cam->width < 0 || cam->height < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative image size");
+    if (n_images < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative image count");
+    if (n_images > 1 && pose_stride < 12) return fail(SVOX_ERR_BAD_SHAPE, "pose_stride must be >= 12 scalars");
+    const double tiles = (double)tiles_of(cam->width) * tiles_of(cam->height) * (n_images > 0 ? n_images : 1);
+    if (tiles >= 2147483647.0) return fail(SVOX_ERR_BAD_SHAPE, "too many pixels for one launch");
     return SVOX_OK;
 }
 
@@ -181,16 +185,16 @@ BatchSource<T> batch_source(const SvoxRaysSpec* rays) {
 }
 
 template <typename T>
-ImageSource<T> image_source(const SvoxCameraSpec* cam, unsigned* blocks) {
+ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pose_stride, unsigned* blocks) {
     ImageSource<T> s;
     s.cam.c2w = (const T*)cam->c2w;
     s.cam.fx = cam->fx;
     s.cam.fy = cam->fy;
     s.cam.width = cam->width;
     s.cam.height = cam->height;
-    const int n_tiles = tiles_of(cam->width) * tiles_of(cam->height);
-    s.chunk = (n_tiles + 7) / 8;
-    *blocks = (unsigned)s.chunk * 8u;
+    s.n_images = n_images;
+    s.pose_stride = pose_stride;
+    *blocks = (unsigned)(tiles_of(cam->width) * tiles_of(cam->height)) * (unsigned)n_images;
     return s;
 }
 
@@ -368,24 +372,29 @@ int svox_volume_render(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const
     return check_launch("volume_render");
 }
 
-int svox_volume_render_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
-                             void* out, void* stream) {
+int svox_volume_render_images(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
+                              int64_t pose_stride, const SvoxRenderOptions* opt, void* out, void* stream) {
     int od;
     int rc = check_render(tree, opt, &od);
     if (rc) return rc;
-    rc = check_camera(cam);
+    rc = check_camera(cam, n_images, pose_stride);
     if (rc) return rc;
-    if (cam->width == 0 || cam->height == 0) return SVOX_OK;
+    if (cam->width == 0 || cam->height == 0 || n_images == 0) return SVOX_OK;
     if (!out) return fail(SVOX_ERR_NULL_POINTER, "out is NULL");
     unsigned blocks;
     if (tree->dtype == SVOX_F32) {
-        const auto src = image_source<float>(cam, &blocks);
+        const auto src = image_source<float>(cam, n_images, pose_stride, &blocks);
         launch_forward<ImageSource<float>, float>(tree, src, blocks, opt, od, out, (hipStream_t)stream);
     } else {
-        const auto src = image_source<double>(cam, &blocks);
+        const auto src = image_source<double>(cam, n_images, pose_stride, &blocks);
         launch_forward<ImageSource<double>, double>(tree, src, blocks, opt, od, out, (hipStream_t)stream);
     }
     return check_launch("volume_render_image");
+}
+
+int svox_volume_render_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
+                             void* out, void* stream) {
+    return svox_volume_render_images(tree, cam, 1, 12, opt, out, stream);
 }
 
 int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
@@ -412,32 +421,39 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
     return check_launch("volume_render_backward");
 }
 
-int svox_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
-                                      const SvoxRenderOptions* opt, const void* grad_output, void* grad_data_out,
-                                      int32_t accumulate, void* stream) {
+int svox_volume_render_images_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
+                                       int64_t pose_stride, const SvoxRenderOptions* opt,
+                                       const void* grad_output, void* grad_data_out, int32_t accumulate,
+                                       void* stream) {
     int od;
     int rc = check_render(tree, opt, &od);
     if (rc) return rc;
-    rc = check_camera(cam);
+    rc = check_camera(cam, n_images, pose_stride);
     if (rc) return rc;
     if (!grad_data_out) return fail(SVOX_ERR_NULL_POINTER, "grad_data_out is NULL");
     if (!accumulate) {
         rc = zero_fill(grad_data_out, data_bytes(tree), (hipStream_t)stream);
         if (rc) return rc;
     }
-    if (cam->width == 0 || cam->height == 0) return SVOX_OK;
+    if (cam->width == 0 || cam->height == 0 || n_images == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
     unsigned blocks;
     if (tree->dtype == SVOX_F32) {
-        const auto src = image_source<float>(cam, &blocks);
+        const auto src = image_source<float>(cam, n_images, pose_stride, &blocks);
         launch_backward<ImageSource<float>, float>(tree, src, blocks, opt, od, grad_output, grad_data_out,
                                                    (hipStream_t)stream);
     } else {
-        const auto src = image_source<double>(cam, &blocks);
+        const auto src = image_source<double>(cam, n_images, pose_stride, &blocks);
         launch_backward<ImageSource<double>, double>(tree, src, blocks, opt, od, grad_output, grad_data_out,
                                                      (hipStream_t)stream);
     }
     return check_launch("volume_render_image_backward");
+}
+
+int svox_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                                      const SvoxRenderOptions* opt, const void* grad_output, void* grad_data_out,
+                                      int32_t accumulate, void* stream) {
+    return svox_volume_render_images_backward(tree, cam, 1, 12, opt, grad_output, grad_data_out, accumulate, stream);
 }
 
 int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCameraSpec* cam,
@@ -466,11 +482,11 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
         if (cam->width == 0 || cam->height == 0) return SVOX_OK;
         unsigned blocks;
         if (tree->dtype == SVOX_F32) {
-            const auto src = image_source<float>(cam, &blocks);
+            const auto src = image_source<float>(cam, 1, 12, &blocks);
             hipLaunchKernelGGL((render_stats_kernel<float, ImageSource<float>>), dim3(blocks), dim3(kMarchThreads), 0,
                                (hipStream_t)stream, make_tree<float>(tree), src, *opt, st);
         } else {
-            const auto src = image_source<double>(cam, &blocks);
+            const auto src = image_source<double>(cam, 1, 12, &blocks);
             hipLaunchKernelGGL((render_stats_kernel<double, ImageSource<double>>), dim3(blocks), dim3(kMarchThreads),
                                0, (hipStream_t)stream, make_tree<double>(tree), src, *opt, st);
         }

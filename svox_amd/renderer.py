@@ -67,6 +67,23 @@ class _VolumeRenderImageFunction(torch.autograd.Function):
         return grad, None, None, None
 
 
+class _VolumeRenderImagesFunction(torch.autograd.Function):
+    """Several poses in one launch (no counterpart in the reference)."""
+
+    @staticmethod
+    def forward(ctx, data, tree, cam, opt):
+        out = _C.volume_render_images(tree, cam, opt)
+        ctx.tree, ctx.cam, ctx.opt = tree, cam, opt
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        if not ctx.needs_input_grad[0]:
+            return None, None, None, None
+        grad = _C.volume_render_images_backward(ctx.tree, ctx.cam, ctx.opt, grad_out.contiguous())
+        return grad, None, None, None
+
+
 def convert_to_ndc(origins, directions, focal, w, h, near=1.0):
     """Rays in normalised device coordinates of a forward-facing scene (svox/renderer.py:92-112).
     The image kernels apply the same map themselves and then normalise the direction; ray batches
@@ -131,14 +148,17 @@ class VolumeRenderer(nn.Module):
 
     def render_persp(self, c2w, width=800, height=800, fx=1111.111, fy=None, cuda=True, fast=False):
         """Render a pinhole image -> (height, width, rgb_dim).  c2w is (3, 4) or (4, 4), OpenGL
-        convention (camera looks down -z, +y up); pixel (ix, iy) looks through its corner."""
+        convention (camera looks down -z, +y up); pixel (ix, iy) looks through its corner.
+
+        Beyond the reference: a stack of poses (n, 3, 4) or (n, 4, 4) renders n images in one
+        kernel launch and returns (n, height, width, rgb_dim)."""
         self._require_gpu(cuda, "VolumeRenderer.render_persp")
         if fy is None:
             fy = fx
         cam = _make_camera_spec(c2w.to(dtype=self.tree.data.dtype, device=self.tree.data.device).contiguous(),
                                 width, height, fx, fy)
-        return _VolumeRenderImageFunction.apply(self.tree.data, self.tree._spec(), cam,
-                                                self._get_options(fast))
+        fn = _VolumeRenderImagesFunction if c2w.dim() == 3 else _VolumeRenderImageFunction
+        return fn.apply(self.tree.data, self.tree._spec(), cam, self._get_options(fast))
 
     def se_grad(self, rays, colors):
         raise NotImplementedError("se_grad is not part of this build")

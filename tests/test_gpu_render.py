@@ -230,3 +230,26 @@ def test_render_persp_autograd_and_empty(gpu, oracle_mod):
     a = r(svox.Rays(rr.origins.to(gpu), rr.dirs.to(gpu), rr.viewdirs.to(gpu))).detach()
     b = r(svox.Rays(rr.origins[perm].to(gpu), rr.dirs[perm].to(gpu), rr.viewdirs[perm].to(gpu))).detach()
     assert torch.equal(a[perm.to(gpu)], b)
+
+
+def test_several_poses_in_one_launch_equal_separate_calls(gpu, oracle_mod):
+    tree = on_gpu(synth.shell_tree(depth=6, n_spheres=5, data_format="SH16", seed=41), gpu)
+    r = svox.VolumeRenderer(tree, step_size=1e-3)
+    poses = torch.stack(synth.orbit_poses(3, seed=2, radius=2.2)).to(gpu)          # (3, 3, 4)
+    W, H, fx = 61, 44, 70.0
+    batch = r.render_persp(poses, width=W, height=H, fx=fx, fast=True)
+    assert batch.shape == (3, H, W, 3)
+    singles = [r.render_persp(p, width=W, height=H, fx=fx, fast=True) for p in poses]
+    for i in range(3):
+        assert torch.equal(batch[i], singles[i])
+    # homogeneous (n, 4, 4) poses give the same pictures
+    hom = torch.cat([poses, torch.tensor([0.0, 0, 0, 1], device=gpu).expand(3, 1, 4)], dim=1).contiguous()
+    assert torch.equal(r.render_persp(hom, width=W, height=H, fx=fx, fast=True), batch)
+    go = torch.randn(3, H, W, 3, generator=torch.Generator().manual_seed(0)).to(gpu)
+    batch.backward(go)
+    g_batch = tree.data.grad.clone()
+    tree.data.grad = None
+    for i in range(3):
+        singles[i].backward(go[i])
+    err, ok = grad_close(g_batch.cpu().numpy(), tree.data.grad.cpu().numpy())
+    assert ok, err
