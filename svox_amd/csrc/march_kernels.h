@@ -527,34 +527,64 @@ __device__ void trace_backward_generic(const TreeDev<T>& tr, const SvoxRenderOpt
     }
 }
 
-// trace_ray_backward, octree flavour.  The first march only accumulates <render, grad_out>
-// (no memory writes); the second replays it and issues every atomic add: colour gradients with the
-// reference's per-sample values, then the density gradient.
+// value of `v` in lane `k` (k uniform across the wavefront)
+__device__ __forceinline__ float read_lane(float v, int k) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), k));
+}
+
+// trace_ray_backward, octree flavour, executed by a whole wavefront (every lane must call it;
+// `valid` is false for lanes without a ray).
+//
+// March 1 accumulates <render, grad_out> per lane and writes nothing.  March 2 replays the ray and
+// produces, per visited leaf with sigma > 0, the reference's gradient record: basis[i] * tmp2[c] for
+// the colour coefficients and the density term.  The records are not scattered lane by lane:
+// after every step the wavefront walks over the lanes that produced one, and for each such leaf
+// all 64 lanes add one element each of the K-long record with a single coalesced atomic
+// instruction (element e from lane e).  Lanes whose rays sit in the same leaf are summed first, so
+// that leaf receives one atomic per element instead of one per ray.  The per-term products are the
+// reference's; only the order in which they are added up differs.
+// `basis_lds` is a [64][kBasis] array private to the wavefront.
 template <class P>
 __device__ __forceinline__ void trace_backward_octree(const TreeDev<float>& tr, const SvoxRenderOptions& opt,
-                                                      const float* origin, const float* dir,
+                                                      bool valid, const float* origin, const float* dir,
                                                       const float* vdir, const float* scaling,
                                                       OctreeCursor& cur, const float* grad_out,
-                                                      float* __restrict__ grad_data) {
+                                                      float* __restrict__ grad_data, float* basis_lds) {
+    constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
+    constexpr int K = P::kRecord;
+    const int lane = threadIdx.x & 63;
     RayState<float> r;
-    if (!setup_ray(r, origin, dir, scaling)) return;
-    float basis[P::kBasis > 0 ? P::kBasis : 1];
-    if constexpr (P::kFormat == SVOX_FORMAT_SH) sh_basis<float>(P::kBasis, vdir, basis);
-    const float go[3] = {grad_out[0], grad_out[1], grad_out[2]};
+    bool live = valid && setup_ray(r, origin, dir, scaling);
+    float basis[D];
+    float go[3] = {0.f, 0.f, 0.f};
+    if (live) {
+        if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+            sh_basis<float>(P::kBasis, vdir, basis);
+#pragma unroll
+            for (int i = 0; i < D; ++i) basis_lds[lane * D + i] = basis[i];
+        }
+        go[0] = grad_out[0];
+        go[1] = grad_out[1];
+        go[2] = grad_out[2];
+    }
+    __syncthreads();  // one wavefront per block: makes every lane's basis visible to the others
     const float pad = opt.rgb_padding;
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     const float step = opt.step_size;
     const float tmin = r.t;
     float accum = 0.0f;
     int reads = 0;
-    {
+    if (live) {
         float light = 1.0f;
         while (r.t < r.tmax) {
             float delta_t;
             const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
-            if (v.leaf < 0) return;
-            const float* rec = tr.data + v.leaf * P::kRecord;
-            const float sigma = rec[P::kRecord - 1];
+            if (v.leaf < 0) {
+                live = false;
+                break;
+            }
+            const float* rec = tr.data + v.leaf * K;
+            const float sigma = rec[K - 1];
             if (sigma > 0.0f) {
                 const float att = expf_fixed(-delta_t * sigma * r.dscale);
                 const float weight = light * (1.0f - att);
@@ -571,40 +601,81 @@ __device__ __forceinline__ void trace_backward_octree(const TreeDev<float>& tr, 
         const float total_grad = (go[0] + go[1]) + go[2];
         accum = fma_(light * opt.background_brightness, total_grad, accum);
     }
-    {
-        float light = 1.0f;
-        r.t = tmin;
-        while (r.t < r.tmax) {
+    // march 2: the wavefront stays together
+    float light = 1.0f;
+    r.t = tmin;
+    while (true) {
+        const bool act = live && (r.t < r.tmax);
+        if (!__any(act)) break;
+        bool emit = false;
+        int32_t leaf = -1;
+        float tmp2[3] = {0.f, 0.f, 0.f};
+        float g_sigma = 0.f;
+        if (act) {
             float delta_t;
             const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
-            if (v.leaf < 0) return;
-            const int64_t base = v.leaf * P::kRecord;
-            const float* rec = tr.data + base;
-            const float sigma = rec[P::kRecord - 1];
-            if (sigma > 0.0f) {
-                const float att = expf_fixed(-delta_t * sigma * r.dscale);
-                const float weight = light * (1.0f - att);
-                float s[3];
-                leaf_colour<P>(rec, basis, s);
-                float total_color = 0.0f;
-                float* g = grad_data + base;
+            if (v.leaf < 0) {
+                live = false;
+            } else {
+                const float* rec = tr.data + v.leaf * K;
+                const float sigma = rec[K - 1];
+                if (sigma > 0.0f) {
+                    const float att = expf_fixed(-delta_t * sigma * r.dscale);
+                    const float weight = light * (1.0f - att);
+                    float s[3];
+                    leaf_colour<P>(rec, basis, s);
+                    float total_color = 0.0f;
 #pragma unroll
-                for (int c = 0; c < 3; ++c) {
-                    if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                        atomicAdd(g + c, weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad);
-                    } else {
-                        const float tmp2 = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) *
-                                                   (double)go[c] * (double)d_rgb_pad);
-#pragma unroll
-                        for (int i = 0; i < P::kBasis; ++i) atomicAdd(g + c * P::kBasis + i, basis[i] * tmp2);
+                    for (int c = 0; c < 3; ++c) {
+                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                            tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
+                        } else {
+                            tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)go[c] *
+                                              (double)d_rgb_pad);
+                        }
+                        total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
                     }
-                    total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+                    light *= att;
+                    accum = fma_(-weight, total_color, accum);
+                    g_sigma = delta_t * r.dscale * fma_(total_color, light, -accum);
+                    leaf = (int32_t)v.leaf;
+                    emit = true;
                 }
-                light *= att;
-                accum = fma_(-weight, total_color, accum);
-                atomicAdd(g + P::kRecord - 1, delta_t * r.dscale * fma_(total_color, light, -accum));
+                r.t += delta_t;
             }
-            r.t += delta_t;
+        }
+        unsigned long long todo = __ballot(emit);
+        while (todo) {
+            const int leader = __ffsll((long long)todo) - 1;
+            const int32_t leaf_l = __builtin_amdgcn_readlane(leaf, leader);
+            unsigned long long same = __ballot(emit && leaf == leaf_l);
+            todo &= ~same;
+            float* g = grad_data + (int64_t)leaf_l * K;
+#pragma unroll
+            for (int e0 = 0; e0 < K; e0 += 64) {
+                const int e = e0 + lane;
+                float val = 0.0f;
+                unsigned long long members = same;
+                while (members) {
+                    const int k = __ffsll((long long)members) - 1;
+                    members &= members - 1;
+                    const float t0 = read_lane(tmp2[0], k);
+                    const float t1 = read_lane(tmp2[1], k);
+                    const float t2 = read_lane(tmp2[2], k);
+                    const float gs = read_lane(g_sigma, k);
+                    float term;
+                    if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                        term = e == 0 ? t0 : e == 1 ? t1 : e == 2 ? t2 : gs;
+                    } else {
+                        const int c = e / D;
+                        const float b = e < 3 * D ? basis_lds[k * D + (e - c * D)] : 0.0f;
+                        const float tc = c == 0 ? t0 : c == 1 ? t1 : t2;
+                        term = e < 3 * D ? b * tc : gs;
+                    }
+                    val += term;
+                }
+                if (e < K) atomicAdd(g + e, val);
+            }
         }
     }
 }
@@ -619,12 +690,14 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(
     load_transform(tr, offset, scaling);
     T origin[3], dir[3], vdir[3];
     const int64_t slot = src.fetch(tr, opt, offset, scaling, origin, dir, vdir);
-    if (slot < 0) return;
     if constexpr (P::kOctree) {
+        __shared__ float basis_lds[kMarchThreads * (P::kBasis > 0 ? P::kBasis : 1)];
         OctreeCursor cur;
         cur.reset(path + threadIdx.x, kMarchThreads);
-        trace_backward_octree<P>(tr, opt, origin, dir, vdir, scaling, cur, grad_out + slot * 3, grad_data);
+        trace_backward_octree<P>(tr, opt, slot >= 0, origin, dir, vdir, scaling, cur,
+                                 grad_out + (slot >= 0 ? slot : 0) * 3, grad_data, basis_lds);
     } else {
+        if (slot < 0) return;
         trace_backward_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, grad_out + slot * out_dim,
                                   grad_data);
     }
