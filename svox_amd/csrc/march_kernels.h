@@ -17,7 +17,6 @@
 namespace svox {
 
 constexpr int kMarchThreads = 64;  // one wavefront per block: finished tiles free their slot at once
-constexpr int kTile = 8;           // image kernels: a block (wavefront) covers an 8x8 pixel tile
 
 // ------------------------------------------------------------------------------------------------
 // ray sources
@@ -93,55 +92,66 @@ __device__ __forceinline__ void maybe_world2ndc(const SvoxRenderOptions& opt, T*
     dir[2] /= n;
 }
 
-// Which ray a thread traces.  Batch: thread i takes ray i.  Image: each block (one wavefront) is
-// an 8x8 pixel tile, so its 64 rays stay close in the tree.  Several images of the same size can
-// share a launch; blocks are numbered image by image, so the dispatcher starts the next image's
-// tiles as the previous image's last tiles drain.
+// Ray sources.  The rays of a launch are numbered 0 .. total()-1 ("items"); a wavefront owns the
+// `per_wave` consecutive items starting at blockIdx.x * per_wave and feeds them to its 64 lanes.
+//   Batch: item i is ray i.
+//   Image: items are numbered so that 64 consecutive items are one 8x8 pixel tile and 256
+//          consecutive items one 16x16 block (four tiles), image after image: the rays a wavefront
+//          holds at any time stay close in the tree, and the dispatcher starts the next image's
+//          blocks as the previous image's last ones drain.  Items that fall outside the image
+//          (sizes that are not multiples of 16) have no ray.
+// fetch_item returns the output slot of the item (ray index / pixel index) or -1, and the ray in
+// tree coordinates.
 template <typename T>
 struct BatchSource {
     RayBatch<T> rays;
-    __device__ __forceinline__ int64_t count() const { return rays.n_rays; }
-    // returns the output slot (ray index) or -1
-    __device__ __forceinline__ int64_t fetch(const TreeDev<T>&, const SvoxRenderOptions&, const T* offset,
-                                             const T* scaling, T* origin, T* dir, T* vdir) const {
-        const int64_t r = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
-        if (r >= rays.n_rays) return -1;
+    int per_wave;
+    int refill_at;   // idle lanes that trigger taking new rays
+    __device__ __forceinline__ int64_t total() const { return rays.n_rays; }
+    __device__ __forceinline__ int64_t fetch_item(int64_t i, const SvoxRenderOptions&, const T* offset,
+                                                  const T* scaling, T* origin, T* dir, T* vdir) const {
+        if (i >= rays.n_rays) return -1;
 #pragma unroll
-        for (int i = 0; i < 3; ++i) {
-            origin[i] = rays.origins[r * 3 + i];
-            dir[i] = rays.dirs[r * 3 + i];
-            vdir[i] = rays.vdirs[r * 3 + i];
+        for (int k = 0; k < 3; ++k) {
+            origin[k] = rays.origins[i * 3 + k];
+            dir[k] = rays.dirs[i * 3 + k];
+            vdir[k] = rays.vdirs[i * 3 + k];
         }
         transform_coord(origin, offset, scaling);
-        return r;
+        return i;
     }
 };
 
-__host__ __device__ inline int tiles_of(int extent) { return (extent + kTile - 1) / kTile; }
+__host__ __device__ inline int blocks16_of(int extent) { return (extent + 15) / 16; }
 
 template <typename T>
 struct ImageSource {
     Camera<T> cam;          // cam.c2w: pose of image 0
     int n_images;
     int64_t pose_stride;    // scalars between consecutive poses
-    __device__ __forceinline__ int64_t count() const { return (int64_t)n_images * cam.width * cam.height; }
-    __device__ __forceinline__ int64_t fetch(const TreeDev<T>&, const SvoxRenderOptions& opt, const T* offset,
-                                             const T* scaling, T* origin, T* dir, T* vdir) const {
-        const int ntx = tiles_of(cam.width), nty = tiles_of(cam.height);
-        const int per_image = ntx * nty;
-        const int image = (int)(blockIdx.x / (unsigned)per_image);
-        const int tile = (int)(blockIdx.x - (unsigned)image * (unsigned)per_image);
+    int per_wave;           // 64 (one 8x8 tile) or 256 (one 16x16 block)
+    int refill_at;          // idle lanes that trigger taking new rays
+    __device__ __forceinline__ int64_t total() const {
+        return (int64_t)n_images * blocks16_of(cam.width) * blocks16_of(cam.height) * 256;
+    }
+    __device__ __forceinline__ int64_t fetch_item(int64_t i, const SvoxRenderOptions& opt, const T* offset,
+                                                  const T* scaling, T* origin, T* dir, T* vdir) const {
+        const int nbx = blocks16_of(cam.width), nby = blocks16_of(cam.height);
+        const int64_t block = i >> 8;
+        const int within = (int)(i & 255);
+        const int image = (int)(block / (nbx * nby));
         if (image >= n_images) return -1;
-        const int ty = tile / ntx, tx = tile - ty * ntx;
-        const int lane = threadIdx.x & 63;
-        const int ix = tx * kTile + (lane & 7);
-        const int iy = ty * kTile + (lane >> 3);
+        const int b = (int)(block - (int64_t)image * (nbx * nby));
+        const int by = b / nbx, bx = b - by * nbx;
+        const int sub = within >> 6, pos = within & 63;
+        const int ix = bx * 16 + (sub & 1) * 8 + (pos & 7);
+        const int iy = by * 16 + (sub >> 1) * 8 + (pos >> 3);
         if (ix >= cam.width || iy >= cam.height) return -1;
         Camera<T> c = cam;
         c.c2w = cam.c2w + (int64_t)image * pose_stride;
         cam2world_ray(ix, iy, c, dir, origin);
 #pragma unroll
-        for (int i = 0; i < 3; ++i) vdir[i] = dir[i];
+        for (int k = 0; k < 3; ++k) vdir[k] = dir[k];
         maybe_world2ndc(opt, dir, origin);
         transform_coord(origin, offset, scaling);
         return ((int64_t)image * cam.height + iy) * cam.width + ix;
@@ -333,96 +343,155 @@ __device__ void trace_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt
     for (int j = 0; j < out_dim; ++j) out[j] = acc[j];
 }
 
-// colour of one leaf record for the octree flavour: 3 sigmoids of basis . coefficients
-template <class P>
+// colour of one leaf record for the octree flavour: 3 sigmoids of basis . coefficients.
+// `basis` is read with stride `kStride` (1: a register array, 64: this lane's column of an LDS array
+// laid out [coefficient][lane], which 64 lanes read without bank conflicts).
+template <class P, int kStride>
 __device__ __forceinline__ void leaf_colour(const float* __restrict__ rec, const float* basis, float* s) {
     if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
 #pragma unroll
         for (int c = 0; c < 3; ++c) s[c] = sigmoid_(rec[c]);
     } else {
+        float b[P::kBasis];
+#pragma unroll
+        for (int i = 0; i < P::kBasis; ++i) b[i] = basis[i * kStride];
 #pragma unroll
         for (int c = 0; c < 3; ++c) {
             float tmp = 0.0f;
 #pragma unroll
-            for (int i = 0; i < P::kBasis; ++i) tmp = fma_(basis[i], rec[c * P::kBasis + i], tmp);
+            for (int i = 0; i < P::kBasis; ++i) tmp = fma_(b[i], rec[c * P::kBasis + i], tmp);
             s[c] = sigmoid_(tmp);
         }
     }
 }
 
-// trace_ray, octree flavour
-template <class P>
-__device__ __forceinline__ void trace_octree(const TreeDev<float>& tr, const SvoxRenderOptions& opt,
-                                             const float* origin, const float* dir, const float* vdir,
-                                             const float* scaling, OctreeCursor& cur, float* out) {
-    RayState<float> r;
-    const float bg = opt.background_brightness;
-    if (!setup_ray(r, origin, dir, scaling)) {
-        out[0] = bg;
-        out[1] = bg;
-        out[2] = bg;
-        return;
-    }
-    float basis[P::kBasis > 0 ? P::kBasis : 1];
-    if constexpr (P::kFormat == SVOX_FORMAT_SH) sh_basis<float>(P::kBasis, vdir, basis);
-    float acc[3] = {0.f, 0.f, 0.f};
-    float light = 1.0f;
-    const float pad = opt.rgb_padding;
-    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
-    const float step = opt.step_size, sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
-    bool stopped = false;
-    int reads = 0;
-    while (r.t < r.tmax) {
-        float delta_t;
-        const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
-        if (v.leaf < 0) break;
-        const float* rec = tr.data + v.leaf * P::kRecord;
-        const float sigma = rec[P::kRecord - 1];
-        if (sigma > sigma_thresh) {
-            const float att = expf_fixed(-delta_t * r.dscale * sigma);
-            const float weight = light * (1.0f - att);
-            float s[3];
-            leaf_colour<P>(rec, basis, s);
-#pragma unroll
-            for (int c = 0; c < 3; ++c) acc[c] = fma_(weight, fma_(s[c], d_rgb_pad, -pad), acc[c]);
-            light *= att;
-            if (light <= stop_thresh) {
-                const float scale = (float)(1.0 / (1.0 - (double)light));
-#pragma unroll
-                for (int c = 0; c < 3; ++c) acc[c] *= scale;
-                stopped = true;
-                break;
-            }
-        }
-        r.t += delta_t;
-    }
-    if (!stopped) {
-#pragma unroll
-        for (int c = 0; c < 3; ++c) acc[c] = fma_(light, bg, acc[c]);
-    }
-    out[0] = acc[0];
-    out[1] = acc[1];
-    out[2] = acc[2];
+// number of set bits of `mask` below this lane
+__device__ __forceinline__ int rank_in(unsigned long long mask) {
+    return (int)__builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
 }
 
-template <class P, class Source>
-__global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<typename P::scalar> tr,
-                                                                       Source src, SvoxRenderOptions opt,
-                                                                       int out_dim,
-                                                                       typename P::scalar* __restrict__ out) {
-    using T = typename P::scalar;
-    __shared__ int32_t path[P::kOctree ? kPathLevels * kMarchThreads : 1];
+// trace_ray for the generic policy: one ray per lane, no sharing of work between lanes
+template <typename T, class Source>
+__global__ __launch_bounds__(kMarchThreads) void render_forward_generic_kernel(TreeDev<T> tr, Source src,
+                                                                               SvoxRenderOptions opt, int out_dim,
+                                                                               T* __restrict__ out) {
     T offset[3], scaling[3];
     load_transform(tr, offset, scaling);
     T origin[3], dir[3], vdir[3];
-    const int64_t slot = src.fetch(tr, opt, offset, scaling, origin, dir, vdir);
+    const int64_t item = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
+    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
     if (slot < 0) return;
-    if constexpr (P::kOctree) {
-        OctreeCursor cur;
-        cur.reset(path + threadIdx.x, kMarchThreads);
-        trace_octree<P>(tr, opt, origin, dir, vdir, scaling, cur, out + slot * 3);
-    } else {
-        trace_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, out + slot * out_dim);
+    trace_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, out + slot * out_dim);
+}
+
+// trace_ray, octree flavour: a persistent wavefront.  Each lane marches one ray, one leaf per loop
+// iteration.  Rays differ wildly in length (most miss the tree or stop early, a few cross hundreds of
+// leaves), so a lane whose ray has ended does not wait for the longest ray of the wavefront: as soon
+// as `refill_at` lanes are idle (ballot), the idle lanes take the next rays of the wavefront's
+// range, ranked by their position among the idle lanes.
+template <class P, class Source>
+__global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<float> tr, Source src,
+                                                                       SvoxRenderOptions opt,
+                                                                       float* __restrict__ out) {
+    constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
+    constexpr int K = P::kRecord;
+    __shared__ int32_t path[kPathLevels * kMarchThreads];
+    __shared__ float basis_t[D * kMarchThreads];   // [coefficient][lane]
+    const int lane = threadIdx.x;
+    float offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    const float bg = opt.background_brightness;
+    const float pad = opt.rgb_padding;
+    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
+    const float step = opt.step_size, sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
+
+    int64_t next = blockIdx.x * (int64_t)src.per_wave;
+    const int64_t total = src.total();
+    const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
+
+    RayState<float> r;
+    float acc[3] = {0.f, 0.f, 0.f};
+    float light = 1.0f;
+    int64_t slot = -1;
+    bool active = false;
+    int reads = 0;
+    OctreeCursor cur;
+    cur.reset(path + lane, kMarchThreads);
+
+    while (true) {
+        const unsigned long long idle = __ballot(!active);
+        const int n_idle = __popcll(idle);
+        if (next < end && n_idle >= src.refill_at) {
+            if (!active) {
+                const int64_t item = next + rank_in(idle);
+                if (item < end) {
+                    float origin[3], dir[3], vdir[3];
+                    slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+                    if (slot >= 0) {
+                        if (setup_ray(r, origin, dir, scaling)) {
+                            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+                                float basis[D];
+                                sh_basis<float>(P::kBasis, vdir, basis);
+#pragma unroll
+                                for (int i = 0; i < D; ++i) basis_t[i * kMarchThreads + lane] = basis[i];
+                            }
+                            acc[0] = acc[1] = acc[2] = 0.0f;
+                            light = 1.0f;
+                            cur.levels = 0;
+                            active = true;
+                        } else {
+                            out[slot * 3] = bg;
+                            out[slot * 3 + 1] = bg;
+                            out[slot * 3 + 2] = bg;
+                        }
+                    }
+                }
+            }
+            next += n_idle;
+            continue;
+        }
+        if (n_idle == kMarchThreads) break;
+        if (active) {
+            bool finished = !(r.t < r.tmax);   // a ray that only touches the cube takes no sample
+            bool stopped = false;
+            if (!finished) {
+                float delta_t;
+                const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
+                if (v.leaf >= 0) {
+                    const float* rec = tr.data + v.leaf * K;
+                    const float sigma = rec[K - 1];
+                    if (sigma > sigma_thresh) {
+                        const float att = expf_fixed(-delta_t * r.dscale * sigma);
+                        const float weight = light * (1.0f - att);
+                        float s[3];
+                        leaf_colour<P, kMarchThreads>(rec, basis_t + lane, s);
+#pragma unroll
+                        for (int c = 0; c < 3; ++c) acc[c] = fma_(weight, fma_(s[c], d_rgb_pad, -pad), acc[c]);
+                        light *= att;
+                        if (light <= stop_thresh) {
+                            const float scale = (float)(1.0 / (1.0 - (double)light));
+#pragma unroll
+                            for (int c = 0; c < 3; ++c) acc[c] *= scale;
+                            stopped = true;
+                        }
+                    }
+                    r.t += delta_t;
+                    finished = stopped || !(r.t < r.tmax);
+                } else {
+                    finished = true;   // malformed tree
+                }
+            }
+            if (finished) {
+                if (!stopped) {
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) acc[c] = fma_(light, bg, acc[c]);
+                }
+                out[slot * 3] = acc[0];
+                out[slot * 3 + 1] = acc[1];
+                out[slot * 3 + 2] = acc[2];
+                active = false;
+            }
+        }
     }
 }
 
@@ -532,123 +601,160 @@ __device__ __forceinline__ float read_lane(float v, int k) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), k));
 }
 
-// trace_ray_backward, octree flavour, executed by a whole wavefront (every lane must call it;
-// `valid` is false for lanes without a ray).
+template <typename T, class Source>
+__global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
+    TreeDev<T> tr, Source src, SvoxRenderOptions opt, int out_dim, const T* __restrict__ grad_out,
+    T* __restrict__ grad_data) {
+    T offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    T origin[3], dir[3], vdir[3];
+    const int64_t item = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
+    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+    if (slot < 0) return;
+    trace_backward_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, grad_out + slot * out_dim, grad_data);
+}
+
+// trace_ray_backward, octree flavour: a persistent wavefront like the forward kernel.
 //
-// March 1 accumulates <render, grad_out> per lane and writes nothing.  March 2 replays the ray and
-// produces, per visited leaf with sigma > 0, the reference's gradient record: basis[i] * tmp2[c] for
-// the colour coefficients and the density term.  The records are not scattered lane by lane:
-// after every step the wavefront walks over the lanes that produced one, and for each such leaf
-// all 64 lanes add one element each of the K-long record with a single coalesced atomic
-// instruction (element e from lane e).  Lanes whose rays sit in the same leaf are summed first, so
-// that leaf receives one atomic per element instead of one per ray.  The per-term products are the
-// reference's; only the order in which they are added up differs.
-// `basis_lds` is a [64][kBasis] array private to the wavefront.
-template <class P>
-__device__ __forceinline__ void trace_backward_octree(const TreeDev<float>& tr, const SvoxRenderOptions& opt,
-                                                      bool valid, const float* origin, const float* dir,
-                                                      const float* vdir, const float* scaling,
-                                                      OctreeCursor& cur, const float* grad_out,
-                                                      float* __restrict__ grad_data, float* basis_lds) {
+// A lane runs its ray twice.  March 1 accumulates <render, grad_out> and writes nothing.  March 2
+// replays the ray and produces, per visited leaf with sigma > 0, the reference's gradient record:
+// basis[i] * tmp2[c] for the colour coefficients and the density term.  The records are not
+// scattered lane by lane: after every step the wavefront walks over the lanes that produced one,
+// and for each such leaf all lanes add one element each of the K-long record with a single
+// coalesced atomic instruction (element e from lane e).  Lanes whose rays sit in the same leaf are
+// summed first, so that leaf receives one atomic per element instead of one per ray.  The per-term
+// products are the reference's; only the order in which they are added up differs.
+template <class P, class Source>
+__global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<float> tr, Source src,
+                                                                        SvoxRenderOptions opt,
+                                                                        const float* __restrict__ grad_out,
+                                                                        float* __restrict__ grad_data) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
-    const int lane = threadIdx.x & 63;
-    RayState<float> r;
-    bool live = valid && setup_ray(r, origin, dir, scaling);
-    float basis[D];
-    float go[3] = {0.f, 0.f, 0.f};
-    if (live) {
-        if constexpr (P::kFormat == SVOX_FORMAT_SH) {
-            sh_basis<float>(P::kBasis, vdir, basis);
-#pragma unroll
-            for (int i = 0; i < D; ++i) basis_lds[lane * D + i] = basis[i];
-        }
-        go[0] = grad_out[0];
-        go[1] = grad_out[1];
-        go[2] = grad_out[2];
-    }
-    __syncthreads();  // one wavefront per block: makes every lane's basis visible to the others
+    __shared__ int32_t path[kPathLevels * kMarchThreads];
+    __shared__ float basis_lds[kMarchThreads * D];   // [lane][coefficient]: read across lanes when emitting
+    __shared__ float basis_t[D * kMarchThreads];     // [coefficient][lane]: read by the owning lane
+    const int lane = threadIdx.x;
+    float offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    const float bg = opt.background_brightness;
     const float pad = opt.rgb_padding;
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     const float step = opt.step_size;
-    const float tmin = r.t;
-    float accum = 0.0f;
+
+    int64_t next = blockIdx.x * (int64_t)src.per_wave;
+    const int64_t total = src.total();
+    const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
+
+    RayState<float> r;
+    float go[3] = {0.f, 0.f, 0.f};
+    float light = 1.0f, accum = 0.0f, tmin = 0.0f;
+    bool active = false, second = false;
     int reads = 0;
-    if (live) {
-        float light = 1.0f;
-        while (r.t < r.tmax) {
-            float delta_t;
-            const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
-            if (v.leaf < 0) {
-                live = false;
-                break;
-            }
-            const float* rec = tr.data + v.leaf * K;
-            const float sigma = rec[K - 1];
-            if (sigma > 0.0f) {
-                const float att = expf_fixed(-delta_t * sigma * r.dscale);
-                const float weight = light * (1.0f - att);
-                float s[3];
-                leaf_colour<P>(rec, basis, s);
-                float total_color = 0.0f;
-#pragma unroll
-                for (int c = 0; c < 3; ++c) total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
-                light *= att;
-                accum = fma_(weight, total_color, accum);
-            }
-            r.t += delta_t;
-        }
-        const float total_grad = (go[0] + go[1]) + go[2];
-        accum = fma_(light * opt.background_brightness, total_grad, accum);
-    }
-    // march 2: the wavefront stays together
-    float light = 1.0f;
-    r.t = tmin;
+    OctreeCursor cur;
+    cur.reset(path + lane, kMarchThreads);
+
     while (true) {
-        const bool act = live && (r.t < r.tmax);
-        if (!__any(act)) break;
+        const unsigned long long idle = __ballot(!active);
+        const int n_idle = __popcll(idle);
+        if (next < end && n_idle >= src.refill_at) {
+            if (!active) {
+                const int64_t item = next + rank_in(idle);
+                if (item < end) {
+                    float origin[3], dir[3], vdir[3];
+                    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+                    if (slot >= 0 && setup_ray(r, origin, dir, scaling)) {
+                        if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+                            float basis[D];
+                            sh_basis<float>(P::kBasis, vdir, basis);
+#pragma unroll
+                            for (int i = 0; i < D; ++i) {
+                                basis_lds[lane * D + i] = basis[i];
+                                basis_t[i * kMarchThreads + lane] = basis[i];
+                            }
+                        }
+                        go[0] = grad_out[slot * 3];
+                        go[1] = grad_out[slot * 3 + 1];
+                        go[2] = grad_out[slot * 3 + 2];
+                        light = 1.0f;
+                        accum = 0.0f;
+                        tmin = r.t;
+                        cur.levels = 0;
+                        second = false;
+                        active = true;
+                    }
+                }
+            }
+            next += n_idle;
+            __syncthreads();  // single-wavefront block: orders the LDS basis writes before later reads
+            continue;
+        }
+        if (n_idle == kMarchThreads) break;
+
         bool emit = false;
         int32_t leaf = -1;
         float tmp2[3] = {0.f, 0.f, 0.f};
         float g_sigma = 0.f;
-        if (act) {
-            float delta_t;
-            const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
-            if (v.leaf < 0) {
-                live = false;
-            } else {
-                const float* rec = tr.data + v.leaf * K;
-                const float sigma = rec[K - 1];
-                if (sigma > 0.0f) {
-                    const float att = expf_fixed(-delta_t * sigma * r.dscale);
-                    const float weight = light * (1.0f - att);
-                    float s[3];
-                    leaf_colour<P>(rec, basis, s);
-                    float total_color = 0.0f;
+        if (active) {
+            bool march_done = !(r.t < r.tmax);
+            if (!march_done) {
+                float delta_t;
+                const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
+                if (v.leaf >= 0) {
+                    const float* rec = tr.data + v.leaf * K;
+                    const float sigma = rec[K - 1];
+                    if (sigma > 0.0f) {
+                        const float att = expf_fixed(-delta_t * sigma * r.dscale);
+                        const float weight = light * (1.0f - att);
+                        float s[3];
+                        leaf_colour<P, kMarchThreads>(rec, basis_t + lane, s);
+                        float total_color = 0.0f;
 #pragma unroll
-                    for (int c = 0; c < 3; ++c) {
-                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                            tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
+                        for (int c = 0; c < 3; ++c)
+                            total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+                        light *= att;
+                        if (!second) {
+                            accum = fma_(weight, total_color, accum);
                         } else {
-                            tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)go[c] *
-                                              (double)d_rgb_pad);
+#pragma unroll
+                            for (int c = 0; c < 3; ++c) {
+                                if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                                    tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
+                                } else {
+                                    tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) *
+                                                      (double)go[c] * (double)d_rgb_pad);
+                                }
+                            }
+                            accum = fma_(-weight, total_color, accum);
+                            g_sigma = delta_t * r.dscale * fma_(total_color, light, -accum);
+                            leaf = (int32_t)v.leaf;
+                            emit = true;
                         }
-                        total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
                     }
-                    light *= att;
-                    accum = fma_(-weight, total_color, accum);
-                    g_sigma = delta_t * r.dscale * fma_(total_color, light, -accum);
-                    leaf = (int32_t)v.leaf;
-                    emit = true;
+                    r.t += delta_t;
+                    march_done = !(r.t < r.tmax);
+                } else {
+                    march_done = true;
+                    second = true;   // malformed tree: give the ray up
                 }
-                r.t += delta_t;
+            }
+            if (march_done) {
+                if (!second) {
+                    const float total_grad = (go[0] + go[1]) + go[2];
+                    accum = fma_(light * bg, total_grad, accum);
+                    light = 1.0f;
+                    r.t = tmin;
+                    second = true;
+                } else {
+                    active = false;
+                }
             }
         }
         unsigned long long todo = __ballot(emit);
         while (todo) {
             const int leader = __ffsll((long long)todo) - 1;
             const int32_t leaf_l = __builtin_amdgcn_readlane(leaf, leader);
-            unsigned long long same = __ballot(emit && leaf == leaf_l);
+            const unsigned long long same = __ballot(emit && leaf == leaf_l);
             todo &= ~same;
             float* g = grad_data + (int64_t)leaf_l * K;
 #pragma unroll
@@ -680,29 +786,6 @@ __device__ __forceinline__ void trace_backward_octree(const TreeDev<float>& tr, 
     }
 }
 
-template <class P, class Source>
-__global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(
-    TreeDev<typename P::scalar> tr, Source src, SvoxRenderOptions opt, int out_dim,
-    const typename P::scalar* __restrict__ grad_out, typename P::scalar* __restrict__ grad_data) {
-    using T = typename P::scalar;
-    __shared__ int32_t path[P::kOctree ? kPathLevels * kMarchThreads : 1];
-    T offset[3], scaling[3];
-    load_transform(tr, offset, scaling);
-    T origin[3], dir[3], vdir[3];
-    const int64_t slot = src.fetch(tr, opt, offset, scaling, origin, dir, vdir);
-    if constexpr (P::kOctree) {
-        __shared__ float basis_lds[kMarchThreads * (P::kBasis > 0 ? P::kBasis : 1)];
-        OctreeCursor cur;
-        cur.reset(path + threadIdx.x, kMarchThreads);
-        trace_backward_octree<P>(tr, opt, slot >= 0, origin, dir, vdir, scaling, cur,
-                                 grad_out + (slot >= 0 ? slot : 0) * 3, grad_data, basis_lds);
-    } else {
-        if (slot < 0) return;
-        trace_backward_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, grad_out + slot * out_dim,
-                                  grad_data);
-    }
-}
-
 // ------------------------------------------------------------------------------------------------
 // visit counters
 // ------------------------------------------------------------------------------------------------
@@ -725,7 +808,8 @@ __global__ __launch_bounds__(kMarchThreads) void render_stats_kernel(TreeDev<T> 
     T offset[3], scaling[3];
     load_transform(tr, offset, scaling);
     T origin[3], dir[3], vdir[3];
-    const int64_t slot = src.fetch(tr, opt, offset, scaling, origin, dir, vdir);
+    const int64_t slot = src.fetch_item(blockIdx.x * (int64_t)kMarchThreads + threadIdx.x, opt, offset, scaling,
+                                        origin, dir, vdir);
     unsigned long long c_rays = 0, c_hit = 0, c_samples = 0, c_shaded = 0, c_bwd = 0, c_bwd_pos = 0, c_levels = 0;
     if (slot >= 0) {
         c_rays = 1;

@@ -6,6 +6,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "../../include/svox_hip.h"
@@ -150,7 +151,7 @@ int check_camera(const SvoxCameraSpec* cam, int n_images = 1, int64_t pose_strid
     if (cam->width < 0 || cam->height < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative image size");
     if (n_images < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative image count");
     if (n_images > 1 && pose_stride < 12) return fail(SVOX_ERR_BAD_SHAPE, "pose_stride must be >= 12 scalars");
-    const double tiles = (double)tiles_of(cam->width) * tiles_of(cam->height) * (n_images > 0 ? n_images : 1);
+    const double tiles = 4.0 * blocks16_of(cam->width) * blocks16_of(cam->height) * (n_images > 0 ? n_images : 1);
     if (tiles >= 2147483647.0) return fail(SVOX_ERR_BAD_SHAPE, "too many pixels for one launch");
     return SVOX_OK;
 }
@@ -174,6 +175,26 @@ int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
     return D;
 }
 
+// Items (rays) a persistent wavefront owns.  With few rays every wavefront gets one 64-item chunk so
+// that the launch spreads over as many SIMDs as possible; with many, 256 items, which lets lanes whose
+// rays end early pick up new ones.
+int pick_per_wave(int64_t total_items) {
+    static const int forced = [] {
+        const char* e = getenv("SVOX_PER_WAVE");
+        return e ? atoi(e) : 0;
+    }();
+    if (forced == 64 || forced == 256 || forced == 512 || forced == 1024) return forced;
+    return total_items >= (int64_t)64 * 1024 * 8 ? 512 : 64;
+}
+
+int pick_refill() {
+    static const int forced = [] {
+        const char* e = getenv("SVOX_REFILL");
+        return e ? atoi(e) : 0;
+    }();
+    return forced >= 1 && forced <= 64 ? forced : 16;
+}
+
 template <typename T>
 BatchSource<T> batch_source(const SvoxRaysSpec* rays) {
     BatchSource<T> s;
@@ -181,11 +202,13 @@ BatchSource<T> batch_source(const SvoxRaysSpec* rays) {
     s.rays.dirs = (const T*)rays->dirs;
     s.rays.vdirs = (const T*)rays->vdirs;
     s.rays.n_rays = rays->n_rays;
+    s.per_wave = pick_per_wave(rays->n_rays);
+    s.refill_at = pick_refill();
     return s;
 }
 
 template <typename T>
-ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pose_stride, unsigned* blocks) {
+ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pose_stride) {
     ImageSource<T> s;
     s.cam.c2w = (const T*)cam->c2w;
     s.cam.fx = cam->fx;
@@ -194,9 +217,23 @@ ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pos
     s.cam.height = cam->height;
     s.n_images = n_images;
     s.pose_stride = pose_stride;
-    *blocks = (unsigned)(tiles_of(cam->width) * tiles_of(cam->height)) * (unsigned)n_images;
+    const int64_t total = (int64_t)n_images * blocks16_of(cam->width) * blocks16_of(cam->height) * 256;
+    // image tiles are coherent (rays of a tile end together) and only part of an image hits the
+    // tree: one tile per wavefront keeps the busy tiles spread over the whole GPU
+    const int pw = pick_per_wave(0);
+    s.per_wave = pw > 256 ? 256 : pw;
+    s.refill_at = pick_refill();
     return s;
 }
+
+template <typename T>
+int64_t total_items_of(const BatchSource<T>& s) { return s.rays.n_rays; }
+template <typename T>
+int64_t total_items_of(const ImageSource<T>& s) {
+    return (int64_t)s.n_images * blocks16_of(s.cam.width) * blocks16_of(s.cam.height) * 256;
+}
+
+unsigned blocks_for(int64_t items, int per_block) { return (unsigned)((items + per_block - 1) / per_block); }
 
 #define SVOX_DISPATCH_OCTREE(D, ...)                                         \
     switch (D) {                                                             \
@@ -209,39 +246,41 @@ ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pos
     }
 
 template <class Source, typename T>
-void launch_forward(const SvoxTreeSpec* tree, const Source& src, unsigned blocks, const SvoxRenderOptions* opt,
-                    int out_dim, void* out, hipStream_t stream) {
+void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, int out_dim,
+                    void* out, hipStream_t stream) {
+    const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
+            const unsigned blocks = blocks_for(items, src.per_wave);
             SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source>), dim3(blocks),
                                                        dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                       src, *opt, out_dim, (float*)out));
+                                                       src, *opt, (float*)out));
             return;
         }
     }
-    hipLaunchKernelGGL((render_forward_kernel<GenericPolicy<T>, Source>), dim3(blocks), dim3(kMarchThreads), 0,
-                       stream, make_tree<T>(tree), src, *opt, out_dim, (T*)out);
+    hipLaunchKernelGGL((render_forward_generic_kernel<T, Source>), dim3(blocks_for(items, kMarchThreads)),
+                       dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (T*)out);
 }
 
 template <class Source, typename T>
-void launch_backward(const SvoxTreeSpec* tree, const Source& src, unsigned blocks, const SvoxRenderOptions* opt,
-                     int out_dim, const void* grad_out, void* grad_data, hipStream_t stream) {
+void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, int out_dim,
+                     const void* grad_out, void* grad_data, hipStream_t stream) {
+    const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
+            const unsigned blocks = blocks_for(items, src.per_wave);
             SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source>), dim3(blocks),
                                                        dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                       src, *opt, out_dim, (const float*)grad_out,
-                                                       (float*)grad_data));
+                                                       src, *opt, (const float*)grad_out, (float*)grad_data));
             return;
         }
     }
-    hipLaunchKernelGGL((render_backward_kernel<GenericPolicy<T>, Source>), dim3(blocks), dim3(kMarchThreads), 0,
-                       stream, make_tree<T>(tree), src, *opt, out_dim, (const T*)grad_out, (T*)grad_data);
+    hipLaunchKernelGGL((render_backward_generic_kernel<T, Source>), dim3(blocks_for(items, kMarchThreads)),
+                       dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (const T*)grad_out,
+                       (T*)grad_data);
 }
-
-unsigned batch_blocks(int64_t n) { return (unsigned)((n + kMarchThreads - 1) / kMarchThreads); }
 
 int64_t data_bytes(const SvoxTreeSpec* t) {
     const int64_t esz = t->dtype == SVOX_F32 ? 4 : 8;
@@ -362,12 +401,11 @@ int svox_volume_render(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const
     if (rc) return rc;
     if (rays->n_rays == 0) return SVOX_OK;
     if (!out) return fail(SVOX_ERR_NULL_POINTER, "out is NULL");
-    const unsigned blocks = batch_blocks(rays->n_rays);
     if (tree->dtype == SVOX_F32)
-        launch_forward<BatchSource<float>, float>(tree, batch_source<float>(rays), blocks, opt, od, out,
+        launch_forward<BatchSource<float>, float>(tree, batch_source<float>(rays), opt, od, out,
                                                   (hipStream_t)stream);
     else
-        launch_forward<BatchSource<double>, double>(tree, batch_source<double>(rays), blocks, opt, od, out,
+        launch_forward<BatchSource<double>, double>(tree, batch_source<double>(rays), opt, od, out,
                                                     (hipStream_t)stream);
     return check_launch("volume_render");
 }
@@ -381,13 +419,12 @@ int svox_volume_render_images(const SvoxTreeSpec* tree, const SvoxCameraSpec* ca
     if (rc) return rc;
     if (cam->width == 0 || cam->height == 0 || n_images == 0) return SVOX_OK;
     if (!out) return fail(SVOX_ERR_NULL_POINTER, "out is NULL");
-    unsigned blocks;
     if (tree->dtype == SVOX_F32) {
-        const auto src = image_source<float>(cam, n_images, pose_stride, &blocks);
-        launch_forward<ImageSource<float>, float>(tree, src, blocks, opt, od, out, (hipStream_t)stream);
+        const auto src = image_source<float>(cam, n_images, pose_stride);
+        launch_forward<ImageSource<float>, float>(tree, src, opt, od, out, (hipStream_t)stream);
     } else {
-        const auto src = image_source<double>(cam, n_images, pose_stride, &blocks);
-        launch_forward<ImageSource<double>, double>(tree, src, blocks, opt, od, out, (hipStream_t)stream);
+        const auto src = image_source<double>(cam, n_images, pose_stride);
+        launch_forward<ImageSource<double>, double>(tree, src, opt, od, out, (hipStream_t)stream);
     }
     return check_launch("volume_render_image");
 }
@@ -411,13 +448,12 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
     }
     if (rays->n_rays == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
-    const unsigned blocks = batch_blocks(rays->n_rays);
     if (tree->dtype == SVOX_F32)
-        launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays), blocks, opt, od, grad_output,
+        launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays), opt, od, grad_output,
                                                    grad_data_out, (hipStream_t)stream);
     else
-        launch_backward<BatchSource<double>, double>(tree, batch_source<double>(rays), blocks, opt, od,
-                                                     grad_output, grad_data_out, (hipStream_t)stream);
+        launch_backward<BatchSource<double>, double>(tree, batch_source<double>(rays), opt, od, grad_output,
+                                                     grad_data_out, (hipStream_t)stream);
     return check_launch("volume_render_backward");
 }
 
@@ -437,14 +473,13 @@ int svox_volume_render_images_backward(const SvoxTreeSpec* tree, const SvoxCamer
     }
     if (cam->width == 0 || cam->height == 0 || n_images == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
-    unsigned blocks;
     if (tree->dtype == SVOX_F32) {
-        const auto src = image_source<float>(cam, n_images, pose_stride, &blocks);
-        launch_backward<ImageSource<float>, float>(tree, src, blocks, opt, od, grad_output, grad_data_out,
+        const auto src = image_source<float>(cam, n_images, pose_stride);
+        launch_backward<ImageSource<float>, float>(tree, src, opt, od, grad_output, grad_data_out,
                                                    (hipStream_t)stream);
     } else {
-        const auto src = image_source<double>(cam, n_images, pose_stride, &blocks);
-        launch_backward<ImageSource<double>, double>(tree, src, blocks, opt, od, grad_output, grad_data_out,
+        const auto src = image_source<double>(cam, n_images, pose_stride);
+        launch_backward<ImageSource<double>, double>(tree, src, opt, od, grad_output, grad_data_out,
                                                      (hipStream_t)stream);
     }
     return check_launch("volume_render_image_backward");
@@ -469,7 +504,7 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
         rc = check_rays(rays);
         if (rc) return rc;
         if (rays->n_rays == 0) return SVOX_OK;
-        const unsigned blocks = batch_blocks(rays->n_rays);
+        const unsigned blocks = blocks_for(rays->n_rays, kMarchThreads);
         if (tree->dtype == SVOX_F32)
             hipLaunchKernelGGL((render_stats_kernel<float, BatchSource<float>>), dim3(blocks), dim3(kMarchThreads), 0,
                                (hipStream_t)stream, make_tree<float>(tree), batch_source<float>(rays), *opt, st);
@@ -480,13 +515,14 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
         rc = check_camera(cam);
         if (rc) return rc;
         if (cam->width == 0 || cam->height == 0) return SVOX_OK;
-        unsigned blocks;
         if (tree->dtype == SVOX_F32) {
-            const auto src = image_source<float>(cam, 1, 12, &blocks);
+            const auto src = image_source<float>(cam, 1, 12);
+            const unsigned blocks = blocks_for(total_items_of(src), kMarchThreads);
             hipLaunchKernelGGL((render_stats_kernel<float, ImageSource<float>>), dim3(blocks), dim3(kMarchThreads), 0,
                                (hipStream_t)stream, make_tree<float>(tree), src, *opt, st);
         } else {
-            const auto src = image_source<double>(cam, 1, 12, &blocks);
+            const auto src = image_source<double>(cam, 1, 12);
+            const unsigned blocks = blocks_for(total_items_of(src), kMarchThreads);
             hipLaunchKernelGGL((render_stats_kernel<double, ImageSource<double>>), dim3(blocks), dim3(kMarchThreads),
                                0, (hipStream_t)stream, make_tree<double>(tree), src, *opt, st);
         }
