@@ -384,11 +384,65 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_generic_kernel(T
     trace_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, out + slot * out_dim);
 }
 
-// trace_ray, octree flavour: a persistent wavefront.  Each lane marches one ray, one leaf per loop
-// iteration.  Rays differ wildly in length (most miss the tree or stop early, a few cross hundreds of
-// leaves), so a lane whose ray has ended does not wait for the longest ray of the wavefront: as soon
-// as `refill_at` lanes are idle (ballot), the idle lanes take the next rays of the wavefront's
-// range, ranked by their position among the idle lanes.
+constexpr int kQueue = 4;  // leaves a lane walks ahead before the wavefront shades them
+
+// Shade list shared by the wavefront: the (lane, slot) pairs of one round whose leaf has to be
+// shaded, compacted so that consecutive lanes can take consecutive entries.
+template <int D>
+struct ShadeShared {
+    int32_t leaf[kQueue * kMarchThreads];       // leaf cell index of entry e
+    int32_t who[kQueue * kMarchThreads];        // owner lane | slot << 8
+    float colour[kQueue * kMarchThreads * 3];   // [slot][lane][channel]: sigmoid(basis . coefficients)
+    float basis[kMarchThreads * D];             // [lane][coefficient]
+};
+
+// Colours of all list entries, computed by the whole wavefront: item p = 3 * entry + channel goes to
+// lane p mod 64.  One item is the reference's dot product for one channel, evaluated in the
+// reference's order (coefficient 0 first) from 16-byte loads of the leaf record and of the owner
+// lane's basis row, followed by the sigmoid.
+template <class P>
+__device__ __forceinline__ void shade_entries(const float* __restrict__ data, ShadeShared<(P::kBasis > 0 ? P::kBasis : 1)>& sh,
+                                              int n_entries, int lane) {
+    constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
+    constexpr int K = P::kRecord;
+    const int n_items = n_entries * 3;
+    for (int p = lane; p < n_items; p += kMarchThreads) {
+        const int e = p / 3, c = p - 3 * e;
+        const int32_t leaf = sh.leaf[e];
+        const int who = sh.who[e];
+        const int owner = who & 255, slot = who >> 8;
+        const float* rec = data + (int64_t)leaf * K;
+        float s;
+        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+            s = sigmoid_(rec[c]);
+        } else {
+            const float* co = rec + c * D;
+            const float* b = sh.basis + owner * D;
+            float tmp = 0.0f;
+#pragma unroll
+            for (int i = 0; i < D; ++i) tmp = fma_(b[i], co[i], tmp);
+            s = sigmoid_(tmp);
+        }
+        sh.colour[(slot * kMarchThreads + owner) * 3 + c] = s;
+    }
+}
+
+// trace_ray, octree flavour: a persistent wavefront working in rounds.
+//
+//   refill    lanes whose ray has ended take the next rays of the wavefront's range (ranked by
+//             ballot among the idle lanes) once `refill_at` lanes are idle: rays differ wildly in
+//             length, and a finished lane does not wait for the longest ray of the wavefront;
+//   walk      every live lane advances its ray by up to kQueue leaves and remembers (leaf, step
+//             length) of each: the next position depends only on the tree, not on the leaf's
+//             contents, so this phase waits for child-table reads only;
+//   sigma     the densities of the remembered leaves are fetched together (kQueue loads in flight);
+//   shade     the leaves with sigma > sigma_thresh of all lanes form one list, and the wavefront
+//             evaluates their colours together (shade_entries), all 64 lanes busy whatever the
+//             number of rays that hit something;
+//   composite every lane folds its leaves, in order, into its colour and transmittance, stops at
+//             stop_thresh and writes the pixel when the ray ends.
+// A ray that stops early has walked at most kQueue - 1 leaves too far; the values are the same as
+// when every leaf is shaded on the spot.
 template <class P, class Source>
 __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<float> tr, Source src,
                                                                        SvoxRenderOptions opt,
@@ -396,7 +450,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[kPathLevels * kMarchThreads];
-    __shared__ float basis_t[D * kMarchThreads];   // [coefficient][lane]
+    __shared__ ShadeShared<D> sh;
     const int lane = threadIdx.x;
     float offset[3], scaling[3];
     load_transform(tr, offset, scaling);
@@ -419,6 +473,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     cur.reset(path + lane, kMarchThreads);
 
     while (true) {
+        // ---- refill
         const unsigned long long idle = __ballot(!active);
         const int n_idle = __popcll(idle);
         if (next < end && n_idle >= src.refill_at) {
@@ -433,7 +488,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                                 float basis[D];
                                 sh_basis<float>(P::kBasis, vdir, basis);
 #pragma unroll
-                                for (int i = 0; i < D; ++i) basis_t[i * kMarchThreads + lane] = basis[i];
+                                for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
                             }
                             acc[0] = acc[1] = acc[2] = 0.0f;
                             light = 1.0f;
@@ -451,37 +506,71 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
             continue;
         }
         if (n_idle == kMarchThreads) break;
-        if (active) {
-            bool finished = !(r.t < r.tmax);   // a ray that only touches the cube takes no sample
-            bool stopped = false;
-            if (!finished) {
+
+        // ---- walk
+        int32_t q_leaf[kQueue];
+        float q_dt[kQueue];
+        int n = 0;
+        bool broken = false;
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            q_leaf[q] = 0;
+            q_dt[q] = 0.0f;
+            if (active && !broken && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
-                    const float* rec = tr.data + v.leaf * K;
-                    const float sigma = rec[K - 1];
-                    if (sigma > sigma_thresh) {
-                        const float att = expf_fixed(-delta_t * r.dscale * sigma);
-                        const float weight = light * (1.0f - att);
-                        float s[3];
-                        leaf_colour<P, kMarchThreads>(rec, basis_t + lane, s);
-#pragma unroll
-                        for (int c = 0; c < 3; ++c) acc[c] = fma_(weight, fma_(s[c], d_rgb_pad, -pad), acc[c]);
-                        light *= att;
-                        if (light <= stop_thresh) {
-                            const float scale = (float)(1.0 / (1.0 - (double)light));
-#pragma unroll
-                            for (int c = 0; c < 3; ++c) acc[c] *= scale;
-                            stopped = true;
-                        }
-                    }
+                    q_leaf[q] = (int32_t)v.leaf;
+                    q_dt[q] = delta_t;
                     r.t += delta_t;
-                    finished = stopped || !(r.t < r.tmax);
+                    n = q + 1;
                 } else {
-                    finished = true;   // malformed tree
+                    broken = true;   // malformed tree: the ray ends here
                 }
             }
-            if (finished) {
+        }
+        // ---- sigma
+        float q_sigma[kQueue];
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q)
+            q_sigma[q] = q < n ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+        // ---- shade list
+        int n_entries = 0;
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            const bool want = q < n && q_sigma[q] > sigma_thresh;
+            const unsigned long long m = __ballot(want);
+            if (want) {
+                const int e = n_entries + rank_in(m);
+                sh.leaf[e] = q_leaf[q];
+                sh.who[e] = lane | (q << 8);
+            }
+            n_entries += __popcll(m);
+        }
+        __syncthreads();   // one wavefront per block: list and basis rows are visible to every lane
+        shade_entries<P>(tr.data, sh, n_entries, lane);
+        __syncthreads();
+        // ---- composite
+        if (active) {
+            bool stopped = false;
+#pragma unroll
+            for (int q = 0; q < kQueue; ++q) {
+                if (q < n && !stopped && q_sigma[q] > sigma_thresh) {
+                    const float att = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
+                    const float weight = light * (1.0f - att);
+                    const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) acc[c] = fma_(weight, fma_(s[c], d_rgb_pad, -pad), acc[c]);
+                    light *= att;
+                    if (light <= stop_thresh) {
+                        const float scale = (float)(1.0 / (1.0 - (double)light));
+#pragma unroll
+                        for (int c = 0; c < 3; ++c) acc[c] *= scale;
+                        stopped = true;
+                    }
+                }
+            }
+            if (stopped || broken || !(r.t < r.tmax)) {
                 if (!stopped) {
 #pragma unroll
                     for (int c = 0; c < 3; ++c) acc[c] = fma_(light, bg, acc[c]);
