@@ -54,6 +54,7 @@ def main():
     ap.add_argument("--train-rays", type=int, default=1 << 20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-bwd", action="store_true", help="skip the forward+backward leg")
+    ap.add_argument("--no-query", action="store_true", help="skip the point-query leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (rays would shard "
@@ -222,6 +223,50 @@ def main():
         tree.data.grad = None
         log(f"[bench] fwd+bwd {fwd_bwd}")
 
+    # ---------------------------------------------------------------- point queries (configs[1])
+    query = None
+    if not args.no_query:
+        qtree = synth.dense_tree(6, "SH9", seed=0, sigma="lognormal", coeff_std=0.5, zero_fraction=0.5).to(dev)
+        Q = 1 << 22
+        pts = torch.rand(Q, 3, generator=torch.Generator().manual_seed(3)).to(dev)
+        Kq, Lq = qtree.data_dim, 7
+
+        def ev_time(fn, n=5):
+            fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(n):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / n
+
+        qspec = qtree._spec()
+        with torch.no_grad():
+            q_ms = ev_time(lambda: C.query_vertical(qspec, pts))
+        go = torch.randn(Q, Kq, device=dev)
+        qb_ms = ev_time(lambda: C.query_vertical_backward(qspec, pts, go))
+        leaves = qtree._all_leaves().to(dev)
+        c_ms = ev_time(lambda: C.calc_corners(qspec, leaves))
+        q_bytes = Q * (12 + 4 * Lq + 4 * Kq + 4 * Kq + 8)
+        qb_bytes = Q * (12 + 4 * Lq + 4 * Kq + 8 * Kq) + qtree.data.numel() * 4
+        c_bytes = leaves.shape[0] * (32 + 12 + 8 * (Lq - 1))
+        query = {
+            "workload": "dense 128^3 SH9 tree (268 MB), 4M uniform points",
+            "query_vertical": {"mpoints_s": round(Q / q_ms / 1e3, 1), "ms": round(q_ms, 4),
+                               "algorithmic_gbs": round(q_bytes / q_ms / 1e6, 1),
+                               "frac_of_peak": round(q_bytes / q_ms / 1e6 / PEAK_HBM_GBS, 4)},
+            "query_vertical_backward": {"mpoints_s": round(Q / qb_ms / 1e3, 1), "ms": round(qb_ms, 4),
+                                        "algorithmic_gbs": round(qb_bytes / qb_ms / 1e6, 1),
+                                        "frac_of_peak": round(qb_bytes / qb_ms / 1e6 / PEAK_HBM_GBS, 4),
+                                        "includes": "zero-fill of the (M,2,2,2,28) gradient"},
+            "calc_corners": {"mleaves_s": round(leaves.shape[0] / c_ms / 1e3, 1), "ms": round(c_ms, 4),
+                             "algorithmic_gbs": round(c_bytes / c_ms / 1e6, 1)},
+        }
+        del qtree, pts, go, leaves
+        log(f"[bench] query {query}")
+
     # ---------------------------------------------------------------- CPU baseline (this host)
     cpu = None
     if not args.no_cpu:
@@ -277,6 +322,7 @@ def main():
         "roofline": roofline,
         "fwd_per_call": per_call,
         "fwd_bwd": fwd_bwd,
+        "query": query,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)

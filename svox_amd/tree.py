@@ -502,7 +502,7 @@ class N3Tree(nn.Module):
     def _all_leaves(self):
         """(n_leaves, 4) int64 [node, x, y, z] of every leaf cell, lexicographic, on the CPU."""
         if self._last_all_leaves is None:
-            self._last_all_leaves = (self.child[:self.n_internal] == 0).nonzero(as_tuple=False).cpu()
+            self._last_all_leaves = (self.child[:self.n_internal] == 0).nonzero(as_tuple=False).cpu().contiguous()
         return self._last_all_leaves
 
     def world2tree(self, indices):
