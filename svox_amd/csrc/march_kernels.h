@@ -703,16 +703,18 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
     trace_backward_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, grad_out + slot * out_dim, grad_data);
 }
 
-// trace_ray_backward, octree flavour: a persistent wavefront like the forward kernel.
+// trace_ray_backward, octree flavour: a persistent wavefront working in the forward kernel's rounds
+// (refill, walk, sigma, shade, composite).
 //
 // A lane runs its ray twice.  March 1 accumulates <render, grad_out> and writes nothing.  March 2
 // replays the ray and produces, per visited leaf with sigma > 0, the reference's gradient record:
 // basis[i] * tmp2[c] for the colour coefficients and the density term.  The records are not
-// scattered lane by lane: after every step the wavefront walks over the lanes that produced one,
-// and for each such leaf all lanes add one element each of the K-long record with a single
+// scattered lane by lane: for every queue slot the wavefront walks over the lanes that produced a
+// record, and for each such leaf all lanes add one element each of the K-long record with a single
 // coalesced atomic instruction (element e from lane e).  Lanes whose rays sit in the same leaf are
 // summed first, so that leaf receives one atomic per element instead of one per ray.  The per-term
 // products are the reference's; only the order in which they are added up differs.
+// Both marches test sigma > 0 and never stop early (rt_kernel.cu:377, 441).
 template <class P, class Source>
 __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<float> tr, Source src,
                                                                         SvoxRenderOptions opt,
@@ -721,8 +723,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[kPathLevels * kMarchThreads];
-    __shared__ float basis_lds[kMarchThreads * D];   // [lane][coefficient]: read across lanes when emitting
-    __shared__ float basis_t[D * kMarchThreads];     // [coefficient][lane]: read by the owning lane
+    __shared__ ShadeShared<D> sh;
     const int lane = threadIdx.x;
     float offset[3], scaling[3];
     load_transform(tr, offset, scaling);
@@ -744,6 +745,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     cur.reset(path + lane, kMarchThreads);
 
     while (true) {
+        // ---- refill
         const unsigned long long idle = __ballot(!active);
         const int n_idle = __popcll(idle);
         if (next < end && n_idle >= src.refill_at) {
@@ -757,10 +759,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                             float basis[D];
                             sh_basis<float>(P::kBasis, vdir, basis);
 #pragma unroll
-                            for (int i = 0; i < D; ++i) {
-                                basis_lds[lane * D + i] = basis[i];
-                                basis_t[i * kMarchThreads + lane] = basis[i];
-                            }
+                            for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
                         }
                         go[0] = grad_out[slot * 3];
                         go[1] = grad_out[slot * 3 + 1];
@@ -775,101 +774,128 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                 }
             }
             next += n_idle;
-            __syncthreads();  // single-wavefront block: orders the LDS basis writes before later reads
             continue;
         }
         if (n_idle == kMarchThreads) break;
 
-        bool emit = false;
-        int32_t leaf = -1;
-        float tmp2[3] = {0.f, 0.f, 0.f};
-        float g_sigma = 0.f;
-        if (active) {
-            bool march_done = !(r.t < r.tmax);
-            if (!march_done) {
+        // ---- walk
+        int32_t q_leaf[kQueue];
+        float q_dt[kQueue];
+        int n = 0;
+        bool broken = false;
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            q_leaf[q] = 0;
+            q_dt[q] = 0.0f;
+            if (active && !broken && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
-                    const float* rec = tr.data + v.leaf * K;
-                    const float sigma = rec[K - 1];
-                    if (sigma > 0.0f) {
-                        const float att = expf_fixed(-delta_t * sigma * r.dscale);
-                        const float weight = light * (1.0f - att);
-                        float s[3];
-                        leaf_colour<P, kMarchThreads>(rec, basis_t + lane, s);
-                        float total_color = 0.0f;
-#pragma unroll
-                        for (int c = 0; c < 3; ++c)
-                            total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
-                        light *= att;
-                        if (!second) {
-                            accum = fma_(weight, total_color, accum);
-                        } else {
-#pragma unroll
-                            for (int c = 0; c < 3; ++c) {
-                                if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                                    tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
-                                } else {
-                                    tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) *
-                                                      (double)go[c] * (double)d_rgb_pad);
-                                }
-                            }
-                            accum = fma_(-weight, total_color, accum);
-                            g_sigma = delta_t * r.dscale * fma_(total_color, light, -accum);
-                            leaf = (int32_t)v.leaf;
-                            emit = true;
-                        }
-                    }
+                    q_leaf[q] = (int32_t)v.leaf;
+                    q_dt[q] = delta_t;
                     r.t += delta_t;
-                    march_done = !(r.t < r.tmax);
+                    n = q + 1;
                 } else {
-                    march_done = true;
-                    second = true;   // malformed tree: give the ray up
-                }
-            }
-            if (march_done) {
-                if (!second) {
-                    const float total_grad = (go[0] + go[1]) + go[2];
-                    accum = fma_(light * bg, total_grad, accum);
-                    light = 1.0f;
-                    r.t = tmin;
-                    second = true;
-                } else {
-                    active = false;
+                    broken = true;
                 }
             }
         }
-        unsigned long long todo = __ballot(emit);
-        while (todo) {
-            const int leader = __ffsll((long long)todo) - 1;
-            const int32_t leaf_l = __builtin_amdgcn_readlane(leaf, leader);
-            const unsigned long long same = __ballot(emit && leaf == leaf_l);
-            todo &= ~same;
-            float* g = grad_data + (int64_t)leaf_l * K;
+        // ---- sigma
+        float q_sigma[kQueue];
 #pragma unroll
-            for (int e0 = 0; e0 < K; e0 += 64) {
-                const int e = e0 + lane;
-                float val = 0.0f;
-                unsigned long long members = same;
-                while (members) {
-                    const int k = __ffsll((long long)members) - 1;
-                    members &= members - 1;
-                    const float t0 = read_lane(tmp2[0], k);
-                    const float t1 = read_lane(tmp2[1], k);
-                    const float t2 = read_lane(tmp2[2], k);
-                    const float gs = read_lane(g_sigma, k);
-                    float term;
-                    if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                        term = e == 0 ? t0 : e == 1 ? t1 : e == 2 ? t2 : gs;
-                    } else {
-                        const int c = e / D;
-                        const float b = e < 3 * D ? basis_lds[k * D + (e - c * D)] : 0.0f;
-                        const float tc = c == 0 ? t0 : c == 1 ? t1 : t2;
-                        term = e < 3 * D ? b * tc : gs;
+        for (int q = 0; q < kQueue; ++q)
+            q_sigma[q] = q < n ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+        // ---- shade list
+        int n_entries = 0;
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            const bool want = q < n && q_sigma[q] > 0.0f;
+            const unsigned long long m = __ballot(want);
+            if (want) {
+                const int e = n_entries + rank_in(m);
+                sh.leaf[e] = q_leaf[q];
+                sh.who[e] = lane | (q << 8);
+            }
+            n_entries += __popcll(m);
+        }
+        __syncthreads();
+        shade_entries<P>(tr.data, sh, n_entries, lane);
+        __syncthreads();
+        // ---- composite and emit, slot by slot
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            bool emit = false;
+            float tmp2[3] = {0.f, 0.f, 0.f};
+            float g_sigma = 0.f;
+            if (active && q < n && q_sigma[q] > 0.0f) {
+                const float att = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
+                const float weight = light * (1.0f - att);
+                const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+                float total_color = 0.0f;
+#pragma unroll
+                for (int c = 0; c < 3; ++c) total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+                light *= att;
+                if (!second) {
+                    accum = fma_(weight, total_color, accum);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) {
+                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                            tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
+                        } else {
+                            tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)go[c] *
+                                              (double)d_rgb_pad);
+                        }
                     }
-                    val += term;
+                    accum = fma_(-weight, total_color, accum);
+                    g_sigma = q_dt[q] * r.dscale * fma_(total_color, light, -accum);
+                    emit = true;
                 }
-                if (e < K) atomicAdd(g + e, val);
+            }
+            unsigned long long todo = __ballot(emit);
+            while (todo) {
+                const int leader = __ffsll((long long)todo) - 1;
+                const int32_t leaf_l = __builtin_amdgcn_readlane(q_leaf[q], leader);
+                const unsigned long long same = __ballot(emit && q_leaf[q] == leaf_l);
+                todo &= ~same;
+                float* g = grad_data + (int64_t)leaf_l * K;
+#pragma unroll
+                for (int e0 = 0; e0 < K; e0 += 64) {
+                    const int e = e0 + lane;
+                    float val = 0.0f;
+                    unsigned long long members = same;
+                    while (members) {
+                        const int k = __ffsll((long long)members) - 1;
+                        members &= members - 1;
+                        const float t0 = read_lane(tmp2[0], k);
+                        const float t1 = read_lane(tmp2[1], k);
+                        const float t2 = read_lane(tmp2[2], k);
+                        const float gs = read_lane(g_sigma, k);
+                        float term;
+                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                            term = e == 0 ? t0 : e == 1 ? t1 : e == 2 ? t2 : gs;
+                        } else {
+                            const int c = e / D;
+                            const float b = e < 3 * D ? sh.basis[k * D + (e - c * D)] : 0.0f;
+                            const float tc = c == 0 ? t0 : c == 1 ? t1 : t2;
+                            term = e < 3 * D ? b * tc : gs;
+                        }
+                        val += term;
+                    }
+                    if (e < K) atomicAdd(g + e, val);
+                }
+            }
+        }
+        // ---- end of a march
+        if (active && (broken || !(r.t < r.tmax))) {
+            if (!second && !broken) {
+                const float total_grad = (go[0] + go[1]) + go[2];
+                accum = fma_(light * bg, total_grad, accum);
+                light = 1.0f;
+                r.t = tmin;
+                second = true;
+            } else {
+                active = false;
             }
         }
     }
