@@ -387,21 +387,25 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_generic_kernel(T
 constexpr int kQueue = 4;  // leaves a lane walks ahead before the wavefront shades them
 
 // Shade list shared by the wavefront: the (lane, slot) pairs of one round whose leaf has to be
-// shaded, compacted so that consecutive lanes can take consecutive entries.
-template <int D>
+// shaded, compacted so that consecutive lanes can take consecutive entries.  kRows: the basis of
+// every lane's ray is kept as a row (needed where other lanes multiply with it); otherwise only
+// the view direction is kept and the basis is re-evaluated where it is used.
+template <int D, bool kRows>
 struct ShadeShared {
     int32_t leaf[kQueue * kMarchThreads];       // leaf cell index of entry e
-    int32_t who[kQueue * kMarchThreads];        // owner lane | slot << 8
+    uint8_t who[kQueue * kMarchThreads];        // owner lane | slot << 6
     float colour[kQueue * kMarchThreads * 3];   // [slot][lane][channel]: sigmoid(basis . coefficients)
-    float basis[kMarchThreads * D];             // [lane][coefficient]
+    float basis[kRows ? kMarchThreads * D : 1]; // [lane][coefficient]
+    float vdir[kRows ? 1 : kMarchThreads * 3];  // [lane][xyz]
 };
 
 // Colours of all list entries, computed by the whole wavefront: item p = 3 * entry + channel goes to
 // lane p mod 64.  One item is the reference's dot product for one channel, evaluated in the
-// reference's order (coefficient 0 first) from 16-byte loads of the leaf record and of the owner
-// lane's basis row, followed by the sigmoid.
-template <class P>
-__device__ __forceinline__ void shade_entries(const float* __restrict__ data, ShadeShared<(P::kBasis > 0 ? P::kBasis : 1)>& sh,
+// reference's order (coefficient 0 first) from 16-byte loads of the leaf record and the owner
+// lane's basis, followed by the sigmoid.
+template <class P, bool kRows>
+__device__ __forceinline__ void shade_entries(const float* __restrict__ data,
+                                              ShadeShared<(P::kBasis > 0 ? P::kBasis : 1), kRows>& sh,
                                               int n_entries, int lane) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
@@ -410,14 +414,21 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data, Sh
         const int e = p / 3, c = p - 3 * e;
         const int32_t leaf = sh.leaf[e];
         const int who = sh.who[e];
-        const int owner = who & 255, slot = who >> 8;
+        const int owner = who & 63, slot = who >> 6;
         const float* rec = data + (int64_t)leaf * K;
         float s;
         if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
             s = sigmoid_(rec[c]);
         } else {
             const float* co = rec + c * D;
-            const float* b = sh.basis + owner * D;
+            float b[D];
+            if constexpr (kRows) {
+#pragma unroll
+                for (int i = 0; i < D; ++i) b[i] = sh.basis[owner * D + i];
+            } else {
+                const float vd[3] = {sh.vdir[owner * 3], sh.vdir[owner * 3 + 1], sh.vdir[owner * 3 + 2]};
+                sh_basis<float>(P::kBasis, vd, b);
+            }
             float tmp = 0.0f;
 #pragma unroll
             for (int i = 0; i < D; ++i) tmp = fma_(b[i], co[i], tmp);
@@ -450,7 +461,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[kPathLevels * kMarchThreads];
-    __shared__ ShadeShared<D> sh;
+    __shared__ ShadeShared<D, false> sh;
     const int lane = threadIdx.x;
     float offset[3], scaling[3];
     load_transform(tr, offset, scaling);
@@ -485,10 +496,9 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                     if (slot >= 0) {
                         if (setup_ray(r, origin, dir, scaling)) {
                             if constexpr (P::kFormat == SVOX_FORMAT_SH) {
-                                float basis[D];
-                                sh_basis<float>(P::kBasis, vdir, basis);
-#pragma unroll
-                                for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
+                                sh.vdir[lane * 3] = vdir[0];
+                                sh.vdir[lane * 3 + 1] = vdir[1];
+                                sh.vdir[lane * 3 + 2] = vdir[2];
                             }
                             acc[0] = acc[1] = acc[2] = 0.0f;
                             light = 1.0f;
@@ -543,12 +553,12 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
             if (want) {
                 const int e = n_entries + rank_in(m);
                 sh.leaf[e] = q_leaf[q];
-                sh.who[e] = lane | (q << 8);
+                sh.who[e] = (uint8_t)(lane | (q << 6));
             }
             n_entries += __popcll(m);
         }
         __syncthreads();   // one wavefront per block: list and basis rows are visible to every lane
-        shade_entries<P>(tr.data, sh, n_entries, lane);
+        shade_entries<P, false>(tr.data, sh, n_entries, lane);
         __syncthreads();
         // ---- composite
         if (active) {
@@ -723,7 +733,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[kPathLevels * kMarchThreads];
-    __shared__ ShadeShared<D> sh;
+    __shared__ ShadeShared<D, true> sh;
     const int lane = threadIdx.x;
     float offset[3], scaling[3];
     load_transform(tr, offset, scaling);
@@ -814,12 +824,12 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             if (want) {
                 const int e = n_entries + rank_in(m);
                 sh.leaf[e] = q_leaf[q];
-                sh.who[e] = lane | (q << 8);
+                sh.who[e] = (uint8_t)(lane | (q << 6));
             }
             n_entries += __popcll(m);
         }
         __syncthreads();
-        shade_entries<P>(tr.data, sh, n_entries, lane);
+        shade_entries<P, true>(tr.data, sh, n_entries, lane);
         __syncthreads();
         // ---- composite and emit, slot by slot
 #pragma unroll
