@@ -1,0 +1,175 @@
+"""Trees whose data tensor has more than 2^31 elements (64-bit addressing inside the kernels) and
+full-size property checks that need no CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import svox_amd as svox
+from svox_amd import csrc as C
+from svox_amd import synth
+from util import grad_close, rays_spec
+
+pytestmark = pytest.mark.gpu
+
+
+def torch_descend(tree, pts):
+    """Independent level-by-level walk with torch ops on the GPU: packed leaf ids for tree-space points."""
+    N = tree.N
+    hi = torch.tensor(np.frombuffer(np.uint32(0x3F7FFFEF).tobytes(), np.float32)[0], device=pts.device)
+    p = torch.minimum(torch.clamp_min(pts, 0.0), hi).clone()
+    node = torch.zeros(pts.shape[0], dtype=torch.long, device=pts.device)
+    out = torch.full((pts.shape[0],), -1, dtype=torch.long, device=pts.device)
+    live = torch.arange(pts.shape[0], device=pts.device)
+    for _ in range(32):
+        p = p * N
+        f = torch.floor(p)
+        p = p - f
+        idx = f.long()
+        cell = ((node * N + idx[:, 0]) * N + idx[:, 1]) * N + idx[:, 2]
+        skip = tree.child.reshape(-1)[cell].long()
+        done = skip == 0
+        out[live[done]] = cell[done]
+        keep = ~done
+        live, p, node = live[keep], p[keep], (node + skip)[keep]
+        if live.numel() == 0:
+            break
+    return out
+
+
+@pytest.fixture(scope="module")
+def big_tree(gpu):
+    """SH25 octree with 3.6 M nodes: 3.6e6 * 8 * 76 = 2.19e9 > 2^31 elements (8.8 GB)."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 * 2 ** 30:
+        pytest.skip("needs 40 GB of free device memory")
+    tree = svox.N3Tree(N=2, data_format="SH25", init_refine=5, depth_limit=9, device=gpu)   # 64^3 leaves, 37 449 nodes
+    g = torch.Generator().manual_seed(0)
+    while tree.n_internal < 3_600_000:
+        leaves = tree._all_leaves()
+        need = 3_600_000 - tree.n_internal
+        pick = torch.randperm(leaves.shape[0], generator=g)[:need]
+        tree.refine(sel=tuple(leaves[pick].T))
+    assert tree.n_internal == 3_600_000 and tree.data.numel() > 2 ** 31
+    # every element holds a function of its own flat index; sigma (last of 76) only on some leaves
+    flat = tree.data.data.view(-1)
+    chunk = 1 << 27
+    for s in range(0, flat.numel(), chunk):
+        e = min(s + chunk, flat.numel())
+        i = torch.arange(s, e, device=gpu)
+        v = (i % 8191).float() / 8191.0 - 0.5
+        is_sigma = (i % 76) == 75
+        dense = ((i // 76) % 5) == 0
+        flat[s:e] = torch.where(is_sigma, torch.where(dense, v.abs() * 40.0 + 1.0, torch.zeros_like(v)), v)
+    return tree
+
+
+def element_value(i):
+    v = (i % 8191).float() / 8191.0 - 0.5
+    is_sigma = (i % 76) == 75
+    dense = ((i // 76) % 5) == 0
+    return torch.where(is_sigma, torch.where(dense, v.abs() * 40.0 + 1.0, torch.zeros_like(v)), v)
+
+
+def test_query_addresses_beyond_2_31(gpu, big_tree):
+    tree = big_tree
+    # half of the points uniform, half at the centres of leaves of the highest-numbered nodes
+    tail = tree._all_leaves()[-(1 << 19):].to(gpu)
+    size = 2.0 ** (-(tree.parent_depth[tail[:, 0], 1].float() + 1.0))
+    centres = synth._leaf_corners(tree, tail) + 0.5 * size[:, None]
+    pts = torch.cat([torch.rand(1 << 19, 3, device=gpu, generator=torch.Generator(device=gpu).manual_seed(1)),
+                     centres]).contiguous()
+    vals, ids = tree(pts, want_node_ids=True, world=False)
+    assert torch.equal(ids[1 << 19:], tree._pack_index(tail))
+    want_ids = torch_descend(tree, pts)
+    assert torch.equal(ids, want_ids)
+    assert (ids * 76 > 2 ** 31).float().mean() > 0.2          # plenty of leaves live past the int32 range
+    cols = torch.arange(76, device=gpu)
+    for s in range(0, pts.shape[0], 1 << 18):
+        e = s + (1 << 18)
+        want = element_value(ids[s:e, None] * 76 + cols[None])
+        assert torch.equal(vals[s:e].detach(), want)
+    # the generic kernel agrees
+    C.set_debug_flags(1)
+    try:
+        vals2, ids2 = tree(pts[:100000], want_node_ids=True, world=False)
+    finally:
+        C.set_debug_flags(0)
+    assert torch.equal(ids2, ids[:100000]) and torch.equal(vals2, vals[:100000])
+    # query backward scatters to the same addresses
+    go = torch.ones(pts.shape[0], 76, device=gpu)
+    tree.data.grad = None
+    vals.backward(go)
+    counts = torch.bincount(ids, minlength=0)
+    nz = counts.nonzero().reshape(-1)
+    got = tree.data.grad.view(-1, 76)[nz]
+    assert torch.equal(got, counts[nz, None].float().expand(-1, 76))
+    assert float(tree.data.grad.sum()) == float(pts.shape[0] * 76)
+    tree.data.grad = None
+
+
+def test_render_specialised_and_generic_kernels_agree_on_a_huge_tree(gpu, big_tree):
+    tree = big_tree
+    rays = synth.sphere_rays(20000, seed=3)
+    r = svox.VolumeRenderer(tree, step_size=1e-3)
+    opt = r._get_options(True)
+    spec = rays_spec(rays, gpu)
+    out = C.volume_render(tree._spec(), spec, opt)
+    stats = C.volume_render_stats(tree._spec(), spec, opt)
+    C.set_debug_flags(1)
+    try:
+        out_generic = C.volume_render(tree._spec(), spec, opt)
+    finally:
+        C.set_debug_flags(0)
+    assert torch.equal(out, out_generic)
+    assert stats["samples_shaded"] > 10000 and torch.isfinite(out).all()
+    go = torch.randn(20000, 3, device=gpu, generator=torch.Generator(device=gpu).manual_seed(2))
+    grad = C.volume_render_backward(tree._spec(), spec, opt, go)
+    C.set_debug_flags(1)
+    try:
+        grad_generic = C.volume_render_backward(tree._spec(), spec, opt, go)
+    finally:
+        C.set_debug_flags(0)
+    touched = grad_generic.view(-1, 76).abs().sum(1).nonzero().reshape(-1)
+    assert (touched * 76 > 2 ** 31).any()
+    assert torch.equal(grad.view(-1, 76).abs().sum(1).nonzero().reshape(-1), touched)
+    err, ok = grad_close(grad.view(-1, 76)[touched].cpu().numpy(), grad_generic.view(-1, 76)[touched].cpu().numpy())
+    assert ok, err
+
+
+def test_full_size_render_properties(gpu):
+    """The benchmark tree at full size (no oracle can run there in seconds): properties the domain fixes."""
+    tree = synth.shell_tree(depth=9, n_spheres=24, data_format="SH16", seed=0, device=gpu)
+    r = svox.VolumeRenderer(tree, step_size=5e-4)
+    pose = synth.orbit_poses(1, seed=1, radius=4.0)[0].to(gpu)
+    with torch.no_grad():
+        img = r.render_persp(pose, width=800, height=800, fx=1111.111, fast=True)
+        # the image kernel and the batch kernel on the same pixel rays
+        rays = svox.VolumeRenderer.persp_rays(pose, 800, 800, 1111.111)
+        sel = torch.randperm(640000, generator=torch.Generator().manual_seed(0))[:200000].to(gpu)
+        batch = r(svox.Rays(rays.origins[sel].contiguous(), rays.dirs[sel].contiguous(), rays.viewdirs[sel].contiguous()), fast=True)
+    diff = (img.reshape(-1, 3)[sel] - batch).abs().max(dim=1).values
+    # persp_rays builds directions in float64 and rounds; the kernel mixes float and double as the reference
+    # does: a pixel whose sample lands within rounding of a cell face can take another leaf
+    assert float(diff.median()) < 1e-6 and float((diff > 1e-3).float().mean()) < 0.01
+    assert torch.isfinite(img).all() and float(img.min()) >= -1e-6 and float(img.max()) <= 1.0 + 1e-4
+    # thresholds only remove work: the exact render differs from the fast one by at most what they cut
+    with torch.no_grad():
+        exact = r.render_persp(pose, width=800, height=800, fx=1111.111, fast=False)
+    assert float((exact - img).abs().max()) < 0.05
+    # counters: every ray is counted once, the fast march visits no more leaves than the exact one
+    from svox_amd.renderer import _make_camera_spec
+    cam = _make_camera_spec(pose.contiguous(), 800, 800, 1111.111, 1111.111)
+    fast_stats = C.volume_render_stats(tree._spec(), cam, r._get_options(True))
+    exact_stats = C.volume_render_stats(tree._spec(), cam, r._get_options(False))
+    assert fast_stats["rays"] == exact_stats["rays"] == 640000
+    assert fast_stats["samples"] <= exact_stats["samples"] == exact_stats["samples_bwd"]
+    # gradient of a linear functional is linear in grad_output
+    pts_rays = svox.Rays(rays.origins[sel[:50000]].contiguous(), rays.dirs[sel[:50000]].contiguous(),
+                         rays.viewdirs[sel[:50000]].contiguous())
+    go = torch.randn(50000, 3, device=gpu)
+    spec = rays_spec(pts_rays)
+    opt = r._get_options(True)
+    g1 = C.volume_render_backward(tree._spec(), spec, opt, go)
+    g2 = C.volume_render_backward(tree._spec(), spec, opt, 2.0 * go)
+    nz = g1.view(-1).abs() > 1e-6
+    assert float(((g2.view(-1)[nz] / g1.view(-1)[nz]) - 2.0).abs().max()) < 1e-3
