@@ -176,15 +176,18 @@ int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
 }
 
 // Items (rays) a persistent wavefront owns.  With few rays every wavefront gets one 64-item chunk so
-// that the launch spreads over as many SIMDs as possible; with many, 256 items, which lets lanes whose
-// rays end early pick up new ones.
-int pick_per_wave(int64_t total_items) {
+// that the launch spreads over as many SIMDs as possible; with many, several chunks, which lets lanes
+// whose rays end early pick up new ones (measured on 1M random rays: forward best at 256 rays per
+// wavefront, backward -- two marches per ray, longer-lived lanes -- at 512).
+// SVOX_PER_WAVE / SVOX_REFILL override the choice for experiments.
+int pick_per_wave(int64_t total_items, bool backward) {
     static const int forced = [] {
         const char* e = getenv("SVOX_PER_WAVE");
         return e ? atoi(e) : 0;
     }();
-    if (forced == 64 || forced == 256 || forced == 512 || forced == 1024) return forced;
-    return total_items >= (int64_t)64 * 1024 * 8 ? 512 : 64;
+    if (forced == 64 || forced == 128 || forced == 256 || forced == 512 || forced == 1024) return forced;
+    if (total_items < (int64_t)64 * 1024 * 8) return 64;
+    return backward ? 512 : 256;
 }
 
 int pick_refill() {
@@ -196,13 +199,13 @@ int pick_refill() {
 }
 
 template <typename T>
-BatchSource<T> batch_source(const SvoxRaysSpec* rays) {
+BatchSource<T> batch_source(const SvoxRaysSpec* rays, bool backward = false) {
     BatchSource<T> s;
     s.rays.origins = (const T*)rays->origins;
     s.rays.dirs = (const T*)rays->dirs;
     s.rays.vdirs = (const T*)rays->vdirs;
     s.rays.n_rays = rays->n_rays;
-    s.per_wave = pick_per_wave(rays->n_rays);
+    s.per_wave = pick_per_wave(rays->n_rays, backward);
     s.refill_at = pick_refill();
     return s;
 }
@@ -220,8 +223,7 @@ ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pos
     const int64_t total = (int64_t)n_images * blocks16_of(cam->width) * blocks16_of(cam->height) * 256;
     // image tiles are coherent (rays of a tile end together) and only part of an image hits the
     // tree: one tile per wavefront keeps the busy tiles spread over the whole GPU
-    const int pw = pick_per_wave(0);
-    s.per_wave = pw > 256 ? 256 : pw;
+    s.per_wave = 64;
     s.refill_at = pick_refill();
     return s;
 }
@@ -449,10 +451,10 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
     if (rays->n_rays == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
     if (tree->dtype == SVOX_F32)
-        launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays), opt, od, grad_output,
+        launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays, true), opt, od, grad_output,
                                                    grad_data_out, (hipStream_t)stream);
     else
-        launch_backward<BatchSource<double>, double>(tree, batch_source<double>(rays), opt, od, grad_output,
+        launch_backward<BatchSource<double>, double>(tree, batch_source<double>(rays, true), opt, od, grad_output,
                                                      grad_data_out, (hipStream_t)stream);
     return check_launch("volume_render_backward");
 }
