@@ -218,8 +218,8 @@ __device__ __forceinline__ Visit step_octree(const TreeDev<float>& tr, const Ray
 #pragma unroll
     for (int j = 0; j < 3; ++j) pc[j] = clamp01(fma_(r.t, r.d[j], r.o[j]));
     Visit v;
-    const int32_t leaf = cur.seek(tr.child, tr.capacity, cell_coord(pc[0]), cell_coord(pc[1]),
-                                  cell_coord(pc[2]), reads);
+    const int32_t leaf = cur.seek(tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]), cell_coord(pc[1]),
+                                  cell_coord(pc[2]));
     float inv_cube;  // 2^-levels: dividing by the power of two 2^levels is this multiplication
     float local[3];
     if (leaf >= 0) {
@@ -460,7 +460,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                                                                        float* __restrict__ out) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
-    __shared__ int32_t path[kPathLevels * kMarchThreads];
+    __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
     __shared__ ShadeShared<D, false> sh;
     const int lane = threadIdx.x;
     float offset[3], scaling[3];
@@ -732,7 +732,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                                                                         float* __restrict__ grad_data) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
-    __shared__ int32_t path[kPathLevels * kMarchThreads];
+    __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
     __shared__ ShadeShared<D, true> sh;
     const int lane = threadIdx.x;
     float offset[3], scaling[3];

@@ -128,8 +128,8 @@ __device__ __forceinline__ float leaf_local(float pc, float cube_sz) {
 }
 
 // Per-lane cursor that remembers the previous descent.  `path` points at this lane's column of an
-// LDS array laid out [kPathLevels][block threads]: path[l * stride] is the node whose child row is
-// indexed at level l + 1 (path[0] is the root, node 0).
+// LDS array laid out [kPathLevels + 1][block threads]: path[l * stride] is the node whose child row
+// is indexed at level l + 1 (path[0] is the root, node 0); the last row is a dump for deeper levels.
 struct OctreeCursor {
     int32_t* path;
     int stride;
@@ -146,39 +146,42 @@ struct OctreeCursor {
     }
 
     // Finds the leaf of the point with integer coordinates (nx, ny, nz).  Returns the leaf cell
-    // index (or -1); `levels` is updated.  `reads` is incremented per child entry read.
-    __device__ __forceinline__ int32_t seek(const int32_t* __restrict__ child, int64_t capacity,
-                                            uint32_t nx, uint32_t ny, uint32_t nz, int* reads) {
+    // index, or -1 if the tree has more levels than the coordinates hold (`levels` becomes 0).
+    // Node ids read from the table are clamped into [0, capacity): a malformed tree yields a wrong
+    // leaf, never an access outside the table.  The loop has a single exit so that lanes which
+    // found their leaf only wait, without extra mask bookkeeping per level.
+    __device__ __forceinline__ int32_t seek(const int32_t* __restrict__ child, int32_t last_node,
+                                            uint32_t nx, uint32_t ny, uint32_t nz) {
         int level = 1;
         int32_t node = 0;
         if (levels > 0) {
             const uint32_t diff = (ix ^ nx) | (iy ^ ny) | (iz ^ nz);
             // first level at which the two points fall into different cells
             const int first_diff = diff ? (kCoordBits - 31 + __builtin_clz(diff)) : kCoordBits + 1;
-            if (first_diff > levels) {
-                ix = nx; iy = ny; iz = nz;
-                return leaf;  // still inside the previous leaf
-            }
+            ix = nx; iy = ny; iz = nz;
+            if (first_diff > levels) return leaf;  // still inside the previous leaf
             level = first_diff < kPathLevels ? first_diff : kPathLevels;
             node = path[(level - 1) * stride];
+        } else {
+            ix = nx; iy = ny; iz = nz;
         }
-        ix = nx; iy = ny; iz = nz;
-        for (; level <= kCoordBits; ++level) {
-            if (level <= kPathLevels) path[(level - 1) * stride] = node;
-            const int32_t cell = node * 8 + cell_at(nx, ny, nz, level);
-            const int32_t skip = child[cell];
-            *reads += 1;
-            if (skip == 0) {
-                levels = level;
-                leaf = cell;
-                return cell;
-            }
-            node += skip;
-            if (node < 0 || node >= capacity) break;
+        int32_t cell, skip;
+        while (true) {
+            path[((level < kPathLevels ? level : kPathLevels + 1) - 1) * stride] = node;
+            cell = node * 8 + cell_at(nx, ny, nz, level);
+            skip = child[cell];
+            if (skip == 0 || level == kCoordBits) break;
+            node = min(max(node + skip, 0), last_node);   // v_med3_i32
+            level += 1;
         }
-        levels = 0;
-        leaf = -1;
-        return -1;
+        if (skip != 0) {
+            levels = 0;
+            leaf = -1;
+            return -1;
+        }
+        levels = level;
+        leaf = cell;
+        return cell;
     }
 };
 
