@@ -70,9 +70,9 @@ TreeDev<T> make_tree(const SvoxTreeSpec* t) {
     return d;
 }
 
-// cell indices fit int32 and the tree is an fp32 octree
+// an fp32 octree whose child table is smaller than 4 GiB (32-bit byte offsets, int32 cell indices)
 bool octree_fast_ok(const SvoxTreeSpec* t) {
-    return !(g_debug_flags & 1) && t->dtype == SVOX_F32 && t->N == 2 && t->capacity < (1ll << 28);
+    return !(g_debug_flags & 1) && t->dtype == SVOX_F32 && t->N == 2 && t->capacity < (1ll << 27);
 }
 
 int zero_fill(void* ptr, int64_t bytes, hipStream_t stream) {

@@ -96,8 +96,10 @@ __device__ __forceinline__ int64_t descend_generic(const int32_t* __restrict__ c
 __device__ __forceinline__ uint32_t cell_coord(float pc) { return (uint32_t)(pc * 16777216.0f); }
 
 __device__ __forceinline__ int cell_at(uint32_t ix, uint32_t iy, uint32_t iz, int level) {
-    const int s = kCoordBits - level;
-    return (int)((((ix >> s) & 1u) << 2) | (((iy >> s) & 1u) << 1) | ((iz >> s) & 1u));
+    const unsigned s = (unsigned)(kCoordBits - level);
+    const unsigned bx = __builtin_amdgcn_ubfe(ix, s, 1u), by = __builtin_amdgcn_ubfe(iy, s, 1u),
+                   bz = __builtin_amdgcn_ubfe(iz, s, 1u);
+    return (int)((((bx << 1) | by) << 1) | bz);
 }
 
 // Octree walk over integer coordinates with no path memory (point queries).
@@ -168,10 +170,13 @@ struct OctreeCursor {
         int32_t cell, skip;
         while (true) {
             path[((level < kPathLevels ? level : kPathLevels + 1) - 1) * stride] = node;
-            cell = node * 8 + cell_at(nx, ny, nz, level);
-            skip = child[cell];
+            cell = (node << 3) | cell_at(nx, ny, nz, level);
+            // the table is smaller than 4 GiB (checked on the host): a 32-bit byte offset from the
+            // uniform base lets the load use the scalar-base addressing form
+            skip = *(const int32_t*)((const char*)child + ((uint32_t)cell << 2));
             if (skip == 0 || level == kCoordBits) break;
-            node = min(max(node + skip, 0), last_node);   // v_med3_i32
+            // a negative or too large id (malformed tree) wraps / clamps to the last node
+            node = (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node);
             level += 1;
         }
         if (skip != 0) {
