@@ -280,6 +280,15 @@ inline void dda_unit(const T* cen, const T* invdir, T* tmin, T* tmax) {
     }
 }
 
+// t += delta_t.  Where t can no longer advance (delta below the spacing of floats at t, or NaN) the
+// reference's `while (t < tmax)` never ends; the ray is ended after this sample instead (the one
+// deliberate departure from the reference, shared with the kernels).
+template <typename T>
+inline T advance_t(T t, T delta_t, T tmax) {
+    const T t_next = t + delta_t;
+    return t_next > t ? t_next : tmax;
+}
+
 struct Counters {
     uint64_t rays = 0, rays_hit = 0, samples = 0, shaded = 0, bwd = 0, bwd_pos = 0, levels = 0;
 };
@@ -381,7 +390,7 @@ void trace_ray(const TreeView<T>& tr, const SvoxRenderOptions& opt, const T* ori
                 return;
             }
         }
-        t += delta_t;
+        t = advance_t(t, delta_t, rs.tmax);
     }
     for (int j = 0; j < out_dim; ++j) out[j] = fma_(light, (T)opt.background_brightness, out[j]);
 }
@@ -447,7 +456,7 @@ void trace_ray_backward(const TreeView<T>& tr, const SvoxRenderOptions& opt, con
                 light *= att;
                 accum = fma_(weight, total_color, accum);
             }
-            t += delta_t;
+            t = advance_t(t, delta_t, rs.tmax);
         }
         T total_grad = T(0);
         for (int j = 0; j < out_dim; ++j) total_grad += grad_out[j];
@@ -493,7 +502,7 @@ void trace_ray_backward(const TreeView<T>& tr, const SvoxRenderOptions& opt, con
                 add(base + tr.K - 1,
                     delta_t * rs.delta_scale * fma_(total_color, light, -accum) * chain);
             }
-            t += delta_t;
+            t = advance_t(t, delta_t, rs.tmax);
         }
     }
 }

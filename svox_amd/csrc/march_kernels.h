@@ -189,6 +189,14 @@ __device__ __forceinline__ bool setup_ray(RayState<T>& r, const T* origin, const
     return !(tmax < T(0) || tmin > tmax);
 }
 
+// t += delta_t.  If t cannot advance any more (a delta below the spacing of floats at t, or NaN), the
+// reference's `while (t < tmax)` loop would never end; the ray is ended after this sample instead.
+template <typename T>
+__device__ __forceinline__ void advance(RayState<T>& r, T delta_t) {
+    const T t_next = r.t + delta_t;
+    r.t = t_next > r.t ? t_next : r.tmax;
+}
+
 struct Visit {
     int64_t leaf;  // cell index node*N^3 + cell, -1 ends the ray (malformed tree)
     int levels;
@@ -336,7 +344,7 @@ __device__ void trace_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt
                 break;
             }
         }
-        r.t += delta_t;
+        advance(r, delta_t);
     }
     if (!stopped)
         for (int j = 0; j < out_dim; ++j) acc[j] = fma_(light, (T)opt.background_brightness, acc[j]);
@@ -532,7 +540,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                 if (v.leaf >= 0) {
                     q_leaf[q] = (int32_t)v.leaf;
                     q_dt[q] = delta_t;
-                    r.t += delta_t;
+                    advance(r, delta_t);
                     n = q + 1;
                 } else {
                     broken = true;   // malformed tree: the ray ends here
@@ -650,7 +658,7 @@ __device__ void trace_backward_generic(const TreeDev<T>& tr, const SvoxRenderOpt
                 light *= att;
                 accum = fma_(weight, total_color, accum);
             }
-            r.t += delta_t;
+            advance(r, delta_t);
         }
         T total_grad = T(0);
         for (int j = 0; j < out_dim; ++j) total_grad += go[j];
@@ -690,7 +698,7 @@ __device__ void trace_backward_generic(const TreeDev<T>& tr, const SvoxRenderOpt
                 atomicAdd(grad_data + base + tr.K - 1,
                           delta_t * r.dscale * fma_(total_color, light, -accum) * chain);
             }
-            r.t += delta_t;
+            advance(r, delta_t);
         }
     }
 }
@@ -803,7 +811,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                 if (v.leaf >= 0) {
                     q_leaf[q] = (int32_t)v.leaf;
                     q_dt[q] = delta_t;
-                    r.t += delta_t;
+                    advance(r, delta_t);
                     n = q + 1;
                 } else {
                     broken = true;
@@ -960,7 +968,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_stats_kernel(TreeDev<T> 
                         if (light <= (T)opt.stop_thresh) fwd_live = false;
                     }
                 }
-                r.t += delta_t;
+                advance(r, delta_t);
             }
         }
     }

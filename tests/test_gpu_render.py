@@ -253,3 +253,42 @@ def test_several_poses_in_one_launch_equal_separate_calls(gpu, oracle_mod):
         singles[i].backward(go[i])
     err, ok = grad_close(g_batch.cpu().numpy(), tree.data.grad.cpu().numpy())
     assert ok, err
+
+
+def pathological_rays():
+    nan, inf = float("nan"), float("inf")
+    o = [[0.5, 0.5, -1.0], [0.5, 0.5, -1.0], [nan, 0.5, 0.5], [0.5, 0.5, -1.0], [1e8, 1e8, 1e8], [0.0, 0.0, 0.0],
+         [1.0, 1.0, 1.0], [0.5, 0.5, 0.5], [0.25, 0.5, -3.0], [-inf, 0.5, 0.5], [0.5, 0.5, -1.0], [0.5, 0.5, 1e30],
+         [0.3, 0.3, -1e-30], [2.0, 0.5, 0.5]]
+    d = [[0.0, 0.0, 0.0], [0.0, 0.0, nan], [0.0, 0.0, 1.0], [0.0, 0.0, inf], [-1.0, -1.0, -1.0], [1.0, 1.0, 1.0],
+         [-1.0, -1.0, -1.0], [1e-30, 0.0, 0.0], [0.0, 0.0, 1.0], [1.0, 0.0, 0.0], [0.0, 0.0, 1e-20], [0.0, 0.0, -1.0],
+         [0.0, 0.0, 1.0], [-1.0, 0.0, 0.0]]
+    o = torch.tensor(o, dtype=torch.float32)
+    d = torch.tensor(d, dtype=torch.float32)
+    return svox.Rays(o, d, d.clone())
+
+
+@pytest.mark.parametrize("fmt", ["SH4", "RGBA"])
+def test_pathological_rays_end_and_match_the_oracle(gpu, oracle_mod, fmt):
+    """Zero / NaN / infinite directions and origins, rays on faces and corners, origins so far away
+    that t cannot advance: every ray ends, and ends the same way as in the oracle."""
+    tree = synth.shell_tree(depth=5, n_spheres=4, data_format=fmt, seed=17)
+    rays = pathological_rays()
+    for kw in (dict(step_size=1e-3), dict(step_size=1e-9, fast=True)):
+        opt = options(tree, **kw)
+        out, ref, stats, ref_stats, dev, ot = render_both(gpu, oracle_mod, tree, rays, opt)
+        assert np.array_equal(out, ref, equal_nan=True)
+        assert stats["samples"] == ref_stats["samples"]
+        C.set_debug_flags(1)
+        try:
+            out_generic = C.volume_render(dev._spec(), rays_spec(rays, gpu), opt).cpu().numpy()
+        finally:
+            C.set_debug_flags(0)
+        assert np.array_equal(out_generic, ref, equal_nan=True)
+        go = torch.ones(rays.origins.shape[0], 3)
+        ref_grad = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+        grad = C.volume_render_backward(dev._spec(), rays_spec(rays, gpu), opt, go.to(gpu)).cpu().numpy()
+        finite = np.isfinite(ref_grad)
+        assert np.array_equal(np.isfinite(grad), finite)
+        err, ok = grad_close(np.where(finite, grad, 0.0), np.where(finite, ref_grad, 0.0))
+        assert ok, err

@@ -452,3 +452,17 @@ def test_image_rays_match_persp_rays_and_convert_to_ndc():
     assert np.abs(o - no.numpy()).max() < 1e-5
     assert np.abs(d - nd.numpy()).max() < 1e-5
     assert np.abs(v - base.dirs.numpy()).max() < 1e-6
+
+
+def test_pathological_rays_terminate():
+    """Degenerate rays must end (the reference would loop forever where t cannot advance)."""
+    tree = synth.shell_tree(depth=5, n_spheres=4, data_format="SH4", seed=17)
+    nan, inf = float("nan"), float("inf")
+    o = np.array([[0.5, 0.5, -1.0], [nan, 0.5, 0.5], [1e8, 1e8, 1e8], [0.5, 0.5, 1e30], [0.5, 0.5, -1.0]], np.float32)
+    d = np.array([[0.0, 0.0, 0.0], [0.0, 0.0, 1.0], [-1.0, -1.0, -1.0], [0.0, 0.0, -1.0], [0.0, 0.0, inf]], np.float32)
+    ot = oracle.Tree.from_n3tree(tree)
+    for step in (1e-3, 1e-9, 0.0):
+        out, stats = oracle.volume_render(ot, o, d, d, options(tree, step_size=step), want_stats=True)
+        assert stats["samples"] < 10000
+        grad = oracle.volume_render_backward(ot, o, d, d, options(tree, step_size=step), np.ones((5, 3), np.float32))
+        assert grad.shape == tuple(tree.data.shape)
