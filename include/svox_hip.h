@@ -186,6 +186,21 @@ int svox_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCamera
                                       const SvoxRenderOptions* opt, const void* grad_output,
                                       void* grad_data_out, int32_t accumulate, void* stream);
 
+/* se_grad(TreeSpec&, RaysSpec&, color, RenderOptions&) -> (color_out, grad, hessdiag);
+ * svox.cpp:54-55, 115, rt_kernel.cu:1111-1139 (kernel :479-715, :846-868).
+ * Rendered colour plus gradient and Gauss-Newton Hessian diagonal of 0.5 * |render - color_ref|^2 with
+ * respect to tree.data.  color_ref and color_out are (B, out_dim), out_dim <= 4; grad_out and
+ * hessdiag_out have the shape of tree.data and are zero-filled by the library.  Thresholds are not
+ * applied (the kernel tests sigma > 0 and never stops early). */
+int svox_se_grad(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
+                 const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out, void* stream);
+
+/* se_grad_persp(TreeSpec&, CameraSpec&, RenderOptions&, color) -> (color_out, grad, hessdiag);
+ * svox.cpp:56-57, 116, rt_kernel.cu:1141-1173 (kernel :870-897).  color_ref and color_out are
+ * (H, W, out_dim). */
+int svox_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
+                       const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out, void* stream);
+
 /* get_out_data_dim, rt_kernel.cu:1009-1015.  Returns -1 for an invalid combination. */
 int svox_out_data_dim(int32_t format, int32_t basis_dim, int32_t data_dim);
 

@@ -53,6 +53,8 @@ def lib():
             "oracle_volume_render_image": (ctypes.c_int, [T, C, O, c_void_p, S, c_int32]),
             "oracle_volume_render_backward": (ctypes.c_int, [T, R, O, c_void_p, c_void_p, c_int32, S, c_int32]),
             "oracle_volume_render_image_backward": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_int32, S, c_int32]),
+            "oracle_se_grad": (ctypes.c_int, [T, R, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int32]),
+            "oracle_se_grad_image": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int32]),
             "oracle_image_rays": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_void_p]),
             "oracle_trace_visits": (c_int64, [T, R, c_int64, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int64]),
         }
@@ -255,6 +257,35 @@ def volume_render_image_backward(tree, c2w, fx, fy, width, height, opt, grad_out
                                                      _ptr(go), _ptr(grad), 0, ctypes.byref(st), n_threads),
            "volume_render_image_backward")
     return (grad, st.as_dict()) if want_stats else grad
+
+
+def se_grad(tree, origins, dirs, vdirs, colors, opt, n_threads=1):
+    """(colour (B, C), grad, hessdiag) of 0.5 * |render - colors|^2; grad and hessdiag shaped like tree.data."""
+    keep, r = _rays(tree, origins, dirs, vdirs)
+    o = _opt(opt)
+    od = lib().oracle_out_data_dim(o.format, o.basis_dim, tree.data.shape[4])
+    ref = _np(colors, tree.dtype)
+    assert ref.shape == (r.n_rays, od)
+    out = np.empty((r.n_rays, od), dtype=tree.dtype)
+    grad, hess = np.empty_like(tree.data), np.empty_like(tree.data)
+    s = tree.spec()
+    _check(lib().oracle_se_grad(ctypes.byref(s), ctypes.byref(r), ctypes.byref(o), _ptr(ref), _ptr(out), _ptr(grad),
+                                _ptr(hess), n_threads), "se_grad")
+    return out, grad, hess
+
+
+def se_grad_image(tree, c2w, fx, fy, width, height, colors, opt, n_threads=1):
+    keep, c = _cam(tree, c2w, fx, fy, width, height)
+    o = _opt(opt)
+    od = lib().oracle_out_data_dim(o.format, o.basis_dim, tree.data.shape[4])
+    ref = _np(colors, tree.dtype)
+    assert ref.shape == (height, width, od)
+    out = np.empty((height, width, od), dtype=tree.dtype)
+    grad, hess = np.empty_like(tree.data), np.empty_like(tree.data)
+    s = tree.spec()
+    _check(lib().oracle_se_grad_image(ctypes.byref(s), ctypes.byref(c), ctypes.byref(o), _ptr(ref), _ptr(out),
+                                      _ptr(grad), _ptr(hess), n_threads), "se_grad_image")
+    return out, grad, hess
 
 
 def image_rays(tree, c2w, fx, fy, width, height, opt):

@@ -507,6 +507,149 @@ void trace_ray_backward(const TreeView<T>& tr, const SvoxRenderOptions& opt, con
     }
 }
 
+// One sample of the squared-error marches (rt_kernel.cu:520-537 and the same lines of the later
+// passes): position, leaf, step length, density.
+template <typename T>
+struct SeSample {
+    int64_t leaf;
+    T delta_t, sigma, raw_sigma;
+};
+
+template <typename T>
+inline bool se_sample(const TreeView<T>& tr, const SvoxRenderOptions& opt, const RaySetup<T>& rs,
+                      T t, SeSample<T>* s) {
+    T pos[3];
+    for (int j = 0; j < 3; ++j) pos[j] = fma_(t, rs.dir[j], rs.origin[j]);
+    T cube_sz;
+    s->leaf = descend(tr, pos, &cube_sz, (int*)nullptr);
+    if (s->leaf < 0) return false;
+    T s0, s1;
+    dda_unit(pos, rs.invdir, &s0, &s1);
+    s->delta_t = (s1 - s0) / cube_sz + (T)opt.step_size;
+    s->raw_sigma = tr.data[s->leaf * tr.K + tr.K - 1];
+    s->sigma = opt.density_softplus ? softplus_m1(s->raw_sigma) : s->raw_sigma;
+    return true;
+}
+
+// sigmoid(basis . coefficients) of channel c of a leaf record (rt_kernel.cu:541-547)
+template <typename T>
+inline T channel_sigmoid(const SvoxRenderOptions& opt, const T* basis, const T* val, int c) {
+    if (opt.format == SVOX_FORMAT_RGBA) return sigmoid_(val[c]);
+    const int off = c * opt.basis_dim;
+    T tmp = T(0);
+    for (int i = opt.min_comp; i <= opt.max_comp; ++i) tmp = fma_(basis[i], val[off + i], tmp);
+    return sigmoid_(tmp);
+}
+
+// trace_ray_se_grad_hess, rt_kernel.cu:479-715: rendered colour, gradient and Gauss-Newton Hessian
+// diagonal of 0.5 * |render - color_ref|^2.  Three marches, all with sigma > 0 and no early stop.
+// `add_grad` / `add_hess` receive the reference's atomicAdds in the reference's order.
+// Note the two spellings of the attenuation argument: -delta_t * delta_scale * sigma in the first
+// march (:538), -delta_t * sigma * delta_scale in the other two (:586, :653).
+template <typename T, typename AddG, typename AddH>
+void trace_ray_se_grad(const TreeView<T>& tr, const SvoxRenderOptions& opt, const T* origin,
+                       const T* dir, const T* vdir, int out_dim, const T* color_ref, T* color_out,
+                       AddG add_grad, AddH add_hess) {
+    RaySetup<T> rs;
+    setup_ray(tr, opt, origin, dir, vdir, &rs);
+    if (!rs.hit) {
+        for (int j = 0; j < out_dim; ++j) color_out[j] = (T)opt.background_brightness;
+        return;
+    }
+    const T pad = (T)opt.rgb_padding;
+    const T d_rgb_pad = (T)(1 + 2 * opt.rgb_padding);
+    const T bg = (T)opt.background_brightness;
+    SeSample<T> s;
+    // PASS 1: residual, :516-566 (color_out arrives zero-filled)
+    {
+        T light = T(1), t = rs.tmin;
+        while (t < rs.tmax) {
+            if (!se_sample(tr, opt, rs, t, &s)) return;
+            if (s.sigma > T(0)) {
+                const T* val = tr.data + s.leaf * tr.K;
+                const T att = exp_sp<T>(-s.delta_t * rs.delta_scale * s.sigma);
+                const T weight = light * (T(1) - att);
+                for (int c = 0; c < out_dim; ++c)
+                    color_out[c] = fma_(weight, fma_(channel_sigmoid(opt, rs.basis, val, c), d_rgb_pad, -pad),
+                                        color_out[c]);
+                light *= att;
+            }
+            t = advance_t(t, s.delta_t, rs.tmax);
+        }
+        for (int j = 0; j < out_dim; ++j) color_out[j] += fma_(light, bg, -color_ref[j]);
+    }
+    // PASS 2: colour gradient and the rendered colour as a suffix sum, :568-637
+    T color_accum[4] = {T(0), T(0), T(0), T(0)};
+    {
+        T light = T(1), t = rs.tmin;
+        while (t < rs.tmax) {
+            if (!se_sample(tr, opt, rs, t, &s)) return;
+            if (s.sigma > T(0)) {
+                const int64_t base = s.leaf * tr.K;
+                const T* val = tr.data + base;
+                const T att = exp_sp<T>(-s.delta_t * s.sigma * rs.delta_scale);
+                const T weight = light * (T(1) - att);
+                for (int c = 0; c < out_dim; ++c) {
+                    const T sg = channel_sigmoid(opt, rs.basis, val, c);
+                    if (opt.format != SVOX_FORMAT_RGBA) {
+                        // `1.0 - sigmoid`: double from there on, rounded on store (:604-605)
+                        const T grad_ci = (T)((double)(weight * sg) * (1.0 - (double)sg) * (double)d_rgb_pad);
+                        const int off = c * opt.basis_dim;
+                        for (int i = opt.min_comp; i <= opt.max_comp; ++i) {
+                            const T grad_wi = rs.basis[i] * grad_ci;
+                            add_grad(base + off + i, grad_wi * color_out[c]);
+                            add_hess(base + off + i, grad_wi * grad_wi);
+                        }
+                    } else {
+                        const T grad_ci = weight * sg * (T(1) - sg) * d_rgb_pad;
+                        add_grad(base + c, grad_ci * color_out[c]);
+                        add_hess(base + c, grad_ci * grad_ci);
+                    }
+                    color_accum[c] = fma_(weight, fma_(sg, d_rgb_pad, -pad), color_accum[c]);
+                }
+                light *= att;
+            }
+            t = advance_t(t, s.delta_t, rs.tmax);
+        }
+        for (int j = 0; j < out_dim; ++j) color_accum[j] = fma_(light, bg, color_accum[j]);
+    }
+    // PASS 3: density gradient, :639-708
+    {
+        T light = T(1), t = rs.tmin;
+        T color_curr[4];
+        while (t < rs.tmax) {
+            if (!se_sample(tr, opt, rs, t, &s)) return;
+            if (s.sigma > T(0)) {
+                const int64_t base = s.leaf * tr.K;
+                const T* val = tr.data + base;
+                const T att = exp_sp<T>(-s.delta_t * s.sigma * rs.delta_scale);
+                const T weight = light * (T(1) - att);
+                for (int c = 0; c < out_dim; ++c) {
+                    color_curr[c] = fma_(channel_sigmoid(opt, rs.basis, val, c), d_rgb_pad, -pad);
+                    color_accum[c] = fma_(-weight, color_curr[c], color_accum[c]);
+                }
+                light *= att;
+                for (int j = 0; j < out_dim; ++j) {
+                    const T grad_sigma = s.delta_t * rs.delta_scale * fma_(color_curr[j], light, -color_accum[j]);
+                    const T grad2_sigma = grad_sigma * grad_sigma;
+                    if (opt.density_softplus) {
+                        const T sg = sigmoid_(s.raw_sigma - T(1));
+                        const T d_sg = sg * (T(1) - sg);
+                        add_grad(base + tr.K - 1, grad_sigma * color_out[j] * sg);
+                        add_hess(base + tr.K - 1, fma_(grad2_sigma * sg, sg, grad_sigma * d_sg));
+                    } else {
+                        add_grad(base + tr.K - 1, grad_sigma * color_out[j]);
+                        add_hess(base + tr.K - 1, grad2_sigma);
+                    }
+                }
+            }
+            t = advance_t(t, s.delta_t, rs.tmax);
+        }
+    }
+    // residual -> colour, :710-713
+    for (int j = 0; j < out_dim; ++j) color_out[j] += color_ref[j];
+}
+
 // cam2world_ray, rt_kernel.cu:758-772.  x and y are formed in double (0.5 * width) and rounded;
 // the radicand x*x + y*y is a scalar_t sum widened to double for `+ 1.0`, then sqrtf.
 template <typename T>
@@ -672,6 +815,47 @@ int render_backward_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
         }
     }
     if (stats) merge(stats, total);
+    return SVOX_OK;
+}
+
+// se_grad / se_grad_persp, rt_kernel.cu:1111-1173
+template <typename T>
+int se_grad_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCameraSpec* cam,
+                 const SvoxRenderOptions* opt, const void* color_ref_v, void* color_out_v,
+                 void* grad_v, void* hess_v, int n_threads) {
+    const TreeView<T> tr = make_view<T>(tree);
+    const int od = oracle_out_data_dim(opt->format, opt->basis_dim, tree->data_dim);
+    if (od > 4) return SVOX_ERR_BAD_SHAPE;  // "Tree's output dim cannot be > 4 for se_grad"
+    const int64_t n = rays ? rays->n_rays : (int64_t)cam->width * cam->height;
+    const T* ref = (const T*)color_ref_v;
+    T* out = (T*)color_out_v;
+    T* grad = (T*)grad_v;
+    T* hess = (T*)hess_v;
+    const int64_t total_elems = tr.M * tr.N * tr.N * tr.N * tr.K;
+    std::memset(grad, 0, sizeof(T) * (size_t)total_elems);
+    std::memset(hess, 0, sizeof(T) * (size_t)total_elems);
+    std::memset(out, 0, sizeof(T) * (size_t)(n * od));
+    const bool par = n_threads > 1;
+#pragma omp parallel for schedule(dynamic, 256) num_threads(n_threads > 0 ? n_threads : 1)
+    for (int64_t r = 0; r < n; ++r) {
+        T origin[3], dir[3], vdir[3];
+        if (rays)
+            batch_ray(tr, *rays, r, origin, dir, vdir);
+        else
+            pixel_ray(tr, *cam, *opt, r, origin, dir, vdir);
+        auto add_to = [par](T* dst) {
+            return [dst, par](int64_t off, T v) {
+                if (par) {
+#pragma omp atomic
+                    dst[off] += v;
+                } else {
+                    dst[off] += v;
+                }
+            };
+        };
+        trace_ray_se_grad(tr, *opt, origin, dir, vdir, od, ref + r * od, out + r * od, add_to(grad),
+                          add_to(hess));
+    }
     return SVOX_OK;
 }
 
@@ -876,6 +1060,31 @@ int oracle_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCame
                                              accumulate, stats, n_threads)
                : render_backward_impl<double>(tree, nullptr, cam, opt, grad_output, grad_data_out,
                                               accumulate, stats, n_threads);
+}
+
+// se_grad, rt_kernel.cu:1111-1139: color_ref and color_out are (B, C); grad and hessdiag have the
+// shape of tree.data and are zero-filled here.
+int oracle_se_grad(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
+                   const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out,
+                   int32_t n_threads) {
+    const int rc = check_render_args(tree, opt);
+    if (rc) return rc;
+    if (!rays || !color_ref || !color_out || !grad_out || !hessdiag_out) return SVOX_ERR_NULL_POINTER;
+    return tree->dtype == SVOX_F32
+               ? se_grad_impl<float>(tree, rays, nullptr, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads)
+               : se_grad_impl<double>(tree, rays, nullptr, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads);
+}
+
+// se_grad_persp, rt_kernel.cu:1141-1173: color_ref and color_out are (H, W, C)
+int oracle_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                         const SvoxRenderOptions* opt, const void* color_ref, void* color_out,
+                         void* grad_out, void* hessdiag_out, int32_t n_threads) {
+    const int rc = check_render_args(tree, opt);
+    if (rc) return rc;
+    if (!cam || !cam->c2w || !color_ref || !color_out || !grad_out || !hessdiag_out) return SVOX_ERR_NULL_POINTER;
+    return tree->dtype == SVOX_F32
+               ? se_grad_impl<float>(tree, nullptr, cam, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads)
+               : se_grad_impl<double>(tree, nullptr, cam, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads);
 }
 
 // The rays the image kernels trace, after cam2world / NDC / world->tree: origins, dirs, vdirs are

@@ -398,6 +398,54 @@ def volume_render_image_backward(tree, cam, opt, grad_output):
     return grad
 
 
+def _check_color(color, shape, dtype):
+    _check_input(color, "color")
+    _same_dtype(color, dtype, "color")
+    if tuple(color.shape) != tuple(shape):
+        raise RuntimeError(f"color must have shape {tuple(shape)}, got {tuple(color.shape)}")
+
+
+def _se_out_dim(spec, opt):
+    od = _render_out_dim(spec, opt)
+    if od > 4:
+        raise RuntimeError("Tree's output dim cannot be > 4 for se_grad")   # rt_kernel.cu:1123-1125
+    return od
+
+
+def se_grad(tree, rays, color, opt):
+    """(result (B, C), grad, hessdiag) of 0.5 * |render - color|^2, grad and hessdiag like tree.data;
+    svox.cpp:115, rt_kernel.cu:1111-1139.  Argument order as in the reference: color before opt."""
+    spec = _pack_tree(tree)
+    rspec = _pack_rays(rays, tree.data.dtype)
+    od = _se_out_dim(spec, opt)
+    _check_color(color, (rspec.n_rays, od), tree.data.dtype)
+    result = torch.empty((rspec.n_rays, od), dtype=tree.data.dtype, device=tree.data.device)
+    grad = torch.empty_like(tree.data)
+    hessdiag = torch.empty_like(tree.data)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_se_grad", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt), color.data_ptr(),
+              result.data_ptr(), grad.data_ptr(), hessdiag.data_ptr(), _stream(tree.data.device))
+    return result, grad, hessdiag
+
+
+def se_grad_persp(tree, cam, opt, color):
+    """Image version: color and result are (H, W, C); svox.cpp:116, rt_kernel.cu:1141-1173.
+    Argument order as in the reference: opt before color."""
+    spec = _pack_tree(tree)
+    cspec = _pack_camera(cam, tree.data.dtype)
+    od = _se_out_dim(spec, opt)
+    _check_color(color, (cspec.height, cspec.width, od), tree.data.dtype)
+    result = torch.empty((cspec.height, cspec.width, od), dtype=tree.data.dtype, device=tree.data.device)
+    grad = torch.empty_like(tree.data)
+    hessdiag = torch.empty_like(tree.data)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_se_grad_image", ctypes.byref(spec), ctypes.byref(cspec), ctypes.byref(copt), color.data_ptr(),
+              result.data_ptr(), grad.data_ptr(), hessdiag.data_ptr(), _stream(tree.data.device))
+    return result, grad, hessdiag
+
+
 def volume_render_stats(tree, rays_or_cam, opt):
     """Visit counts of one launch (dict); `rays_or_cam` is a RaysSpec or a CameraSpec."""
     spec = _pack_tree(tree)

@@ -119,6 +119,12 @@ SIGNATURES = {
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int32, c_void_p]),
     "svox_volume_render_image_backward": (
         ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int32, c_void_p]),
+    "svox_se_grad": (
+        ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p, c_void_p,
+                       c_void_p]),
+    "svox_se_grad_image": (
+        ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p, c_void_p,
+                       c_void_p]),
     "svox_volume_render_stats": (
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p]),
 }

@@ -920,6 +920,385 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 }
 
 // ------------------------------------------------------------------------------------------------
+// squared-error gradient and Gauss-Newton Hessian diagonal
+// ------------------------------------------------------------------------------------------------
+// sigmoid(basis . coefficients) of channel c, rt_kernel.cu:541-547
+template <typename T>
+__device__ __forceinline__ T channel_sigmoid(const SvoxRenderOptions& opt, const T* basis, const T* val, int c) {
+    if (opt.format == SVOX_FORMAT_RGBA) return sigmoid_(val[c]);
+    const int off = c * opt.basis_dim;
+    T tmp = T(0);
+    for (int i = opt.min_comp; i <= opt.max_comp; ++i) tmp = fma_(basis[i], val[off + i], tmp);
+    return sigmoid_(tmp);
+}
+
+// trace_ray_se_grad_hess, rt_kernel.cu:479-715, generic flavour: three marches (residual; colour
+// gradients and the rendered colour as a running suffix; density gradients), all with sigma > 0 and
+// no early stop.  The attenuation argument is spelled -delta_t * delta_scale * sigma in the first
+// march and -delta_t * sigma * delta_scale in the other two, as in the reference.  The reference's
+// out_dim atomics per sample on the density entry are summed first and added once.
+template <typename T>
+__device__ void trace_se_grad_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt, const T* origin,
+                                      const T* dir, const T* vdir, const T* scaling, int out_dim,
+                                      const T* color_ref, T* color_out, T* grad, T* hess) {
+    RayState<T> r;
+    if (!setup_ray(r, origin, dir, scaling)) {
+        for (int j = 0; j < out_dim; ++j) color_out[j] = (T)opt.background_brightness;
+        return;
+    }
+    T basis[SVOX_MAX_BASIS_DIM];
+    precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
+    const T pad = (T)opt.rgb_padding;
+    const T d_rgb_pad = (T)(1 + 2 * opt.rgb_padding);
+    const T bg = (T)opt.background_brightness;
+    const T tmin = r.t;
+    T resid[4] = {T(0), T(0), T(0), T(0)};
+    {
+        T light = T(1);
+        while (r.t < r.tmax) {
+            T delta_t;
+            const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+            if (v.leaf < 0) break;
+            const T* val = tr.data + v.leaf * tr.K;
+            T sigma = val[tr.K - 1];
+            if (opt.density_softplus) sigma = softplus_m1(sigma);
+            if (sigma > T(0)) {
+                const T att = exp_sp<T>(-delta_t * r.dscale * sigma);
+                const T weight = light * (T(1) - att);
+                for (int c = 0; c < out_dim; ++c)
+                    resid[c] = fma_(weight, fma_(channel_sigmoid(opt, basis, val, c), d_rgb_pad, -pad), resid[c]);
+                light *= att;
+            }
+            advance(r, delta_t);
+        }
+        for (int j = 0; j < out_dim; ++j) resid[j] += fma_(light, bg, -color_ref[j]);
+    }
+    T color_accum[4] = {T(0), T(0), T(0), T(0)};
+    {
+        T light = T(1);
+        r.t = tmin;
+        while (r.t < r.tmax) {
+            T delta_t;
+            const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+            if (v.leaf < 0) break;
+            const int64_t base = v.leaf * tr.K;
+            const T* val = tr.data + base;
+            T sigma = val[tr.K - 1];
+            if (opt.density_softplus) sigma = softplus_m1(sigma);
+            if (sigma > T(0)) {
+                const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
+                const T weight = light * (T(1) - att);
+                for (int c = 0; c < out_dim; ++c) {
+                    const T sg = channel_sigmoid(opt, basis, val, c);
+                    if (opt.format != SVOX_FORMAT_RGBA) {
+                        const T grad_ci = (T)((double)(weight * sg) * (1.0 - (double)sg) * (double)d_rgb_pad);
+                        const int off = c * opt.basis_dim;
+                        for (int i = opt.min_comp; i <= opt.max_comp; ++i) {
+                            const T grad_wi = basis[i] * grad_ci;
+                            atomicAdd(grad + base + off + i, grad_wi * resid[c]);
+                            atomicAdd(hess + base + off + i, grad_wi * grad_wi);
+                        }
+                    } else {
+                        const T grad_ci = weight * sg * (T(1) - sg) * d_rgb_pad;
+                        atomicAdd(grad + base + c, grad_ci * resid[c]);
+                        atomicAdd(hess + base + c, grad_ci * grad_ci);
+                    }
+                    color_accum[c] = fma_(weight, fma_(sg, d_rgb_pad, -pad), color_accum[c]);
+                }
+                light *= att;
+            }
+            advance(r, delta_t);
+        }
+        for (int j = 0; j < out_dim; ++j) color_accum[j] = fma_(light, bg, color_accum[j]);
+    }
+    {
+        T light = T(1);
+        r.t = tmin;
+        while (r.t < r.tmax) {
+            T delta_t;
+            const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+            if (v.leaf < 0) break;
+            const int64_t base = v.leaf * tr.K;
+            const T* val = tr.data + base;
+            const T raw_sigma = val[tr.K - 1];
+            const T sigma = opt.density_softplus ? softplus_m1(raw_sigma) : raw_sigma;
+            if (sigma > T(0)) {
+                const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
+                const T weight = light * (T(1) - att);
+                T color_curr[4];
+                for (int c = 0; c < out_dim; ++c) {
+                    color_curr[c] = fma_(channel_sigmoid(opt, basis, val, c), d_rgb_pad, -pad);
+                    color_accum[c] = fma_(-weight, color_curr[c], color_accum[c]);
+                }
+                light *= att;
+                T g = T(0), h = T(0);
+                for (int j = 0; j < out_dim; ++j) {
+                    const T grad_sigma = delta_t * r.dscale * fma_(color_curr[j], light, -color_accum[j]);
+                    const T grad2_sigma = grad_sigma * grad_sigma;
+                    if (opt.density_softplus) {
+                        const T sg = sigmoid_(raw_sigma - T(1));
+                        const T d_sg = sg * (T(1) - sg);
+                        g += grad_sigma * resid[j] * sg;
+                        h += fma_(grad2_sigma * sg, sg, grad_sigma * d_sg);
+                    } else {
+                        g += grad_sigma * resid[j];
+                        h += grad2_sigma;
+                    }
+                }
+                atomicAdd(grad + base + tr.K - 1, g);
+                atomicAdd(hess + base + tr.K - 1, h);
+            }
+            advance(r, delta_t);
+        }
+    }
+    for (int j = 0; j < out_dim; ++j) color_out[j] = resid[j] + color_ref[j];
+}
+
+template <typename T, class Source>
+__global__ __launch_bounds__(kMarchThreads) void se_grad_generic_kernel(TreeDev<T> tr, Source src,
+                                                                        SvoxRenderOptions opt, int out_dim,
+                                                                        const T* __restrict__ color_ref,
+                                                                        T* __restrict__ color_out,
+                                                                        T* __restrict__ grad, T* __restrict__ hess) {
+    T offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    T origin[3], dir[3], vdir[3];
+    const int64_t item = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
+    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+    if (slot < 0) return;
+    trace_se_grad_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, color_ref + slot * out_dim,
+                             color_out + slot * out_dim, grad, hess);
+}
+
+// trace_ray_se_grad_hess, octree flavour: the backward kernel's persistent wavefront and rounds.
+// Two marches instead of three: march 1 forms the residual with the first spelling of the
+// attenuation and, beside it, the rendered colour with the second spelling (what the reference's
+// second march accumulates); march 2 then produces, per leaf with sigma > 0, both the colour terms
+// (the reference's second march) and the density terms (its third).  Every term has the reference's
+// value; records are added cooperatively, one coalesced atomic instruction per record element and
+// output array, after summing the lanes whose rays sit in the same leaf.
+template <class P, class Source>
+__global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> tr, Source src, SvoxRenderOptions opt,
+                                                                const float* __restrict__ color_ref,
+                                                                float* __restrict__ color_out,
+                                                                float* __restrict__ grad_data,
+                                                                float* __restrict__ hess_data) {
+    constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
+    constexpr int K = P::kRecord;
+    __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
+    __shared__ ShadeShared<D, true> sh;
+    const int lane = threadIdx.x;
+    float offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    const float bg = opt.background_brightness;
+    const float pad = opt.rgb_padding;
+    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
+    const float step = opt.step_size;
+
+    int64_t next = blockIdx.x * (int64_t)src.per_wave;
+    const int64_t total = src.total();
+    const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
+
+    RayState<float> r;
+    float ref[3] = {0.f, 0.f, 0.f};
+    float resid[3] = {0.f, 0.f, 0.f};    // march 1: colour so far; afterwards the residual
+    float caccum[3] = {0.f, 0.f, 0.f};   // rendered colour not yet passed (second spelling)
+    float light = 1.0f, light1 = 1.0f, tmin = 0.0f;
+    int64_t slot = -1;
+    bool active = false, second = false;
+    int reads = 0;
+    OctreeCursor cur;
+    cur.reset(path + lane, kMarchThreads);
+
+    while (true) {
+        // ---- refill
+        const unsigned long long idle = __ballot(!active);
+        const int n_idle = __popcll(idle);
+        if (next < end && n_idle >= src.refill_at) {
+            if (!active) {
+                const int64_t item = next + rank_in(idle);
+                if (item < end) {
+                    float origin[3], dir[3], vdir[3];
+                    slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+                    if (slot >= 0) {
+                        if (setup_ray(r, origin, dir, scaling)) {
+                            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+                                float basis[D];
+                                sh_basis<float>(P::kBasis, vdir, basis);
+#pragma unroll
+                                for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
+                            }
+#pragma unroll
+                            for (int c = 0; c < 3; ++c) {
+                                ref[c] = color_ref[slot * 3 + c];
+                                resid[c] = 0.0f;
+                                caccum[c] = 0.0f;
+                            }
+                            light = light1 = 1.0f;
+                            tmin = r.t;
+                            cur.levels = 0;
+                            second = false;
+                            active = true;
+                        } else {
+                            color_out[slot * 3] = bg;
+                            color_out[slot * 3 + 1] = bg;
+                            color_out[slot * 3 + 2] = bg;
+                        }
+                    }
+                }
+            }
+            next += n_idle;
+            continue;
+        }
+        if (n_idle == kMarchThreads) break;
+
+        // ---- walk
+        int32_t q_leaf[kQueue];
+        float q_dt[kQueue];
+        int n = 0;
+        bool broken = false;
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            q_leaf[q] = 0;
+            q_dt[q] = 0.0f;
+            if (active && !broken && r.t < r.tmax) {
+                float delta_t;
+                const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
+                if (v.leaf >= 0) {
+                    q_leaf[q] = (int32_t)v.leaf;
+                    q_dt[q] = delta_t;
+                    advance(r, delta_t);
+                    n = q + 1;
+                } else {
+                    broken = true;
+                }
+            }
+        }
+        // ---- sigma
+        float q_sigma[kQueue];
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q)
+            q_sigma[q] = q < n ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+        // ---- shade list
+        int n_entries = 0;
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            const bool want = q < n && q_sigma[q] > 0.0f;
+            const unsigned long long m = __ballot(want);
+            if (want) {
+                const int e = n_entries + rank_in(m);
+                sh.leaf[e] = q_leaf[q];
+                sh.who[e] = (uint8_t)(lane | (q << 6));
+            }
+            n_entries += __popcll(m);
+        }
+        __syncthreads();
+        shade_entries<P, true>(tr.data, sh, n_entries, lane);
+        __syncthreads();
+        // ---- composite and emit, slot by slot
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            bool emit = false;
+            float gci[3] = {0.f, 0.f, 0.f};
+            float g_sigma = 0.f, h_sigma = 0.f;
+            if (active && q < n && q_sigma[q] > 0.0f) {
+                const float att = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
+                const float weight = light * (1.0f - att);
+                const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+                float col[3];
+#pragma unroll
+                for (int c = 0; c < 3; ++c) col[c] = fma_(s[c], d_rgb_pad, -pad);
+                light *= att;
+                if (!second) {
+                    const float att1 = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
+                    const float weight1 = light1 * (1.0f - att1);
+                    light1 *= att1;
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) {
+                        resid[c] = fma_(weight1, col[c], resid[c]);
+                        caccum[c] = fma_(weight, col[c], caccum[c]);
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) {
+                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                            gci[c] = weight * s[c] * (1.0f - s[c]) * d_rgb_pad;
+                        } else {
+                            gci[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)d_rgb_pad);
+                        }
+                        caccum[c] = fma_(-weight, col[c], caccum[c]);
+                        const float gs = q_dt[q] * r.dscale * fma_(col[c], light, -caccum[c]);
+                        g_sigma += gs * resid[c];
+                        h_sigma += gs * gs;
+                    }
+                    emit = true;
+                }
+            }
+            unsigned long long todo = __ballot(emit);
+            while (todo) {
+                const int leader = __ffsll((long long)todo) - 1;
+                const int32_t leaf_l = __builtin_amdgcn_readlane(q_leaf[q], leader);
+                const unsigned long long same = __ballot(emit && q_leaf[q] == leaf_l);
+                todo &= ~same;
+                float* g = grad_data + (int64_t)leaf_l * K;
+                float* h = hess_data + (int64_t)leaf_l * K;
+#pragma unroll
+                for (int e0 = 0; e0 < K; e0 += 64) {
+                    const int e = e0 + lane;
+                    float g_val = 0.0f, h_val = 0.0f;
+                    unsigned long long members = same;
+                    while (members) {
+                        const int k = __ffsll((long long)members) - 1;
+                        members &= members - 1;
+                        const float t0 = read_lane(gci[0], k), t1 = read_lane(gci[1], k), t2 = read_lane(gci[2], k);
+                        const float r0 = read_lane(resid[0], k), r1 = read_lane(resid[1], k),
+                                    r2 = read_lane(resid[2], k);
+                        const float gs = read_lane(g_sigma, k), hs = read_lane(h_sigma, k);
+                        float g_term, h_term;
+                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                            const float tc = e == 0 ? t0 : e == 1 ? t1 : t2;
+                            const float rc = e == 0 ? r0 : e == 1 ? r1 : r2;
+                            g_term = e < 3 ? tc * rc : gs;
+                            h_term = e < 3 ? tc * tc : hs;
+                        } else {
+                            const int c = e / D;
+                            const float b = e < 3 * D ? sh.basis[k * D + (e - c * D)] : 0.0f;
+                            const float gw = b * (c == 0 ? t0 : c == 1 ? t1 : t2);
+                            const float rc = c == 0 ? r0 : c == 1 ? r1 : r2;
+                            g_term = e < 3 * D ? gw * rc : gs;
+                            h_term = e < 3 * D ? gw * gw : hs;
+                        }
+                        g_val += g_term;
+                        h_val += h_term;
+                    }
+                    if (e < K) {
+                        atomicAdd(g + e, g_val);
+                        atomicAdd(h + e, h_val);
+                    }
+                }
+            }
+        }
+        // ---- end of a march
+        if (active && (broken || !(r.t < r.tmax))) {
+            if (!second && !broken) {
+#pragma unroll
+                for (int c = 0; c < 3; ++c) {
+                    resid[c] += fma_(light1, bg, -ref[c]);
+                    caccum[c] = fma_(light, bg, caccum[c]);
+                }
+                light = 1.0f;
+                r.t = tmin;
+                second = true;
+            } else {
+#pragma unroll
+                for (int c = 0; c < 3; ++c) color_out[slot * 3 + c] = resid[c] + ref[c];
+                active = false;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // visit counters
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ unsigned long long wave_sum(unsigned long long v) {

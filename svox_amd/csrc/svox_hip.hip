@@ -289,6 +289,38 @@ int64_t data_bytes(const SvoxTreeSpec* t) {
     return t->capacity * t->N * t->N * t->N * t->data_dim * esz;
 }
 
+template <class Source, typename T>
+void launch_se_grad(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, int out_dim,
+                    const void* color_ref, void* color_out, void* grad, void* hess, hipStream_t stream) {
+    const int64_t items = total_items_of(src);
+    if constexpr (sizeof(T) == 4) {
+        const int D = fast_basis(tree, opt);
+        if (D >= 0) {
+            const unsigned blocks = blocks_for(items, src.per_wave);
+            SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source>), dim3(blocks), dim3(kMarchThreads),
+                                                       0, stream, make_tree<float>(tree), src, *opt,
+                                                       (const float*)color_ref, (float*)color_out, (float*)grad,
+                                                       (float*)hess));
+            return;
+        }
+    }
+    hipLaunchKernelGGL((se_grad_generic_kernel<T, Source>), dim3(blocks_for(items, kMarchThreads)),
+                       dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (const T*)color_ref,
+                       (T*)color_out, (T*)grad, (T*)hess);
+}
+
+// shared argument checks and zero-fills of the two squared-error entry points
+int se_grad_prepare(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, void* grad, void* hess, int* od,
+                    hipStream_t stream) {
+    int rc = check_render(tree, opt, od);
+    if (rc) return rc;
+    if (*od > 4) return fail(SVOX_ERR_BAD_SHAPE, "Tree's output dim cannot be > 4 for se_grad");
+    if (!grad || !hess) return fail(SVOX_ERR_NULL_POINTER, "grad_out / hessdiag_out is NULL");
+    rc = zero_fill(grad, data_bytes(tree), stream);
+    if (rc) return rc;
+    return zero_fill(hess, data_bytes(tree), stream);
+}
+
 }  // namespace
 
 #pragma GCC visibility push(default)
@@ -491,6 +523,45 @@ int svox_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCamera
                                       const SvoxRenderOptions* opt, const void* grad_output, void* grad_data_out,
                                       int32_t accumulate, void* stream) {
     return svox_volume_render_images_backward(tree, cam, 1, 12, opt, grad_output, grad_data_out, accumulate, stream);
+}
+
+int svox_se_grad(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
+                 const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out, void* stream) {
+    int od;
+    int rc = check_rays(rays);
+    if (rc) return rc;
+    rc = se_grad_prepare(tree, opt, grad_out, hessdiag_out, &od, (hipStream_t)stream);
+    if (rc) return rc;
+    if (rays->n_rays == 0) return SVOX_OK;
+    if (!color_ref || !color_out) return fail(SVOX_ERR_NULL_POINTER, "color_ref / color_out is NULL");
+    if (tree->dtype == SVOX_F32)
+        launch_se_grad<BatchSource<float>, float>(tree, batch_source<float>(rays, true), opt, od, color_ref,
+                                                  color_out, grad_out, hessdiag_out, (hipStream_t)stream);
+    else
+        launch_se_grad<BatchSource<double>, double>(tree, batch_source<double>(rays, true), opt, od, color_ref,
+                                                    color_out, grad_out, hessdiag_out, (hipStream_t)stream);
+    return check_launch("se_grad");
+}
+
+int svox_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
+                       const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out, void* stream) {
+    int od;
+    int rc = check_camera(cam, 1, 12);
+    if (rc) return rc;
+    rc = se_grad_prepare(tree, opt, grad_out, hessdiag_out, &od, (hipStream_t)stream);
+    if (rc) return rc;
+    if (cam->width == 0 || cam->height == 0) return SVOX_OK;
+    if (!color_ref || !color_out) return fail(SVOX_ERR_NULL_POINTER, "color_ref / color_out is NULL");
+    if (tree->dtype == SVOX_F32) {
+        const auto src = image_source<float>(cam, 1, 12);
+        launch_se_grad<ImageSource<float>, float>(tree, src, opt, od, color_ref, color_out, grad_out, hessdiag_out,
+                                                  (hipStream_t)stream);
+    } else {
+        const auto src = image_source<double>(cam, 1, 12);
+        launch_se_grad<ImageSource<double>, double>(tree, src, opt, od, color_ref, color_out, grad_out,
+                                                    hessdiag_out, (hipStream_t)stream);
+    }
+    return check_launch("se_grad_persp");
 }
 
 int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCameraSpec* cam,

@@ -161,10 +161,20 @@ class VolumeRenderer(nn.Module):
         return fn.apply(self.tree.data, self.tree._spec(), cam, self._get_options(fast))
 
     def se_grad(self, rays, colors):
-        raise NotImplementedError("se_grad is not part of this build")
+        """Rendered colour plus gradient and Hessian diagonal (Gauss-Newton: squared Jacobian rows) of
+        0.5 * sum (render - colors)^2 for a ray batch -> (colors (B, rgb_dim), grad, diag_hessian), the
+        last two shaped like tree.data.  rgb_dim must be <= 4.  svox/renderer.py:324-348."""
+        self._require_gpu(True, "VolumeRenderer.se_grad")
+        return _C.se_grad(self.tree._spec(), _rays_spec_from_rays(rays), colors, self._get_options(False))
 
     def se_grad_persp(self, c2w, colors, width=800, height=800, fx=1111.111, fy=None):
-        raise NotImplementedError("se_grad_persp is not part of this build")
+        """Image version of se_grad: colors is (height, width, rgb_dim).  svox/renderer.py:350-385."""
+        self._require_gpu(True, "VolumeRenderer.se_grad_persp")
+        if fy is None:
+            fy = fx
+        cam = _make_camera_spec(c2w.to(dtype=self.tree.data.dtype, device=self.tree.data.device).contiguous(),
+                                width, height, fx, fy)
+        return _C.se_grad_persp(self.tree._spec(), cam, self._get_options(False), colors)
 
     @staticmethod
     def persp_rays(c2w, width=800, height=800, fx=1111.111, fy=None):

@@ -466,3 +466,104 @@ def test_pathological_rays_terminate():
         assert stats["samples"] < 10000
         grad = oracle.volume_render_backward(ot, o, d, d, options(tree, step_size=step), np.ones((5, 3), np.float32))
         assert grad.shape == tuple(tree.data.shape)
+
+
+# ------------------------------------------------------------------------------------------
+# squared-error gradient and Gauss-Newton Hessian diagonal (se_grad)
+# ------------------------------------------------------------------------------------------
+def _se_case(fmt, dtype=torch.float64, n_rays=24, seed=11):
+    tree = svox.N3Tree(data_format=fmt, init_refine=1, dtype=dtype)
+    g = torch.Generator().manual_seed(seed)
+    tree.data.data.normal_(generator=g)
+    tree.data.data[..., -1] = tree.data.data[..., -1].abs() * 3
+    tree.data.data[0, 0, 0, 1, -1] = 0.0            # an empty leaf among the others
+    rays = synth.sphere_rays(n_rays, seed=seed, dtype=dtype)
+    ref = torch.rand(n_rays, 3, generator=g, dtype=dtype)
+    return tree, rays, ref
+
+
+@pytest.mark.parametrize("fmt,basis", [("RGBA", -1), ("SH4", 4)])
+def test_se_grad_is_the_gradient_and_jacobian_row_norm_of_the_squared_error(fmt, basis):
+    """colour = render; grad = d/d(data) of 0.5 |render - ref|^2; hessdiag = sum over rays and channels
+    of (d render_c / d data)^2 -- both from torch.autograd through the fallback restatement."""
+    tree, rays, ref = _se_case(fmt)
+    opt = options(tree, step_size=1e-3)
+    ot = oracle.Tree.from_n3tree(tree)
+    colour, grad, hess = oracle.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, opt)
+
+    data = tree.data.detach().clone().requires_grad_(True)
+    out = torch_fallback.render(data, tree.child, tree.parent_depth, tree.invradius, tree.offset, rays.origins,
+                                rays.dirs, rays.viewdirs, basis)
+    assert np.abs(colour - out.detach().numpy()).max() < 2e-6
+    assert np.abs(colour - oracle.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)).max() < 1e-6
+    (want_grad,) = torch.autograd.grad(0.5 * ((out - ref) ** 2).sum(), data, retain_graph=True)
+    want_hess = torch.zeros_like(data)
+    for r in range(out.shape[0]):
+        for c in range(3):
+            (row,) = torch.autograd.grad(out[r, c], data, retain_graph=True)
+            want_hess += row ** 2
+    assert np.abs(grad - want_grad.numpy()).max() <= 1e-4 * np.abs(want_grad.numpy()).max()
+    assert np.abs(hess - want_hess.numpy()).max() <= 1e-4 * np.abs(want_hess.numpy()).max()
+    assert (hess >= 0).all() and hess[..., -1].max() > 0 and hess[..., 0].max() > 0
+
+
+def test_se_grad_agrees_with_the_backward_march_on_the_residual():
+    for fmt in ("RGBA", "SH9"):
+        tree = synth.dense_tree(2, fmt, seed=21, sigma="lognormal", coeff_std=0.7)
+        rays = synth.sphere_rays(500, seed=8)
+        ref = torch.rand(500, 3, generator=torch.Generator().manual_seed(2))
+        ot = oracle.Tree.from_n3tree(tree)
+        opt = options(tree, step_size=1e-3, rgb_padding=0.02, background_brightness=0.7)
+        colour, grad, hess = oracle.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, opt)
+        want = oracle.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, colour - ref.numpy())
+        assert np.abs(grad - want).max() <= 2e-5 * np.abs(want).max()
+        # thresholds play no part (rt_kernel.cu:536, 584, 651 test sigma > 0 only)
+        again = oracle.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, options(
+            tree, step_size=1e-3, rgb_padding=0.02, background_brightness=0.7, fast=True))
+        assert all(np.array_equal(a, b) for a, b in zip((colour, grad, hess), again))
+        # rays that miss: background colour, no gradient (rt_kernel.cu:504-510)
+        c_miss, g_miss, h_miss = oracle.se_grad(ot, rays.origins, -rays.dirs, rays.viewdirs, ref, opt)
+        assert np.all(c_miss == np.float32(0.7)) and not g_miss.any() and not h_miss.any()
+
+
+def test_se_grad_softplus_terms_follow_from_the_plain_ones():
+    """With density_softplus the density entries are the plain ones (on a tree that stores
+    softplus(raw) directly) times sigmoid(raw - 1), and the Hessian entry gains
+    sigmoid' * sum_c d(render_c)/d(sigma), which the backward march with grad_out = 1 gives
+    (rt_kernel.cu:683-695)."""
+    tree, rays, ref = _se_case("SH4", seed=13)
+    raw = tree.data.data[..., -1].clone()
+    soft = torch.log1p(torch.exp(raw - 1))
+    plain = svox.N3Tree(data_format="SH4", init_refine=1, dtype=torch.float64)
+    plain.data.data.copy_(tree.data.data)
+    # what the march sees as sigma: logf(1 + expf(raw - 1)) evaluated in single precision
+    seen = np.log((1 + oracle.expf((raw - 1).numpy().astype(np.float32))).astype(np.float32)).astype(np.float64)
+    assert np.abs(seen - soft.numpy()).max() < 1e-6
+    plain.data.data[..., -1] = torch.from_numpy(seen)
+    o, d, v = rays.origins, rays.dirs, rays.viewdirs
+    c_s, g_s, h_s = oracle.se_grad(oracle.Tree.from_n3tree(tree), o, d, v, ref, options(tree, density_softplus=True))
+    c_p, g_p, h_p = oracle.se_grad(oracle.Tree.from_n3tree(plain), o, d, v, ref, options(plain))
+    ones = oracle.volume_render_backward(oracle.Tree.from_n3tree(plain), o, d, v, options(plain),
+                                         np.ones((o.shape[0], 3)))
+    # (numpy's float32 log and the C library's logf may differ in the last place)
+    assert np.allclose(c_s, c_p, rtol=0, atol=1e-6)
+    assert np.allclose(g_s[..., :-1], g_p[..., :-1], rtol=1e-5, atol=1e-8)
+    sg = 1 / (1 + np.exp(-(raw.numpy() - 1)))
+    live = seen > 0
+    assert np.allclose(g_s[..., -1][live], (g_p[..., -1] * sg)[live], rtol=1e-5, atol=1e-9)
+    want_h = h_p[..., -1] * sg * sg + ones[..., -1] * sg * (1 - sg)
+    assert np.allclose(h_s[..., -1][live], want_h[live], rtol=1e-5, atol=1e-9)
+
+
+def test_se_grad_image_is_se_grad_on_the_image_rays():
+    tree = synth.dense_tree(2, "SH4", seed=5)
+    c2w = synth.look_at_pose(torch.tensor([0.5, 0.5, 0.5]) + 2.5 * torch.tensor([0.3, -0.5, 0.8]))
+    ot = oracle.Tree.from_n3tree(tree)
+    opt = options(tree, step_size=1e-3)
+    W, H, fx = 20, 14, 25.0
+    ref = torch.rand(H, W, 3, generator=torch.Generator().manual_seed(4))
+    colour, grad, hess = oracle.se_grad_image(ot, c2w, fx, fx, W, H, ref, opt)
+    o, d, v = oracle.image_rays(ot, c2w, fx, fx, W, H, opt)
+    # image_rays returns tree-space origins; this tree's transform is the identity
+    c2, g2, h2 = oracle.se_grad(ot, o, d, v, ref.reshape(-1, 3), opt)
+    assert np.array_equal(colour.reshape(-1, 3), c2) and np.array_equal(grad, g2) and np.array_equal(hess, h2)
