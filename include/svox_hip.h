@@ -201,6 +201,17 @@ int svox_se_grad(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxR
 int svox_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
                        const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out, void* stream);
 
+/* grid_weight_render(data, CameraSpec&, RenderOptions&, offset, scaling) -> {grid_weight, grid_hit};
+ * svox.cpp:38-40, 120, rt_kernel.cu:1174-1203 (kernel :898-1003).
+ * Marches the pixel rays of one camera through a dense density grid data (reso, reso, reso): per
+ * cell with sigma > opt->sigma_thresh, grid_weight_out holds the largest compositing weight any ray
+ * gave the cell and grid_hit_out the number of such visits.  offset and scaling are 3 scalars each
+ * in device memory (world -> grid coordinates).  Both outputs are zero-filled by the library and
+ * must be 16-byte aligned.  `dtype` is the scalar type of data, offset, scaling, c2w and outputs. */
+int svox_grid_weight_render(const void* data, int32_t reso, int32_t dtype, const SvoxCameraSpec* cam,
+                            const SvoxRenderOptions* opt, const void* offset, const void* scaling,
+                            void* grid_weight_out, void* grid_hit_out, void* stream);
+
 /* get_out_data_dim, rt_kernel.cu:1009-1015.  Returns -1 for an invalid combination. */
 int svox_out_data_dim(int32_t format, int32_t basis_dim, int32_t data_dim);
 

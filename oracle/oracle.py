@@ -55,6 +55,8 @@ def lib():
             "oracle_volume_render_image_backward": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_int32, S, c_int32]),
             "oracle_se_grad": (ctypes.c_int, [T, R, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int32]),
             "oracle_se_grad_image": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int32]),
+            "oracle_grid_weight_render": (ctypes.c_int, [c_void_p, c_int32, c_int32, C, O, c_void_p, c_void_p, c_void_p,
+                                                         c_void_p]),
             "oracle_image_rays": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_void_p]),
             "oracle_trace_visits": (c_int64, [T, R, c_int64, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int64]),
         }
@@ -286,6 +288,21 @@ def se_grad_image(tree, c2w, fx, fy, width, height, colors, opt, n_threads=1):
     _check(lib().oracle_se_grad_image(ctypes.byref(s), ctypes.byref(c), ctypes.byref(o), _ptr(ref), _ptr(out),
                                       _ptr(grad), _ptr(hess), n_threads), "se_grad_image")
     return out, grad, hess
+
+
+def grid_weight_render(data, c2w, fx, fy, width, height, opt, offset, scaling):
+    """(grid_weight, grid_hit) of a dense (reso, reso, reso) density grid seen from one camera."""
+    d = _np(data)
+    assert d.ndim == 3 and d.shape[0] == d.shape[1] == d.shape[2]
+    c = _np(c2w, d.dtype)
+    cam = _abi.CameraSpecC(_ptr(c), float(fx), float(fy), int(width), int(height))
+    off, sc = _np(offset, d.dtype), _np(scaling, d.dtype)
+    o = _opt(opt)
+    weight, hit = np.empty_like(d), np.empty_like(d)
+    _check(lib().oracle_grid_weight_render(_ptr(d), d.shape[0], 0 if d.dtype == np.float32 else 1, ctypes.byref(cam),
+                                           ctypes.byref(o), _ptr(off), _ptr(sc), _ptr(weight), _ptr(hit)),
+           "grid_weight_render")
+    return weight, hit
 
 
 def image_rays(tree, c2w, fx, fy, width, height, opt):

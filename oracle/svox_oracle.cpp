@@ -818,6 +818,63 @@ int render_backward_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
     return SVOX_OK;
 }
 
+// grid_trace_ray + grid_weight_render_kernel, rt_kernel.cu:898-1003: march through a dense
+// reso^3 density grid; per visited cell with sigma > sigma_thresh the largest compositing weight any
+// ray gave it (atomicMax) and the number of such visits.
+template <typename T>
+int grid_weight_impl(const void* data_v, int reso, const SvoxCameraSpec* cam,
+                     const SvoxRenderOptions* opt, const void* offset_v, const void* scaling_v,
+                     void* weight_v, void* hit_v) {
+    const T* data = (const T*)data_v;
+    T* grid_weight = (T*)weight_v;
+    T* grid_hit = (T*)hit_v;
+    const size_t cells = (size_t)reso * reso * reso;
+    std::memset(grid_weight, 0, sizeof(T) * cells);
+    std::memset(grid_hit, 0, sizeof(T) * cells);
+    TreeView<T> tr{};   // only the transform is used
+    for (int i = 0; i < 3; ++i) {
+        tr.offset[i] = ((const T*)offset_v)[i];
+        tr.scaling[i] = ((const T*)scaling_v)[i];
+    }
+    const int64_t n = (int64_t)cam->width * cam->height;
+    for (int64_t pix = 0; pix < n; ++pix) {
+        T origin[3], dir[3], vdir[3];
+        pixel_ray(tr, *cam, *opt, pix, origin, dir, vdir);
+        const T delta_scale = delta_scale_of(tr.scaling, dir);
+        T invdir[3], tmin, tmax;
+        for (int i = 0; i < 3; ++i) invdir[i] = (T)(1.0 / ((double)dir[i] + 1e-9));
+        dda_unit(origin, invdir, &tmin, &tmax);
+        if (tmax < T(0) || tmin > tmax) continue;
+        T light = T(1), t = tmin;
+        const T cube_sz = (T)reso;
+        while (t < tmax) {
+            T pos[3];
+            for (int j = 0; j < 3; ++j) pos[j] = fma_(t, dir[j], origin[j]);
+            clamp_coord(pos);
+            int32_t uvw[3];
+            for (int j = 0; j < 3; ++j) {
+                pos[j] *= (T)reso;
+                uvw[j] = (int32_t)std::floor(pos[j]);
+                pos[j] -= (T)uvw[j];
+            }
+            const int32_t node_id = uvw[0] * reso * reso + uvw[1] * reso + uvw[2];
+            T s0, s1;
+            dda_unit(pos, invdir, &s0, &s1);
+            const T delta_t = (s1 - s0) / cube_sz + (T)opt->step_size;
+            const T sigma = data[node_id];
+            if (sigma > (T)opt->sigma_thresh) {
+                const T att = exp_sp<T>(-delta_t * delta_scale * sigma);
+                const T weight = light * (T(1) - att);
+                light *= att;
+                grid_weight[node_id] = (T)std::fmax((float)weight, (float)grid_weight[node_id]);
+                grid_hit[node_id] += T(1);
+            }
+            t = advance_t(t, delta_t, tmax);
+        }
+    }
+    return SVOX_OK;
+}
+
 // se_grad / se_grad_persp, rt_kernel.cu:1111-1173
 template <typename T>
 int se_grad_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCameraSpec* cam,
@@ -1085,6 +1142,20 @@ int oracle_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
     return tree->dtype == SVOX_F32
                ? se_grad_impl<float>(tree, nullptr, cam, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads)
                : se_grad_impl<double>(tree, nullptr, cam, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads);
+}
+
+// grid_weight_render, rt_kernel.cu:1174-1203.  data, grid_weight_out and grid_hit_out are
+// (reso, reso, reso); offset and scaling are 3 scalars each.
+int oracle_grid_weight_render(const void* data, int32_t reso, int32_t dtype,
+                              const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
+                              const void* offset, const void* scaling, void* grid_weight_out,
+                              void* grid_hit_out) {
+    if (!data || !cam || !cam->c2w || !opt || !offset || !scaling || !grid_weight_out || !grid_hit_out)
+        return SVOX_ERR_NULL_POINTER;
+    if (reso < 1 || reso > 1290) return SVOX_ERR_BAD_SHAPE;   // int32 cell ids
+    return dtype == SVOX_F32
+               ? grid_weight_impl<float>(data, reso, cam, opt, offset, scaling, grid_weight_out, grid_hit_out)
+               : grid_weight_impl<double>(data, reso, cam, opt, offset, scaling, grid_weight_out, grid_hit_out);
 }
 
 // The rays the image kernels trace, after cam2world / NDC / world->tree: origins, dirs, vdirs are

@@ -446,6 +446,32 @@ def se_grad_persp(tree, cam, opt, color):
     return result, grad, hessdiag
 
 
+def grid_weight_render(data, cam, opt, offset, scaling):
+    """[grid_weight, grid_hit], both zeros_like(data) + per-cell max weight / visit count of one
+    camera's rays through the dense (reso, reso, reso) density grid `data`; svox.cpp:120,
+    rt_kernel.cu:1174-1203."""
+    _check_input(data, "data")
+    if not data.is_floating_point():
+        raise RuntimeError("data must be a floating point tensor")
+    if data.dim() != 3 or not (data.shape[0] == data.shape[1] == data.shape[2]):
+        raise RuntimeError("data must be a cubic (reso, reso, reso) grid")
+    for name, x in (("offset", offset), ("scaling", scaling)):
+        _check_input(x, name)
+        _same_dtype(x, data.dtype, name)
+        if x.numel() != 3:
+            raise RuntimeError(f"{name} must have 3 elements")
+    cspec = _pack_camera(cam, data.dtype)
+    grid_weight = torch.empty_like(data)
+    grid_hit = torch.empty_like(data)
+    copt = opt._pack()
+    with torch.cuda.device(data.device):
+        _call("svox_grid_weight_render", data.data_ptr(), int(data.shape[0]),
+              _abi.SVOX_F32 if data.dtype == torch.float32 else _abi.SVOX_F64, ctypes.byref(cspec),
+              ctypes.byref(copt), offset.data_ptr(), scaling.data_ptr(), grid_weight.data_ptr(),
+              grid_hit.data_ptr(), _stream(data.device))
+    return [grid_weight, grid_hit]
+
+
 def volume_render_stats(tree, rays_or_cam, opt):
     """Visit counts of one launch (dict); `rays_or_cam` is a RaysSpec or a CameraSpec."""
     spec = _pack_tree(tree)

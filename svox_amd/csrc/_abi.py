@@ -125,6 +125,9 @@ SIGNATURES = {
     "svox_se_grad_image": (
         ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p, c_void_p,
                        c_void_p]),
+    "svox_grid_weight_render": (
+        ctypes.c_int, [c_void_p, c_int32, c_int32, P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p,
+                       c_void_p, c_void_p]),
     "svox_volume_render_stats": (
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p]),
 }

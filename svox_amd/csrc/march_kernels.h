@@ -1299,6 +1299,57 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
 }
 
 // ------------------------------------------------------------------------------------------------
+// dense-grid weight render
+// ------------------------------------------------------------------------------------------------
+// grid_trace_ray + grid_weight_render_kernel, rt_kernel.cu:898-1003: one pixel ray per lane through a
+// dense reso^3 density grid; per cell with sigma > sigma_thresh the largest compositing weight any
+// ray gave it and the number of visits.
+template <typename T>
+__global__ __launch_bounds__(kMarchThreads) void grid_weight_kernel(const T* __restrict__ data, int reso,
+                                                                    ImageSource<T> src, SvoxRenderOptions opt,
+                                                                    const T* __restrict__ offset_p,
+                                                                    const T* __restrict__ scaling_p,
+                                                                    T* __restrict__ grid_weight,
+                                                                    T* __restrict__ grid_hit) {
+    T offset[3], scaling[3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        offset[i] = offset_p[i];
+        scaling[i] = scaling_p[i];
+    }
+    T origin[3], dir[3], vdir[3];
+    const int64_t item = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
+    if (src.fetch_item(item, opt, offset, scaling, origin, dir, vdir) < 0) return;
+    RayState<T> r;
+    if (!setup_ray(r, origin, dir, scaling)) return;
+    const T cube_sz = (T)reso;
+    T light = T(1);
+    while (r.t < r.tmax) {
+        T pos[3];
+        int32_t uvw[3];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            pos[j] = clamp01(fma_(r.t, r.d[j], r.o[j])) * cube_sz;
+            uvw[j] = (int32_t)floor_(pos[j]);
+            pos[j] -= (T)uvw[j];
+        }
+        const int32_t node_id = uvw[0] * reso * reso + uvw[1] * reso + uvw[2];
+        T s0, s1;
+        dda_unit(pos, r.inv, &s0, &s1);
+        const T delta_t = (s1 - s0) / cube_sz + (T)opt.step_size;
+        const T sigma = data[node_id];
+        if (sigma > (T)opt.sigma_thresh) {
+            const T att = exp_sp<T>(-delta_t * r.dscale * sigma);
+            const T weight = light * (T(1) - att);
+            light *= att;
+            atomic_max_float(grid_weight + node_id, weight);
+            atomicAdd(grid_hit + node_id, T(1));
+        }
+        advance(r, delta_t);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // visit counters
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ unsigned long long wave_sum(unsigned long long v) {

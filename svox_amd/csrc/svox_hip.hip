@@ -564,6 +564,38 @@ int svox_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, cons
     return check_launch("se_grad_persp");
 }
 
+int svox_grid_weight_render(const void* data, int32_t reso, int32_t dtype, const SvoxCameraSpec* cam,
+                            const SvoxRenderOptions* opt, const void* offset, const void* scaling,
+                            void* grid_weight_out, void* grid_hit_out, void* stream) {
+    if (!data || !opt || !offset || !scaling || !grid_weight_out || !grid_hit_out)
+        return fail(SVOX_ERR_NULL_POINTER, "grid_weight_render: NULL argument");
+    if (dtype != SVOX_F32 && dtype != SVOX_F64) return fail(SVOX_ERR_BAD_DTYPE, "dtype must be SVOX_F32 or SVOX_F64");
+    // cell ids are 32-bit, as in the reference (reso^3 < 2^31)
+    if (reso < 1 || reso > 1290) return fail(SVOX_ERR_BAD_SHAPE, "grid resolution must be in [1, 1290]");
+    int rc = check_camera(cam, 1, 12);
+    if (rc) return rc;
+    const int64_t bytes = (int64_t)reso * reso * reso * (dtype == SVOX_F32 ? 4 : 8);
+    rc = zero_fill(grid_weight_out, bytes, (hipStream_t)stream);
+    if (rc) return rc;
+    rc = zero_fill(grid_hit_out, bytes, (hipStream_t)stream);
+    if (rc) return rc;
+    if (cam->width == 0 || cam->height == 0) return SVOX_OK;
+    if (dtype == SVOX_F32) {
+        const auto src = image_source<float>(cam, 1, 12);
+        hipLaunchKernelGGL((grid_weight_kernel<float>), dim3(blocks_for(total_items_of(src), kMarchThreads)),
+                           dim3(kMarchThreads), 0, (hipStream_t)stream, (const float*)data, reso, src, *opt,
+                           (const float*)offset, (const float*)scaling, (float*)grid_weight_out,
+                           (float*)grid_hit_out);
+    } else {
+        const auto src = image_source<double>(cam, 1, 12);
+        hipLaunchKernelGGL((grid_weight_kernel<double>), dim3(blocks_for(total_items_of(src), kMarchThreads)),
+                           dim3(kMarchThreads), 0, (hipStream_t)stream, (const double*)data, reso, src, *opt,
+                           (const double*)offset, (const double*)scaling, (double*)grid_weight_out,
+                           (double*)grid_hit_out);
+    }
+    return check_launch("grid_weight_render");
+}
+
 int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCameraSpec* cam,
                              const SvoxRenderOptions* opt, SvoxMarchStats* stats_out, void* stream) {
     int od;

@@ -567,3 +567,57 @@ def test_se_grad_image_is_se_grad_on_the_image_rays():
     # image_rays returns tree-space origins; this tree's transform is the identity
     c2, g2, h2 = oracle.se_grad(ot, o, d, v, ref.reshape(-1, 3), opt)
     assert np.array_equal(colour.reshape(-1, 3), c2) and np.array_equal(grad, g2) and np.array_equal(hess, h2)
+
+
+# ------------------------------------------------------------------------------------------
+# dense-grid weight render (grid_weight_render)
+# ------------------------------------------------------------------------------------------
+def test_grid_weight_render_axis_aligned_closed_form():
+    """One pixel looking straight down -z through a uniform grid: 8 cells, step lengths
+    1/8 + step, 1/8, 1/8, ...; weights are the compositing weights; one hit per cell."""
+    reso, s, step = 8, 3.0, 1e-3
+    data = np.full((reso, reso, reso), s, np.float32)
+    c2w = torch.tensor([[1.0, 0, 0, 0.3], [0, 1, 0, 0.6], [0, 0, 1, 2.0]])
+    tree = svox.N3Tree(data_format="RGBA")
+    opt = options(tree, step_size=step)
+    weight, hit = oracle.grid_weight_render(data, c2w, 1e9, 1e9, 1, 1, opt, np.zeros(3), np.ones(3))
+    want_hit = np.zeros_like(data)
+    want_hit[2, 4, :] = 1
+    assert np.array_equal(hit, want_hit)
+    first = np.exp(-s * (1 / reso + step))
+    later = np.exp(-s / reso)
+    want = np.array([1 - first] + [first * later ** (k - 1) * (1 - later) for k in range(1, reso)])
+    assert np.abs(weight[2, 4, ::-1] - want).max() < 1e-5
+    assert weight.sum() == weight[2, 4].sum()
+    # a threshold above the density: nothing is recorded
+    weight, hit = oracle.grid_weight_render(data, c2w, 1e9, 1e9, 1, 1, options(tree, step_size=step, sigma_thresh=5.0),
+                                            np.zeros(3), np.ones(3))
+    assert not weight.any() and not hit.any()
+
+
+def test_grid_weight_render_equals_max_accumulation_on_the_dense_tree():
+    """A dense 16^3 tree is the same volume as its 16^3 grid of leaf densities: the tree march with a
+    max-accumulator gives, leaf by leaf, what the grid march gives cell by cell."""
+    tree = svox.N3Tree(data_format="RGBA", init_refine=3, radius=0.7, center=[0.4, 0.5, 0.6])
+    g = torch.Generator().manual_seed(3)
+    tree.data.data.normal_(generator=g)
+    tree.data.data[..., -1] = (tree.data.data[..., -1] * 4).clamp_min(0)     # about half the cells empty
+    reso = 16
+    ax = (torch.arange(reso) + 0.5) / reso
+    centres = torch.stack(torch.meshgrid(ax, ax, ax, indexing="ij"), -1).reshape(-1, 3)
+    ot = oracle.Tree.from_n3tree(tree, world=False)
+    values, ids = oracle.query_vertical(ot, centres)
+    sigma_grid = values[:, -1].reshape(reso, reso, reso)
+    c2w = synth.look_at_pose(torch.tensor([0.4, 0.5, 0.6]) + 2.0 * torch.tensor([0.5, 0.3, 0.8]),
+                             target=torch.tensor([0.4, 0.5, 0.6]))
+    opt = options(tree, step_size=1e-3, sigma_thresh=0.5)
+    W, H, fx = 40, 30, 30.0
+    weight, hit = oracle.grid_weight_render(sigma_grid, c2w, fx, fx, W, H, opt, tree.offset, tree.invradius)
+    ow = oracle.Tree.from_n3tree(tree)
+    ow.weight_accum = np.zeros(tree.child.shape, np.float32)
+    ow.weight_accum_max = True
+    _, stats = oracle.volume_render_image(ow, c2w, fx, fx, W, H, opt, want_stats=True)
+    assert stats["samples_shaded"] > 1000
+    assert np.array_equal(weight.reshape(-1), ow.weight_accum.reshape(-1)[ids])
+    assert hit.sum() == stats["samples_shaded"]
+    assert not hit[sigma_grid <= 0.5].any() and not weight[sigma_grid <= 0.5].any()
