@@ -462,7 +462,9 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
 //             stop_thresh and writes the pixel when the ray ends.
 // A ray that stops early has walked at most kQueue - 1 leaves too far; the values are the same as
 // when every leaf is shaded on the spot.
-template <class P, class Source>
+// kAccum: the compositing weight of every shaded leaf is also added to (or maximised into)
+// tr.weight_accum at the leaf's cell index (rt_kernel.cu:298-304).
+template <class P, class Source, bool kAccum>
 __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<float> tr, Source src,
                                                                        SvoxRenderOptions opt,
                                                                        float* __restrict__ out) {
@@ -580,6 +582,12 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
 #pragma unroll
                     for (int c = 0; c < 3; ++c) acc[c] = fma_(weight, fma_(s[c], d_rgb_pad, -pad), acc[c]);
                     light *= att;
+                    if constexpr (kAccum) {
+                        if (tr.weight_accum_max)
+                            atomic_max_float(tr.weight_accum + q_leaf[q], weight);
+                        else
+                            atomicAdd(tr.weight_accum + q_leaf[q], weight);
+                    }
                     if (light <= stop_thresh) {
                         const float scale = (float)(1.0 / (1.0 - (double)light));
 #pragma unroll

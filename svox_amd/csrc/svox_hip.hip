@@ -166,7 +166,7 @@ int check_rays(const SvoxRaysSpec* rays) {
 
 // default options on an fp32 octree whose record matches the format: the specialised kernels
 int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
-    if (!octree_fast_ok(tree) || tree->weight_accum || opt->density_softplus) return -1;
+    if (!octree_fast_ok(tree) || opt->density_softplus) return -1;
     if (opt->format == SVOX_FORMAT_RGBA) return tree->data_dim == 4 ? 0 : -1;
     if (opt->format != SVOX_FORMAT_SH) return -1;
     const int D = opt->basis_dim;
@@ -255,9 +255,15 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
-            SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source>), dim3(blocks),
-                                                       dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                       src, *opt, (float*)out));
+            if (tree->weight_accum) {
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, true>), dim3(blocks),
+                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                           src, *opt, (float*)out));
+            } else {
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, false>), dim3(blocks),
+                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                           src, *opt, (float*)out));
+            }
             return;
         }
     }

@@ -160,24 +160,37 @@ def test_generic_options_double_and_lobes(gpu, oracle_mod):
         assert ok, (name, err)
 
 
-def test_weight_accumulation(gpu, oracle_mod):
-    tree = synth.dense_tree(2, "RGBA", seed=14)
-    rays = synth.sphere_rays(500, seed=2)
-    opt = options(tree)
-    for op in ("sum", "max"):
-        ot = oracle_mod.Tree.from_n3tree(tree)
-        ot.weight_accum = np.zeros(tree.child.shape, dtype=np.float32)
-        ot.weight_accum_max = op == "max"
-        oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
-        dev = on_gpu(tree, gpu)
-        renderer = svox.VolumeRenderer(dev)
-        with dev.accumulate_weights(op=op) as accum:
-            renderer(svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu)))
-            got = accum.value.cpu().numpy()
-        if op == "max":
-            assert np.array_equal(got, ot.weight_accum)
-        else:
-            assert np.abs(got - ot.weight_accum).max() <= 1e-5 * max(1.0, np.abs(ot.weight_accum).max())
+@pytest.mark.parametrize("generic", [0, 1])
+def test_weight_accumulation(gpu, oracle_mod, generic):
+    """accumulate_weights (sum / max) through the renderer, batch and image, thresholds and early stop
+    included: the octree kernels and the generic ones against the oracle."""
+    cases = [(synth.dense_tree(2, "RGBA", seed=14), synth.sphere_rays(500, seed=2), False),
+             (synth.shell_tree(depth=6, n_spheres=6, data_format="SH9", seed=4), synth.sphere_rays(4000, seed=3), True)]
+    c2w = synth.orbit_poses(1, seed=6, radius=2.5)[0]
+    W, H, fx = 70, 50, 60.0
+    for tree, rays, fast in cases:
+        opt = options(tree, fast=fast)
+        for op in ("sum", "max"):
+            ot = oracle_mod.Tree.from_n3tree(tree)
+            ot.weight_accum = np.zeros(tree.child.shape, dtype=np.float32)
+            ot.weight_accum_max = op == "max"
+            oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+            oracle_mod.volume_render_image(ot, c2w, fx, fx, W, H, opt)
+            assert ot.weight_accum.max() > 0
+            dev = on_gpu(tree, gpu)
+            renderer = svox.VolumeRenderer(dev)
+            C.set_debug_flags(generic)
+            try:
+                with dev.accumulate_weights(op=op) as accum:
+                    renderer(svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu)), fast=fast)
+                    renderer.render_persp(c2w.to(gpu), width=W, height=H, fx=fx, fast=fast)
+                    got = accum.value.cpu().numpy()
+            finally:
+                C.set_debug_flags(0)
+            if op == "max":
+                assert np.array_equal(got, ot.weight_accum)
+            else:
+                assert np.abs(got - ot.weight_accum).max() <= 1e-5 * max(1.0, np.abs(ot.weight_accum).max())
 
 
 def test_toy_example_through_python_api(gpu):

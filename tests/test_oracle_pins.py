@@ -621,3 +621,16 @@ def test_grid_weight_render_equals_max_accumulation_on_the_dense_tree():
     assert np.array_equal(weight.reshape(-1), ow.weight_accum.reshape(-1)[ids])
     assert hit.sum() == stats["samples_shaded"]
     assert not hit[sigma_grid <= 0.5].any() and not weight[sigma_grid <= 0.5].any()
+
+
+def test_weight_accumulation_sums_to_the_opacity_of_the_rays():
+    """Colours all sigmoid(0) = 0.5 and a white background: out = 0.5 * sum(w) + (1 - sum(w)), so the
+    accumulator's total must be sum over rays of 2 - 2 * out (rt_kernel.cu:298-304)."""
+    tree = synth.dense_tree(3, "RGBA", seed=2)
+    tree.data.data[..., :-1] = 0.0
+    rays = synth.sphere_rays(300, seed=12)
+    ot = oracle.Tree.from_n3tree(tree)
+    ot.weight_accum = np.zeros(tree.child.shape, np.float32)
+    out = oracle.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, options(tree, background_brightness=1.0))
+    assert abs(ot.weight_accum.sum(dtype=np.float64) - (2 - 2 * out[:, 0].astype(np.float64)).sum()) < 2e-3
+    assert not ot.weight_accum[tree.child.numpy() != 0].any()      # only leaves receive weight
