@@ -173,3 +173,55 @@ def test_full_size_render_properties(gpu):
     g2 = C.volume_render_backward(tree._spec(), spec, opt, 2.0 * go)
     nz = g1.view(-1).abs() > 1e-6
     assert float(((g2.view(-1)[nz] / g1.view(-1)[nz]) - 2.0).abs().max()) < 1e-3
+
+
+def test_config5_depth10_sh25_ndc_against_the_oracle(gpu, oracle_mod):
+    """BASELINE config 5 at full size: depth-10 octree (42 M leaves, 13.5 GB of SH25 records, more than
+    2^31 elements), forward-facing NDC camera 1008x756.  One whole image, its visit counts, its
+    gradient and a million point queries are compared with the CPU oracle."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 100 * 2 ** 30:
+        pytest.skip("needs 100 GB of free device memory")
+    tree = synth.shell_tree(depth=10, data_format="SH25", seed=5, device=gpu, geometry="noise")
+    assert tree.data.numel() > 2 ** 31 and tree.info["leaves"] > 30_000_000
+    tree.invradius.data[:] = 0.5
+    tree.offset.data[:] = 0.5          # NDC cube [-1, 1]^3 -> [0, 1]^3
+    W, H, fx = 1008, 756, 815.0
+    c2w = torch.tensor([[1.0, 0, 0, 0.05], [0, 1, 0, -0.05], [0, 0, 1, 0.25]])
+    r = svox.VolumeRenderer(tree, step_size=5e-4, ndc=svox.NDCConfig(W, H, fx))
+    opt = r._get_options(True)
+    from svox_amd.renderer import _make_camera_spec
+    cam = _make_camera_spec(c2w.to(gpu), W, H, fx, fx)
+    img = C.volume_render_image(tree._spec(), cam, opt)
+    stats = C.volume_render_stats(tree._spec(), cam, opt)
+    print("config 5 stats", stats, flush=True)
+
+    host = oracle_mod.Tree(tree.data.detach().cpu().numpy(), tree.child.cpu().numpy(), tree.parent_depth.cpu().numpy(),
+                           tree.offset.cpu().numpy(), tree.invradius.cpu().numpy())
+    threads = min(16, oracle_mod.max_threads())
+    ref, ref_stats = oracle_mod.volume_render_image(host, c2w, fx, fx, W, H, opt, want_stats=True, n_threads=threads)
+    assert np.array_equal(img.cpu().numpy(), ref)
+    for k in ("rays", "rays_hit", "samples", "samples_shaded", "levels"):
+        assert stats[k] == ref_stats[k], k
+    assert stats["rays_hit"] > 0.9 * W * H and stats["samples_shaded"] > 5_000_000
+
+    # gradient of the whole image (compared on the GPU: the arrays are 13.5 GB each)
+    go = torch.randn(H, W, 3, generator=torch.Generator().manual_seed(1)) * 1e-2
+    grad = C.volume_render_image_backward(tree._spec(), cam, opt, go.to(gpu))
+    ref_grad = torch.from_numpy(oracle_mod.volume_render_image_backward(host, c2w, fx, fx, W, H, opt, go,
+                                                                        n_threads=threads)).to(gpu)
+    floor = float(ref_grad.abs().max()) * 1e-3
+    worst = 0.0
+    for s in range(0, grad.shape[0], 1 << 19):        # in slices, to bound the temporaries
+        a, b = grad[s:s + (1 << 19)], ref_grad[s:s + (1 << 19)]
+        worst = max(worst, float(((a - b).abs() / b.abs().clamp_min(floor)).max()))
+    # an OpenMP oracle adds in a thread-dependent order too; both sides are within 1e-4 of the exact sum
+    assert worst <= 2e-4, worst
+    del grad, ref_grad
+
+    # point queries: values and leaf ids of a million points
+    pts = torch.rand(1_000_000, 3, generator=torch.Generator().manual_seed(2))
+    vals, ids = tree(pts.to(gpu), want_node_ids=True)
+    ref_vals, ref_ids = oracle_mod.query_vertical(host, pts)
+    assert np.array_equal(ids.cpu().numpy(), ref_ids)
+    assert np.array_equal(vals.detach().cpu().numpy(), ref_vals)
