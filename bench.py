@@ -55,6 +55,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-bwd", action="store_true", help="skip the forward+backward leg")
     ap.add_argument("--no-query", action="store_true", help="skip the point-query leg")
+    ap.add_argument("--no-large", action="store_true", help="skip the depth-10 SH25 NDC leg (BASELINE configs[4])")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (rays would shard "
@@ -276,6 +277,66 @@ def main():
         del qtree, pts, go, leaves
         log(f"[bench] query {query}")
 
+    # ---------------------------------------------------------------- depth-10 SH25 tree, NDC (configs[4])
+    large = None
+    free_bytes, _ = torch.cuda.mem_get_info()
+    if not args.no_large and free_bytes > 100 * 2 ** 30:
+        ltree = synth.shell_tree(depth=10, data_format="SH25", seed=5, device=dev, geometry="noise")
+        ltree.invradius.data[:] = 0.5
+        ltree.offset.data[:] = 0.5
+        LW, LH, lfx = 1008, 756, 815.0
+        lposes = torch.stack([torch.tensor([[1.0, 0, 0, 0.1 * i - 0.15], [0, 1, 0, 0.05 * i - 0.05],
+                                            [0, 0, 1, 0.2 + 0.05 * i]]) for i in range(4)]).to(dev)
+        lrend = svox.VolumeRenderer(ltree, step_size=5e-4, ndc=svox.NDCConfig(LW, LH, lfx))
+        lopt = lrend._get_options(True)
+        lspec = ltree._spec()
+        lstats = [C.volume_render_stats(lspec, _make_camera_spec(p.contiguous(), LW, LH, lfx, lfx), lopt)
+                  for p in lposes]
+        l_bytes = sum(forward_bytes(st, LW * LH, 76, 12) for st in lstats)
+        lcam = _make_camera_spec(lposes, LW, LH, lfx, lfx)
+
+        def ev_time(fn, n=5):
+            fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(n):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / n
+
+        with torch.no_grad():
+            l_ms = ev_time(lambda: C.volume_render_images(lspec, lcam, lopt))
+            Ql = 1 << 24
+            lpts = torch.rand(Ql, 3, generator=torch.Generator().manual_seed(4)).to(dev)
+            lq_ms = ev_time(lambda: C.query_vertical(lspec, lpts), n=3)
+        lgo = torch.randn(Ql, 76, device=dev)
+        lqb_ms = ev_time(lambda: C.query_vertical_backward(lspec, lpts, lgo), n=2)
+        lq_bytes = Ql * (12 + 4 * 10 + 4 * 76 + 4 * 76 + 8)
+        lqb_bytes = Ql * (12 + 4 * 10 + 4 * 76 + 8 * 76) + ltree.data.numel() * 4
+        large = {
+            "workload": "ndc1024_sh25: depth-10 octree, SH25, NDC camera, 4 poses x 1008x756 in one launch, "
+                        "step 5e-4, thresholds 1e-2; queries on 16M uniform points",
+            "nodes": ltree.info["nodes"], "leaves": ltree.info["leaves"],
+            "occupancy": round(ltree.info["occupancy"], 5), "data_gib": round(ltree.data.numel() * 4 / 2 ** 30, 2),
+            "forward": {"mrays_s": round(4 * LW * LH / l_ms / 1e3, 1), "ms": round(l_ms, 4),
+                        "samples_per_ray": round(sum(st["samples"] for st in lstats) / (4 * LW * LH), 2),
+                        "shaded_per_ray": round(sum(st["samples_shaded"] for st in lstats) / (4 * LW * LH), 2),
+                        "algorithmic_gbs": round(l_bytes / l_ms / 1e6, 1),
+                        "frac_of_peak": round(l_bytes / l_ms / 1e6 / PEAK_HBM_GBS, 4)},
+            "query_vertical": {"mpoints_s": round(Ql / lq_ms / 1e3, 1), "ms": round(lq_ms, 4),
+                               "algorithmic_gbs": round(lq_bytes / lq_ms / 1e6, 1),
+                               "frac_of_peak": round(lq_bytes / lq_ms / 1e6 / PEAK_HBM_GBS, 4)},
+            "query_vertical_backward": {"mpoints_s": round(Ql / lqb_ms / 1e3, 1), "ms": round(lqb_ms, 4),
+                                        "algorithmic_gbs": round(lqb_bytes / lqb_ms / 1e6, 1),
+                                        "frac_of_peak": round(lqb_bytes / lqb_ms / 1e6 / PEAK_HBM_GBS, 4),
+                                        "includes": "zero-fill of the 13.5 GB gradient"},
+        }
+        del ltree, lpts, lgo, lspec, lrend, lcam
+        torch.cuda.empty_cache()
+        log(f"[bench] large {large}")
+
     # ---------------------------------------------------------------- CPU baseline (this host)
     cpu = None
     if not args.no_cpu:
@@ -332,6 +393,7 @@ def main():
         "fwd_per_call": per_call,
         "fwd_bwd": fwd_bwd,
         "query": query,
+        "large": large,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)

@@ -8,8 +8,8 @@
 //      wavefront is one contiguous run of 64*K scalars, so consecutive lanes touch consecutive
 //      addresses on that side and K-long runs on the tree side, instead of one lane copying K
 //      scalars in a serial loop.
-// Blocks are persistent (grid-stride over tiles of 256 points) so the LDS copy of the child rows
-// is filled once per block.
+// Blocks are persistent (grid-stride over tiles of 512 points, two per lane) so the LDS copy of the
+// child rows is filled once per block.
 #pragma once
 
 #include "tree_walk.h"
@@ -21,23 +21,47 @@ constexpr int kWave = 64;
 
 enum QueryMode { kQueryGather = 0, kQueryScatterAdd = 1, kQueryAssign = 2 };
 
+constexpr int kQueryPts = 2;   // points a lane walks in lockstep (their child reads overlap)
+
+// Leaves of a lane's kQueryPts points: leaf[u] = packed leaf id or -1.
 template <typename T, bool kOctree>
-__device__ __forceinline__ int64_t query_leaf(const TreeDev<T>& tr, const int32_t* lds_child,
-                                              int32_t lds_nodes, const T* offset, const T* scaling,
-                                              const T* p) {
-    T xyz[3] = {p[0], p[1], p[2]};
-    transform_coord(xyz, offset, scaling);
-    if constexpr (kOctree) {
-        const float cx = clamp01(xyz[0]), cy = clamp01(xyz[1]), cz = clamp01(xyz[2]);
-        int levels;
-        const int32_t leaf = descend_octree(tr.child, lds_child, lds_nodes, tr.capacity,
-                                            cell_coord(cx), cell_coord(cy), cell_coord(cz), &levels);
-        if (leaf >= 0) return leaf;
-        // deeper than the integer coordinates resolve: repeat with the floating-point walk
+__device__ __forceinline__ void query_leaves(const TreeDev<T>& tr, const int32_t* lds_child, int32_t lds_nodes,
+                                             const T* offset, const T* scaling, const T* __restrict__ points,
+                                             const int64_t* q, int64_t n_points, int64_t* leaf) {
+    T xyz[kQueryPts][3];
+    bool valid[kQueryPts];
+#pragma unroll
+    for (int u = 0; u < kQueryPts; ++u) {
+        valid[u] = q[u] < n_points;
+        leaf[u] = -1;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) xyz[u][k] = valid[u] ? points[q[u] * 3 + k] : T(0);
+        transform_coord(xyz[u], offset, scaling);
     }
-    T cube;
-    int levels;
-    return descend_generic<T>(tr.child, tr.capacity, tr.N, xyz, &cube, &levels);
+    if constexpr (kOctree) {
+        uint32_t ix[kQueryPts], iy[kQueryPts], iz[kQueryPts];
+        int32_t cell[kQueryPts];
+#pragma unroll
+        for (int u = 0; u < kQueryPts; ++u) {
+            ix[u] = cell_coord(clamp01(xyz[u][0]));
+            iy[u] = cell_coord(clamp01(xyz[u][1]));
+            iz[u] = cell_coord(clamp01(xyz[u][2]));
+        }
+        descend_octree_multi<kQueryPts>(tr.child, lds_child, lds_nodes, tr.capacity, ix, iy, iz, valid, cell);
+#pragma unroll
+        for (int u = 0; u < kQueryPts; ++u) {
+            leaf[u] = cell[u];
+            valid[u] = valid[u] && cell[u] < 0;   // deeper than the integer coordinates resolve:
+        }                                         // repeat those with the floating-point walk
+    }
+#pragma unroll
+    for (int u = 0; u < kQueryPts; ++u) {
+        if (valid[u]) {
+            T cube;
+            int levels;
+            leaf[u] = descend_generic<T>(tr.child, tr.capacity, tr.N, xyz[u], &cube, &levels);
+        }
+    }
 }
 
 // MODE gather:      values[q][0..Kx) = data[leaf_q][0..Kx), ids[q] = leaf_q        (Kx = K)
@@ -56,44 +80,95 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(TreeDev<T> tr, con
     T offset[3], scaling[3];
     load_transform(tr, offset, scaling);
     const int lane = threadIdx.x & (kWave - 1);
-    const int64_t n_tiles = (n_points + kQueryThreads - 1) / kQueryThreads;
+    constexpr int kTile = kQueryThreads * kQueryPts;   // points per block and iteration
+    const int64_t n_tiles = (n_points + kTile - 1) / kTile;
     const int64_t row = (MODE == kQueryAssign) ? (int64_t)tr.K : (int64_t)Kx;
-    const int step_e = kWave % Kx, step_p = kWave / Kx;
+    // records and output rows start on 16-byte boundaries: move 16-byte pieces
+    const bool vec16 = (Kx * (int)sizeof(T)) % 16 == 0 && (((uintptr_t)tr.data | (uintptr_t)values) & 15u) == 0;
 
     for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-        const int64_t wave_base = tile * kQueryThreads + (threadIdx.x & ~(kWave - 1));
-        const int64_t q = wave_base + lane;
-        int64_t leaf = -1;
-        if (q < n_points) {
-            leaf = query_leaf<T, kOctree>(tr, lds_child, lds_nodes, offset, scaling, points + q * 3);
-            if (MODE == kQueryGather && ids) ids[q] = leaf;
+        // a wavefront owns kQueryPts runs of 64 consecutive points; lane l walks point l of each run
+        const int64_t wave_first = tile * kTile + (int64_t)(threadIdx.x / kWave) * (kWave * kQueryPts);
+        int64_t q[kQueryPts], leaves[kQueryPts];
+#pragma unroll
+        for (int u = 0; u < kQueryPts; ++u) q[u] = wave_first + u * kWave + lane;
+        query_leaves<T, kOctree>(tr, lds_child, lds_nodes, offset, scaling, points, q, n_points, leaves);
+        if (MODE == kQueryGather && ids) {
+#pragma unroll
+            for (int u = 0; u < kQueryPts; ++u)
+                if (q[u] < n_points) ids[q[u]] = leaves[u];
         }
-        // phase 2: flat index f = p*Kx + e over the wavefront's 64 rows
-        const int64_t remaining = n_points - wave_base;
-        const int n_rows = remaining < kWave ? (int)(remaining > 0 ? remaining : 0) : kWave;
-        const int total = n_rows * Kx;
-        int p = lane / Kx, e = lane % Kx;
-        T* lin = values + wave_base * Kx;
-        for (int f = lane; __any(f < total); f += kWave) {
-            // every lane takes part in the shuffle; rows past the end read lane 0's leaf
-            const int src_lane = f < total ? p : 0;
-            const int lo = __shfl((int)(leaf & 0xffffffff), src_lane);
-            const int hi = __shfl((int)(leaf >> 32), src_lane);
-            const int64_t lf = ((int64_t)hi << 32) | (uint32_t)lo;
-            if (f < total && lf >= 0) {
-                if (MODE == kQueryGather) {
-                    lin[f] = tr.data[lf * row + e];
-                } else if (MODE == kQueryScatterAdd) {
-                    atomicAdd(target + lf * row + e, lin[f]);
-                } else {
-                    tr.data[lf * row + e] = lin[f];
+        // phase 2, run by run: the 64 rows of a run, flat index f = p * Kx + e
+#pragma unroll
+        for (int u = 0; u < kQueryPts; ++u) {
+            const int64_t wave_base = wave_first + u * kWave;
+            const int64_t leaf = leaves[u];
+            const int64_t remaining = n_points - wave_base;
+            const int n_rows = remaining < kWave ? (int)(remaining > 0 ? remaining : 0) : kWave;
+            T* lin = values + wave_base * Kx;
+            const int leaf_lo = (int)(leaf & 0xffffffff), leaf_hi = (int)(leaf >> 32);
+            if (MODE == kQueryGather && vec16) {
+                // 16-byte pieces: a record is `pieces` of them, and kBatch loads per lane are in flight
+                // before the first store (the compiler must assume that the output aliases the tree)
+                constexpr int kPer = 16 / (int)sizeof(T);
+                constexpr int kBatch = 4;
+                const int pieces = Kx / kPer;
+                const int total = n_rows * pieces;
+                const int step_e = kWave % pieces, step_p = kWave / pieces;
+                int p = lane / pieces, e = lane % pieces;
+                uint4* lin16 = (uint4*)lin;
+                for (int f0 = 0; f0 < total; f0 += kWave * kBatch) {
+                    uint4 buf[kBatch];
+#pragma unroll
+                    for (int b = 0; b < kBatch; ++b) {
+                        const int f = f0 + b * kWave + lane;
+                        // every lane takes part in the shuffle; rows past the end read lane 0's leaf
+                        const int src_lane = f < total ? p : 0;
+                        const int lo = __shfl(leaf_lo, src_lane);
+                        const int hi = __shfl(leaf_hi, src_lane);
+                        const int64_t lf = ((int64_t)hi << 32) | (uint32_t)lo;
+                        buf[b] = make_uint4(0u, 0u, 0u, 0u);
+                        if (f < total && lf >= 0) buf[b] = ((const uint4*)(tr.data + lf * row))[e];
+                        e += step_e;
+                        p += step_p;
+                        if (e >= pieces) {
+                            e -= pieces;
+                            p += 1;
+                        }
+                    }
+#pragma unroll
+                    for (int b = 0; b < kBatch; ++b) {
+                        const int f = f0 + b * kWave + lane;
+                        if (f < total) lin16[f] = buf[b];
+                    }
                 }
+                continue;
             }
-            e += step_e;
-            p += step_p;
-            if (e >= Kx) {
-                e -= Kx;
-                p += 1;
+            const int total = n_rows * Kx;
+            const int step_e = kWave % Kx, step_p = kWave / Kx;
+            int p = lane / Kx, e = lane % Kx;
+            for (int f = lane; __any(f < total); f += kWave) {
+                const int src_lane = f < total ? p : 0;
+                const int lo = __shfl(leaf_lo, src_lane);
+                const int hi = __shfl(leaf_hi, src_lane);
+                const int64_t lf = ((int64_t)hi << 32) | (uint32_t)lo;
+                if (f < total && lf >= 0) {
+                    if (MODE == kQueryGather) {
+                        lin[f] = tr.data[lf * row + e];
+                    } else if (MODE == kQueryScatterAdd) {
+                        atomicAdd(target + lf * row + e, lin[f]);
+                    } else {
+                        tr.data[lf * row + e] = lin[f];
+                    }
+                } else if (MODE == kQueryGather && f < total) {
+                    lin[f] = T(0);   // malformed tree: no leaf
+                }
+                e += step_e;
+                p += step_p;
+                if (e >= Kx) {
+                    e -= Kx;
+                    p += 1;
+                }
             }
         }
     }

@@ -99,7 +99,8 @@ int launch_query(const SvoxTreeSpec* tree, const void* points, int64_t n, void* 
                  int64_t* ids, int32_t Kx, hipStream_t stream, const char* what) {
     if (n == 0) return SVOX_OK;
     const TreeDev<T> tr = make_tree<T>(tree);
-    const int64_t tiles = (n + kQueryThreads - 1) / kQueryThreads;
+    const int64_t per_tile = (int64_t)kQueryThreads * kQueryPts;
+    const int64_t tiles = (n + per_tile - 1) / per_tile;
     const int64_t blocks = tiles < 256 * 8 ? tiles : 256 * 8;
     if constexpr (sizeof(T) == 4) {
         if (octree_fast_ok(tree)) {

@@ -123,6 +123,49 @@ __device__ __forceinline__ int32_t descend_octree(const int32_t* __restrict__ ch
     return -1;  // deeper than the integer coordinates resolve; the host routes such trees elsewhere
 }
 
+// The same walk for kPts points of one lane in lockstep: the child reads of the points are
+// independent, so they are in flight together and the lane waits once per level instead of once
+// per level and point.  leaf[u] = cell index or -1.
+template <int kPts>
+__device__ __forceinline__ void descend_octree_multi(const int32_t* __restrict__ child, const int32_t* lds_child,
+                                                     int32_t lds_nodes, int64_t capacity, const uint32_t* ix,
+                                                     const uint32_t* iy, const uint32_t* iz, const bool* valid,
+                                                     int32_t* leaf) {
+    int32_t node[kPts];
+    bool live[kPts];
+    bool any_live = false;
+#pragma unroll
+    for (int u = 0; u < kPts; ++u) {
+        node[u] = 0;
+        leaf[u] = -1;
+        live[u] = valid[u];
+        any_live |= live[u];
+    }
+    for (int level = 1; level <= kCoordBits && any_live; ++level) {
+        int32_t cell[kPts], skip[kPts];
+#pragma unroll
+        for (int u = 0; u < kPts; ++u) {
+            cell[u] = node[u] * 8 + cell_at(ix[u], iy[u], iz[u], level);
+            skip[u] = 0;
+            if (live[u]) skip[u] = node[u] < lds_nodes ? lds_child[cell[u]] : child[cell[u]];
+        }
+        any_live = false;
+#pragma unroll
+        for (int u = 0; u < kPts; ++u) {
+            if (live[u]) {
+                if (skip[u] == 0) {
+                    leaf[u] = cell[u];
+                    live[u] = false;
+                } else {
+                    node[u] += skip[u];
+                    if (node[u] < 0 || node[u] >= capacity) live[u] = false;
+                }
+            }
+            any_live |= live[u];
+        }
+    }
+}
+
 // leaf-local position frac(pc * 2^levels) and the reciprocal cell count 2^-levels
 __device__ __forceinline__ float leaf_local(float pc, float cube_sz) {
     const float s = pc * cube_sz;
