@@ -399,12 +399,20 @@ constexpr int kQueue = 4;  // leaves a lane walks ahead before the wavefront sha
 // every lane's ray is kept as a row (needed where other lanes multiply with it); otherwise only
 // the view direction is kept and the basis is re-evaluated where it is used.
 template <int D, bool kRows>
-struct ShadeShared {
+struct ShadeShared;
+template <int D>
+struct ShadeShared<D, true> {
     int32_t leaf[kQueue * kMarchThreads];       // leaf cell index of entry e
     uint8_t who[kQueue * kMarchThreads];        // owner lane | slot << 6
     float colour[kQueue * kMarchThreads * 3];   // [slot][lane][channel]: sigmoid(basis . coefficients)
-    float basis[kRows ? kMarchThreads * D : 1]; // [lane][coefficient]
-    float vdir[kRows ? 1 : kMarchThreads * 3];  // [lane][xyz]
+    float basis[kMarchThreads * D];             // [lane][coefficient]
+};
+template <int D>
+struct ShadeShared<D, false> {
+    int32_t leaf[kQueue * kMarchThreads];
+    uint8_t who[kQueue * kMarchThreads];
+    float colour[kQueue * kMarchThreads * 3];
+    float vdir[kMarchThreads * 3];              // [lane][xyz]
 };
 
 // Colours of all list entries, computed by the whole wavefront: item p = 3 * entry + channel goes to
@@ -464,7 +472,9 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
 // when every leaf is shaded on the spot.
 // kAccum: the compositing weight of every shaded leaf is also added to (or maximised into)
 // tr.weight_accum at the leaf's cell index (rt_kernel.cu:298-304).
-template <class P, class Source, bool kAccum>
+// kRefill: the wavefront owns more than 64 rays and refills idle lanes; without it the 64 rays are
+// set up once before the loop, and nothing the set-up needs stays live inside it.
+template <class P, class Source, bool kAccum, bool kRefill>
 __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<float> tr, Source src,
                                                                        SvoxRenderOptions opt,
                                                                        float* __restrict__ out) {
@@ -493,39 +503,48 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
-    while (true) {
-        // ---- refill
-        const unsigned long long idle = __ballot(!active);
-        const int n_idle = __popcll(idle);
-        if (next < end && n_idle >= src.refill_at) {
-            if (!active) {
-                const int64_t item = next + rank_in(idle);
-                if (item < end) {
-                    float origin[3], dir[3], vdir[3];
-                    slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
-                    if (slot >= 0) {
-                        if (setup_ray(r, origin, dir, scaling)) {
-                            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
-                                sh.vdir[lane * 3] = vdir[0];
-                                sh.vdir[lane * 3 + 1] = vdir[1];
-                                sh.vdir[lane * 3 + 2] = vdir[2];
-                            }
-                            acc[0] = acc[1] = acc[2] = 0.0f;
-                            light = 1.0f;
-                            cur.levels = 0;
-                            active = true;
-                        } else {
-                            out[slot * 3] = bg;
-                            out[slot * 3 + 1] = bg;
-                            out[slot * 3 + 2] = bg;
-                        }
-                    }
-                }
+    // takes ray `item` into this lane: a miss is answered at once, a hit becomes the lane's ray
+    auto start = [&](int64_t item) {
+        float origin[3], dir[3], vdir[3];
+        slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+        if (slot < 0) return;
+        if (setup_ray(r, origin, dir, scaling)) {
+            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+                sh.vdir[lane * 3] = vdir[0];
+                sh.vdir[lane * 3 + 1] = vdir[1];
+                sh.vdir[lane * 3 + 2] = vdir[2];
             }
-            next += n_idle;
-            continue;
+            acc[0] = acc[1] = acc[2] = 0.0f;
+            light = 1.0f;
+            cur.levels = 0;
+            active = true;
+        } else {
+            out[slot * 3] = bg;
+            out[slot * 3 + 1] = bg;
+            out[slot * 3 + 2] = bg;
         }
-        if (n_idle == kMarchThreads) break;
+    };
+    if constexpr (!kRefill) {
+        if (next + lane < end) start(next + lane);
+    }
+
+    while (true) {
+        if constexpr (kRefill) {
+            // ---- refill
+            const unsigned long long idle = __ballot(!active);
+            const int n_idle = __popcll(idle);
+            if (next < end && n_idle >= src.refill_at) {
+                if (!active) {
+                    const int64_t item = next + rank_in(idle);
+                    if (item < end) start(item);
+                }
+                next += n_idle;
+                continue;
+            }
+            if (n_idle == kMarchThreads) break;
+        } else {
+            if (!__any(active)) break;
+        }
 
         // ---- walk
         int32_t q_leaf[kQueue];

@@ -256,15 +256,20 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
+#define SVOX_LAUNCH_FORWARD(ACCUM, REFILL)                                                                     \
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, ACCUM, REFILL>), dim3(blocks), \
+                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), src,     \
+                                               *opt, (float*)out))
+            const bool refill = src.per_wave > kMarchThreads;
             if (tree->weight_accum) {
-                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, true>), dim3(blocks),
-                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                           src, *opt, (float*)out));
+                // accumulation is an analysis pass: one variant is enough
+                SVOX_LAUNCH_FORWARD(true, true);
+            } else if (refill) {
+                SVOX_LAUNCH_FORWARD(false, true);
             } else {
-                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, false>), dim3(blocks),
-                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                           src, *opt, (float*)out));
+                SVOX_LAUNCH_FORWARD(false, false);
             }
+#undef SVOX_LAUNCH_FORWARD
             return;
         }
     }

@@ -23,7 +23,7 @@ namespace svox {
 
 constexpr int kMaxWalkLevels = 64;   // a deeper (malformed) tree ends the walk with leaf -1
 constexpr int kCoordBits = 24;       // integer cell coordinates hold 24 levels of an octree
-constexpr int kPathLevels = 12;      // levels of the previous path remembered per lane
+constexpr int kPathLevels = 11;      // levels of the previous path remembered per lane
 
 template <typename T>
 struct TreeDev {
