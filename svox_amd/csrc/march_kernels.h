@@ -107,6 +107,7 @@ struct BatchSource {
     RayBatch<T> rays;
     int per_wave;
     int refill_at;   // idle lanes that trigger taking new rays
+    int xcd_group;   // see chunk_of_block; 1 for unrelated rays
     __device__ __forceinline__ int64_t total() const { return rays.n_rays; }
     __device__ __forceinline__ int64_t fetch_item(int64_t i, const SvoxRenderOptions&, const T* offset,
                                                   const T* scaling, T* origin, T* dir, T* vdir) const {
@@ -124,6 +125,21 @@ struct BatchSource {
 
 __host__ __device__ inline int blocks16_of(int extent) { return (extent + 15) / 16; }
 
+// Which chunk of items the wavefront of block `b` (of gridDim.x) works on.  Workgroups are handed
+// to the 8 XCDs in turn (block b runs on XCD b mod 8), and every XCD has its own L2.  With
+// group > 1, runs of `group` consecutive chunks go to one XCD, so neighbouring image tiles, whose
+// rays read the same child rows and leaf records, share that L2; the runs themselves still rotate
+// over the XCDs, which keeps the load balanced.  A bijection on [0, gridDim.x).
+__device__ __forceinline__ int64_t chunk_of_block(unsigned b, unsigned n_blocks, int group) {
+    constexpr unsigned kXcds = 8;
+    if (group <= 1) return b;
+    const unsigned span = kXcds * (unsigned)group;
+    const unsigned full = n_blocks / span * span;
+    if (b >= full) return b;
+    const unsigned xcd = b % kXcds, j = b / kXcds;
+    return (int64_t)((j / group) * kXcds + xcd) * group + j % group;
+}
+
 template <typename T>
 struct ImageSource {
     Camera<T> cam;          // cam.c2w: pose of image 0
@@ -131,6 +147,7 @@ struct ImageSource {
     int64_t pose_stride;    // scalars between consecutive poses
     int per_wave;           // 64 (one 8x8 tile) or 256 (one 16x16 block)
     int refill_at;          // idle lanes that trigger taking new rays
+    int xcd_group;          // see chunk_of_block
     __device__ __forceinline__ int64_t total() const {
         return (int64_t)n_images * blocks16_of(cam.width) * blocks16_of(cam.height) * 256;
     }
@@ -490,7 +507,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     const float step = opt.step_size, sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
 
-    int64_t next = blockIdx.x * (int64_t)src.per_wave;
+    int64_t next = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)src.per_wave;
     const int64_t total = src.total();
     const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
@@ -760,7 +777,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
 // summed first, so that leaf receives one atomic per element instead of one per ray.  The per-term
 // products are the reference's; only the order in which they are added up differs.
 // Both marches test sigma > 0 and never stop early (rt_kernel.cu:377, 441).
-template <class P, class Source>
+template <class P, class Source, bool kRefill>
 __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<float> tr, Source src,
                                                                         SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
@@ -777,7 +794,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     const float step = opt.step_size;
 
-    int64_t next = blockIdx.x * (int64_t)src.per_wave;
+    int64_t next = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)src.per_wave;
     const int64_t total = src.total();
     const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
@@ -789,39 +806,49 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
-    while (true) {
-        // ---- refill
-        const unsigned long long idle = __ballot(!active);
-        const int n_idle = __popcll(idle);
-        if (next < end && n_idle >= src.refill_at) {
-            if (!active) {
-                const int64_t item = next + rank_in(idle);
-                if (item < end) {
-                    float origin[3], dir[3], vdir[3];
-                    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
-                    if (slot >= 0 && setup_ray(r, origin, dir, scaling)) {
-                        if constexpr (P::kFormat == SVOX_FORMAT_SH) {
-                            float basis[D];
-                            sh_basis<float>(P::kBasis, vdir, basis);
+    // takes ray `item` into this lane if it hits the tree
+    auto start = [&](int64_t item) {
+        float origin[3], dir[3], vdir[3];
+        const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+        if (slot >= 0 && setup_ray(r, origin, dir, scaling)) {
+            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+                float basis[D];
+                sh_basis<float>(P::kBasis, vdir, basis);
 #pragma unroll
-                            for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
-                        }
-                        go[0] = grad_out[slot * 3];
-                        go[1] = grad_out[slot * 3 + 1];
-                        go[2] = grad_out[slot * 3 + 2];
-                        light = 1.0f;
-                        accum = 0.0f;
-                        tmin = r.t;
-                        cur.levels = 0;
-                        second = false;
-                        active = true;
-                    }
-                }
+                for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
-            next += n_idle;
-            continue;
+            go[0] = grad_out[slot * 3];
+            go[1] = grad_out[slot * 3 + 1];
+            go[2] = grad_out[slot * 3 + 2];
+            light = 1.0f;
+            accum = 0.0f;
+            tmin = r.t;
+            cur.levels = 0;
+            second = false;
+            active = true;
         }
-        if (n_idle == kMarchThreads) break;
+    };
+    if constexpr (!kRefill) {
+        if (next + lane < end) start(next + lane);
+    }
+
+    while (true) {
+        if constexpr (kRefill) {
+            // ---- refill
+            const unsigned long long idle = __ballot(!active);
+            const int n_idle = __popcll(idle);
+            if (next < end && n_idle >= src.refill_at) {
+                if (!active) {
+                    const int64_t item = next + rank_in(idle);
+                    if (item < end) start(item);
+                }
+                next += n_idle;
+                continue;
+            }
+            if (n_idle == kMarchThreads) break;
+        } else {
+            if (!__any(active)) break;
+        }
 
         // ---- walk
         int32_t q_leaf[kQueue];
@@ -1104,7 +1131,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_generic_kernel(TreeDev<
 // (the reference's second march) and the density terms (its third).  Every term has the reference's
 // value; records are added cooperatively, one coalesced atomic instruction per record element and
 // output array, after summing the lanes whose rays sit in the same leaf.
-template <class P, class Source>
+template <class P, class Source, bool kRefill>
 __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> tr, Source src, SvoxRenderOptions opt,
                                                                 const float* __restrict__ color_ref,
                                                                 float* __restrict__ color_out,
@@ -1122,7 +1149,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     const float step = opt.step_size;
 
-    int64_t next = blockIdx.x * (int64_t)src.per_wave;
+    int64_t next = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)src.per_wave;
     const int64_t total = src.total();
     const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
@@ -1137,47 +1164,56 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
-    while (true) {
-        // ---- refill
-        const unsigned long long idle = __ballot(!active);
-        const int n_idle = __popcll(idle);
-        if (next < end && n_idle >= src.refill_at) {
-            if (!active) {
-                const int64_t item = next + rank_in(idle);
-                if (item < end) {
-                    float origin[3], dir[3], vdir[3];
-                    slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
-                    if (slot >= 0) {
-                        if (setup_ray(r, origin, dir, scaling)) {
-                            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
-                                float basis[D];
-                                sh_basis<float>(P::kBasis, vdir, basis);
+    // takes ray `item` into this lane: a miss is answered at once, a hit becomes the lane's ray
+    auto start = [&](int64_t item) {
+        float origin[3], dir[3], vdir[3];
+        slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+        if (slot < 0) return;
+        if (setup_ray(r, origin, dir, scaling)) {
+            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+                float basis[D];
+                sh_basis<float>(P::kBasis, vdir, basis);
 #pragma unroll
-                                for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
-                            }
-#pragma unroll
-                            for (int c = 0; c < 3; ++c) {
-                                ref[c] = color_ref[slot * 3 + c];
-                                resid[c] = 0.0f;
-                                caccum[c] = 0.0f;
-                            }
-                            light = light1 = 1.0f;
-                            tmin = r.t;
-                            cur.levels = 0;
-                            second = false;
-                            active = true;
-                        } else {
-                            color_out[slot * 3] = bg;
-                            color_out[slot * 3 + 1] = bg;
-                            color_out[slot * 3 + 2] = bg;
-                        }
-                    }
-                }
+                for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
-            next += n_idle;
-            continue;
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                ref[c] = color_ref[slot * 3 + c];
+                resid[c] = 0.0f;
+                caccum[c] = 0.0f;
+            }
+            light = light1 = 1.0f;
+            tmin = r.t;
+            cur.levels = 0;
+            second = false;
+            active = true;
+        } else {
+            color_out[slot * 3] = bg;
+            color_out[slot * 3 + 1] = bg;
+            color_out[slot * 3 + 2] = bg;
         }
-        if (n_idle == kMarchThreads) break;
+    };
+    if constexpr (!kRefill) {
+        if (next + lane < end) start(next + lane);
+    }
+
+    while (true) {
+        if constexpr (kRefill) {
+            // ---- refill
+            const unsigned long long idle = __ballot(!active);
+            const int n_idle = __popcll(idle);
+            if (next < end && n_idle >= src.refill_at) {
+                if (!active) {
+                    const int64_t item = next + rank_in(idle);
+                    if (item < end) start(item);
+                }
+                next += n_idle;
+                continue;
+            }
+            if (n_idle == kMarchThreads) break;
+        } else {
+            if (!__any(active)) break;
+        }
 
         // ---- walk
         int32_t q_leaf[kQueue];

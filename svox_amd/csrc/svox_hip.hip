@@ -199,6 +199,17 @@ int pick_refill() {
     return forced >= 1 && forced <= 64 ? forced : 16;
 }
 
+// Image tiles handed to one XCD in a row (chunk_of_block): 16 tiles are four 16x16 pixel blocks.
+// Measured on 8 poses of 800x800: 1 -> 16 shortens the launch by 2-3 %, larger runs gain no more and
+// start to unbalance the XCDs.  SVOX_XCD_GROUP overrides it for experiments.
+int pick_xcd_group() {
+    static const int forced = [] {
+        const char* e = getenv("SVOX_XCD_GROUP");
+        return e ? atoi(e) : 0;
+    }();
+    return forced >= 1 && forced <= 4096 ? forced : 16;
+}
+
 template <typename T>
 BatchSource<T> batch_source(const SvoxRaysSpec* rays, bool backward = false) {
     BatchSource<T> s;
@@ -208,6 +219,7 @@ BatchSource<T> batch_source(const SvoxRaysSpec* rays, bool backward = false) {
     s.rays.n_rays = rays->n_rays;
     s.per_wave = pick_per_wave(rays->n_rays, backward);
     s.refill_at = pick_refill();
+    s.xcd_group = 1;
     return s;
 }
 
@@ -226,6 +238,7 @@ ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pos
     // tree: one tile per wavefront keeps the busy tiles spread over the whole GPU
     s.per_wave = 64;
     s.refill_at = pick_refill();
+    s.xcd_group = pick_xcd_group();
     return s;
 }
 
@@ -285,9 +298,15 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
-            SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source>), dim3(blocks),
-                                                       dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                       src, *opt, (const float*)grad_out, (float*)grad_data));
+            if (src.per_wave > kMarchThreads) {
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, true>), dim3(blocks),
+                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                           src, *opt, (const float*)grad_out, (float*)grad_data));
+            } else {
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, false>), dim3(blocks),
+                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                           src, *opt, (const float*)grad_out, (float*)grad_data));
+            }
             return;
         }
     }
@@ -309,10 +328,17 @@ void launch_se_grad(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
-            SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source>), dim3(blocks), dim3(kMarchThreads),
-                                                       0, stream, make_tree<float>(tree), src, *opt,
-                                                       (const float*)color_ref, (float*)color_out, (float*)grad,
-                                                       (float*)hess));
+            if (src.per_wave > kMarchThreads) {
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source, true>), dim3(blocks),
+                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                           src, *opt, (const float*)color_ref, (float*)color_out,
+                                                           (float*)grad, (float*)hess));
+            } else {
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source, false>), dim3(blocks),
+                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                           src, *opt, (const float*)color_ref, (float*)color_out,
+                                                           (float*)grad, (float*)hess));
+            }
             return;
         }
     }

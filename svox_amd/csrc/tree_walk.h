@@ -173,8 +173,9 @@ __device__ __forceinline__ float leaf_local(float pc, float cube_sz) {
 }
 
 // Per-lane cursor that remembers the previous descent.  `path` points at this lane's column of an
-// LDS array laid out [kPathLevels + 1][block threads]: path[l * stride] is the node whose child row
-// is indexed at level l + 1 (path[0] is the root, node 0); the last row is a dump for deeper levels.
+// LDS array laid out [kPathLevels + 1][block threads]: path[l * stride], l < kPathLevels, is the node
+// whose child row is indexed at level l + 1 (path[0] is the root, node 0); the last row is a dump
+// for the levels below kPathLevels, which a restart never resumes from.
 struct OctreeCursor {
     int32_t* path;
     int stride;
@@ -212,7 +213,7 @@ struct OctreeCursor {
         }
         int32_t cell, skip;
         while (true) {
-            path[((level < kPathLevels ? level : kPathLevels + 1) - 1) * stride] = node;
+            path[((level <= kPathLevels ? level : kPathLevels + 1) - 1) * stride] = node;
             cell = (node << 3) | cell_at(nx, ny, nz, level);
             // the table is smaller than 4 GiB (checked on the host): a 32-bit byte offset from the
             // uniform base lets the load use the scalar-base addressing form

@@ -79,6 +79,38 @@ def dense_tree(levels, data_format="RGBA", seed=0, device="cpu", zero_fraction=0
     return tree.to(device) if str(device) != "cpu" else tree
 
 
+def deep_tree(levels, data_format="SH4", seed=0, base_refine=2, dtype=torch.float32):
+    """Octree that is `levels` levels deep along one root-to-leaf chain: a dense 2^base_refine grid
+    whose leaf at a seeded point is split again and again.  Returns (tree, point): the point lies in
+    the deepest leaf.  Densities are positive everywhere, growing towards the deep end, so that rays
+    through the point shade leaves of every size."""
+    g = _gen(seed)
+    tree = N3Tree(N=2, data_format=data_format, init_refine=base_refine, depth_limit=levels + 2, dtype=dtype)
+    point = 0.2 + 0.6 * torch.rand(3, generator=g, dtype=torch.float64)
+    while True:
+        child = tree.child
+        node, q, depth = 0, point.clone(), 0
+        while True:
+            q = q * 2
+            idx = q.floor().long()
+            q = q - idx
+            depth += 1
+            skip = int(child[node, idx[0], idx[1], idx[2]])
+            if skip == 0:
+                break
+            node += skip
+        if depth >= levels:
+            break
+        tree.refine(sel=(torch.tensor([node]), idx[0:1], idx[1:2], idx[2:3]))
+    shape = tree.data.shape
+    vals = torch.randn(shape, generator=g) * 0.5
+    node_depth = tree.parent_depth[:, 1].to(torch.float32)
+    sigma = (0.5 + torch.rand(shape[:-1], generator=g)) * (2.0 + node_depth)[:, None, None, None]
+    vals[..., -1] = sigma
+    tree.data.data[:] = vals.to(dtype)
+    return tree, point.to(dtype)
+
+
 def _sdf_spheres(p, centers, radii):
     """Distance to the surface of the union of spheres (exact outside, a lower bound inside)."""
     d = (p[:, None, :] - centers[None]).norm(dim=-1) - radii[None]
