@@ -215,9 +215,15 @@ __device__ __forceinline__ void advance(RayState<T>& r, T delta_t) {
 }
 
 struct Visit {
-    int64_t leaf;  // cell index node*N^3 + cell, -1 ends the ray (malformed tree)
+    int64_t leaf;  // cell index node*N^3 + cell; -1 ends the ray (malformed tree); -2 descent pending
     int levels;
 };
+
+// Child entries one lane reads per turn of the octree walk (OctreeCursor::seek).  A lane that needs
+// more (its ray crossed the boundary of a large cell and has to descend many levels) goes on in its
+// next turn, so that the other lanes of the wavefront do not wait for it: measured, the lanes need
+// 2.0 entries per leaf on average, but the slowest lane of a wavefront 4.8.
+constexpr int kSeekBudget = 2;
 
 // One sample with the reference's walk: position, leaf, step length.  rt_kernel.cu:262-275.
 template <typename T>
@@ -244,7 +250,13 @@ __device__ __forceinline__ Visit step_octree(const TreeDev<float>& tr, const Ray
     for (int j = 0; j < 3; ++j) pc[j] = clamp01(fma_(r.t, r.d[j], r.o[j]));
     Visit v;
     const int32_t leaf = cur.seek(tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]), cell_coord(pc[1]),
-                                  cell_coord(pc[2]));
+                                  cell_coord(pc[2]), kSeekBudget);
+    if (leaf == OctreeCursor::kPending) {   // the descent goes on in the lane's next turn
+        v.leaf = OctreeCursor::kPending;
+        v.levels = 0;
+        *delta_t = 0.0f;
+        return v;
+    }
     float inv_cube;  // 2^-levels: dividing by the power of two 2^levels is this multiplication
     float local[3];
     if (leaf >= 0) {
@@ -533,7 +545,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
             }
             acc[0] = acc[1] = acc[2] = 0.0f;
             light = 1.0f;
-            cur.levels = 0;
+            cur.restart();
             active = true;
         } else {
             out[slot * 3] = bg;
@@ -566,21 +578,29 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         // ---- walk
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-        int n = 0;
-        bool broken = false;
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
             q_leaf[q] = 0;
             q_dt[q] = 0.0f;
+        }
+        int n = 0;
+        bool broken = false;
+#pragma unroll
+        for (int turn = 0; turn < kQueue; ++turn) {
             if (active && !broken && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
-                    q_leaf[q] = (int32_t)v.leaf;
-                    q_dt[q] = delta_t;
+#pragma unroll
+                    for (int q = 0; q < kQueue; ++q) {
+                        if (n == q) {
+                            q_leaf[q] = (int32_t)v.leaf;
+                            q_dt[q] = delta_t;
+                        }
+                    }
                     advance(r, delta_t);
-                    n = q + 1;
-                } else {
+                    n += 1;
+                } else if (v.leaf != OctreeCursor::kPending) {
                     broken = true;   // malformed tree: the ray ends here
                 }
             }
@@ -823,7 +843,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             light = 1.0f;
             accum = 0.0f;
             tmin = r.t;
-            cur.levels = 0;
+            cur.restart();
             second = false;
             active = true;
         }
@@ -853,22 +873,30 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         // ---- walk
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-        int n = 0;
-        bool broken = false;
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
             q_leaf[q] = 0;
             q_dt[q] = 0.0f;
+        }
+        int n = 0;
+        bool broken = false;
+#pragma unroll
+        for (int turn = 0; turn < kQueue; ++turn) {
             if (active && !broken && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
-                    q_leaf[q] = (int32_t)v.leaf;
-                    q_dt[q] = delta_t;
+#pragma unroll
+                    for (int q = 0; q < kQueue; ++q) {
+                        if (n == q) {
+                            q_leaf[q] = (int32_t)v.leaf;
+                            q_dt[q] = delta_t;
+                        }
+                    }
                     advance(r, delta_t);
-                    n = q + 1;
-                } else {
-                    broken = true;
+                    n += 1;
+                } else if (v.leaf != OctreeCursor::kPending) {
+                    broken = true;   // malformed tree: the ray ends here
                 }
             }
         }
@@ -1184,7 +1212,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
             }
             light = light1 = 1.0f;
             tmin = r.t;
-            cur.levels = 0;
+            cur.restart();
             second = false;
             active = true;
         } else {
@@ -1218,22 +1246,30 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         // ---- walk
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-        int n = 0;
-        bool broken = false;
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
             q_leaf[q] = 0;
             q_dt[q] = 0.0f;
+        }
+        int n = 0;
+        bool broken = false;
+#pragma unroll
+        for (int turn = 0; turn < kQueue; ++turn) {
             if (active && !broken && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
-                    q_leaf[q] = (int32_t)v.leaf;
-                    q_dt[q] = delta_t;
+#pragma unroll
+                    for (int q = 0; q < kQueue; ++q) {
+                        if (n == q) {
+                            q_leaf[q] = (int32_t)v.leaf;
+                            q_dt[q] = delta_t;
+                        }
+                    }
                     advance(r, delta_t);
-                    n = q + 1;
-                } else {
-                    broken = true;
+                    n += 1;
+                } else if (v.leaf != OctreeCursor::kPending) {
+                    broken = true;   // malformed tree: the ray ends here
                 }
             }
         }

@@ -182,25 +182,43 @@ struct OctreeCursor {
     uint32_t ix, iy, iz;  // coordinates of the previous query
     int levels;           // levels of the previous leaf, 0 = no previous query
     int32_t leaf;         // its cell index
+    int pend_level;       // > 0: a descent was interrupted before reading the child row at this level
+    int32_t pend_node;    //      of this node
+
+    static constexpr int32_t kPending = -2;
 
     __device__ __forceinline__ void reset(int32_t* lane_path, int lane_stride) {
         path = lane_path;
         stride = lane_stride;
         levels = 0;
         leaf = -1;
+        pend_level = 0;
+        pend_node = 0;
         ix = iy = iz = 0;
     }
 
-    // Finds the leaf of the point with integer coordinates (nx, ny, nz).  Returns the leaf cell
-    // index, or -1 if the tree has more levels than the coordinates hold (`levels` becomes 0).
+    // forget the previous query (a new ray)
+    __device__ __forceinline__ void restart() {
+        levels = 0;
+        pend_level = 0;
+    }
+
+    // Finds the leaf of the point with integer coordinates (nx, ny, nz), reading at most `budget`
+    // child entries.  Returns the leaf cell index; kPending if the budget ran out (call again with
+    // the same point to go on); -1 if the tree has more levels than the coordinates hold (`levels`
+    // becomes 0).  The budget bounds how long the lanes of a wavefront wait for the one lane that
+    // has to descend many levels: that lane continues in its next turn instead.
     // Node ids read from the table are clamped into [0, capacity): a malformed tree yields a wrong
     // leaf, never an access outside the table.  The loop has a single exit so that lanes which
     // found their leaf only wait, without extra mask bookkeeping per level.
     __device__ __forceinline__ int32_t seek(const int32_t* __restrict__ child, int32_t last_node,
-                                            uint32_t nx, uint32_t ny, uint32_t nz) {
+                                            uint32_t nx, uint32_t ny, uint32_t nz, int budget) {
         int level = 1;
         int32_t node = 0;
-        if (levels > 0) {
+        if (pend_level > 0) {
+            level = pend_level;
+            node = pend_node;
+        } else if (levels > 0) {
             const uint32_t diff = (ix ^ nx) | (iy ^ ny) | (iz ^ nz);
             // first level at which the two points fall into different cells
             const int first_diff = diff ? (kCoordBits - 31 + __builtin_clz(diff)) : kCoordBits + 1;
@@ -211,6 +229,7 @@ struct OctreeCursor {
         } else {
             ix = nx; iy = ny; iz = nz;
         }
+        const int stop_level = level + budget - 1 < kCoordBits ? level + budget - 1 : kCoordBits;
         int32_t cell, skip;
         while (true) {
             path[((level <= kPathLevels ? level : kPathLevels + 1) - 1) * stride] = node;
@@ -218,15 +237,19 @@ struct OctreeCursor {
             // the table is smaller than 4 GiB (checked on the host): a 32-bit byte offset from the
             // uniform base lets the load use the scalar-base addressing form
             skip = *(const int32_t*)((const char*)child + ((uint32_t)cell << 2));
-            if (skip == 0 || level == kCoordBits) break;
+            if (skip == 0 || level == stop_level) break;
             // a negative or too large id (malformed tree) wraps / clamps to the last node
             node = (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node);
             level += 1;
         }
+        pend_level = 0;
         if (skip != 0) {
-            levels = 0;
+            levels = 0;   // the path rows written so far stay valid, but there is no previous leaf
             leaf = -1;
-            return -1;
+            if (level == kCoordBits) return -1;
+            pend_level = level + 1;
+            pend_node = (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node);
+            return kPending;
         }
         levels = level;
         leaf = cell;

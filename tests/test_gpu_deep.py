@@ -45,13 +45,18 @@ def test_deep_tree_render(gpu, oracle_mod, levels, fmt):
             C.set_debug_flags(0)
         assert np.array_equal(out, ref), generic
         assert stats["samples"] == ref_stats["samples"] and stats["levels"] == ref_stats["levels"]
-    go = torch.randn(4000, 3, generator=torch.Generator().manual_seed(1))
-    want = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    # gradients on fewer rays: thousands of rays adding into under a hundred leaves would make the
+    # fp32 summation order (sequential in the oracle, atomics here) the largest term of the comparison
+    m = 1000
+    sub = svox.Rays(rays.origins[:m].contiguous(), rays.dirs[:m].contiguous(), rays.viewdirs[:m].contiguous())
+    rs = rays_spec(sub, gpu)
+    go = torch.randn(m, 3, generator=torch.Generator().manual_seed(1))
+    want = oracle_mod.volume_render_backward(ot, sub.origins, sub.dirs, sub.viewdirs, opt, go)
     got = C.volume_render_backward(dev._spec(), rs, opt, go.to(gpu)).cpu().numpy()
     err, ok = grad_close(got, want)
     assert ok, err
-    colour = torch.rand(4000, 3, generator=torch.Generator().manual_seed(2))
-    want = oracle_mod.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, colour, opt)
+    colour = torch.rand(m, 3, generator=torch.Generator().manual_seed(2))
+    want = oracle_mod.se_grad(ot, sub.origins, sub.dirs, sub.viewdirs, colour, opt)
     got = C.se_grad(dev._spec(), rs, colour.to(gpu), opt)
     assert np.array_equal(got[0].cpu().numpy(), want[0])
     for g, w in zip(got[1:], want[1:]):
