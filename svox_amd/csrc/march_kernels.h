@@ -222,7 +222,8 @@ struct Visit {
 // Child entries one lane reads per turn of the octree walk (OctreeCursor::seek).  A lane that needs
 // more (its ray crossed the boundary of a large cell and has to descend many levels) goes on in its
 // next turn, so that the other lanes of the wavefront do not wait for it: measured, the lanes need
-// 2.0 entries per leaf on average, but the slowest lane of a wavefront 4.8.
+// 2.0 entries per leaf on average, but the slowest lane of a wavefront 4.8.  (Budgets of 1 and 3, and
+// extra turns per round for the interrupted lanes, were measured slower.)
 constexpr int kSeekBudget = 2;
 
 // One sample with the reference's walk: position, leaf, step length.  rt_kernel.cu:262-275.
@@ -587,7 +588,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         bool broken = false;
 #pragma unroll
         for (int turn = 0; turn < kQueue; ++turn) {
-            if (active && !broken && r.t < r.tmax) {
+            if (active && !broken && n < kQueue && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
@@ -882,7 +883,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         bool broken = false;
 #pragma unroll
         for (int turn = 0; turn < kQueue; ++turn) {
-            if (active && !broken && r.t < r.tmax) {
+            if (active && !broken && n < kQueue && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
@@ -1255,7 +1256,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         bool broken = false;
 #pragma unroll
         for (int turn = 0; turn < kQueue; ++turn) {
-            if (active && !broken && r.t < r.tmax) {
+            if (active && !broken && n < kQueue && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
