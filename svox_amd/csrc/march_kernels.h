@@ -250,8 +250,8 @@ __device__ __forceinline__ Visit step_octree(const TreeDev<float>& tr, const Ray
 #pragma unroll
     for (int j = 0; j < 3; ++j) pc[j] = clamp01(fma_(r.t, r.d[j], r.o[j]));
     Visit v;
-    const int32_t leaf = cur.seek(tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]), cell_coord(pc[1]),
-                                  cell_coord(pc[2]), kSeekBudget);
+    const int32_t leaf = cur.seek<kSeekBudget>(tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]),
+                                               cell_coord(pc[1]), cell_coord(pc[2]));
     if (leaf == OctreeCursor::kPending) {   // the descent goes on in the lane's next turn
         v.leaf = OctreeCursor::kPending;
         v.levels = 0;

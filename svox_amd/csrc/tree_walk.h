@@ -203,16 +203,16 @@ struct OctreeCursor {
         pend_level = 0;
     }
 
-    // Finds the leaf of the point with integer coordinates (nx, ny, nz), reading at most `budget`
+    // Finds the leaf of the point with integer coordinates (nx, ny, nz), reading at most kBudget
     // child entries.  Returns the leaf cell index; kPending if the budget ran out (call again with
     // the same point to go on); -1 if the tree has more levels than the coordinates hold (`levels`
     // becomes 0).  The budget bounds how long the lanes of a wavefront wait for the one lane that
     // has to descend many levels: that lane continues in its next turn instead.
     // Node ids read from the table are clamped into [0, capacity): a malformed tree yields a wrong
-    // leaf, never an access outside the table.  The loop has a single exit so that lanes which
-    // found their leaf only wait, without extra mask bookkeeping per level.
+    // leaf, never an access outside the table.
+    template <int kBudget>
     __device__ __forceinline__ int32_t seek(const int32_t* __restrict__ child, int32_t last_node,
-                                            uint32_t nx, uint32_t ny, uint32_t nz, int budget) {
+                                            uint32_t nx, uint32_t ny, uint32_t nz) {
         int level = 1;
         int32_t node = 0;
         if (pend_level > 0) {
@@ -229,26 +229,33 @@ struct OctreeCursor {
         } else {
             ix = nx; iy = ny; iz = nz;
         }
-        const int stop_level = level + budget - 1 < kCoordBits ? level + budget - 1 : kCoordBits;
-        int32_t cell, skip;
-        while (true) {
-            path[((level <= kPathLevels ? level : kPathLevels + 1) - 1) * stride] = node;
-            cell = (node << 3) | cell_at(nx, ny, nz, level);
-            // the table is smaller than 4 GiB (checked on the host): a 32-bit byte offset from the
-            // uniform base lets the load use the scalar-base addressing form
-            skip = *(const int32_t*)((const char*)child + ((uint32_t)cell << 2));
-            if (skip == 0 || level == stop_level) break;
-            // a negative or too large id (malformed tree) wraps / clamps to the last node
-            node = (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node);
-            level += 1;
+        // kBudget reads, written out one after the other: no loop bookkeeping between them
+        int32_t cell = 0, skip = 1;
+        bool done = false;
+#pragma unroll
+        for (int it = 0; it < kBudget; ++it) {
+            if (!done) {
+                path[((level <= kPathLevels ? level : kPathLevels + 1) - 1) * stride] = node;
+                cell = (node << 3) | cell_at(nx, ny, nz, level);
+                // the table is smaller than 4 GiB (checked on the host): a 32-bit byte offset from the
+                // uniform base lets the load use the scalar-base addressing form
+                skip = *(const int32_t*)((const char*)child + ((uint32_t)cell << 2));
+                if (skip == 0 || level == kCoordBits) {
+                    done = true;
+                } else {
+                    // a negative or too large id (malformed tree) wraps / clamps to the last node
+                    node = (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node);
+                    level += 1;
+                }
+            }
         }
         pend_level = 0;
         if (skip != 0) {
             levels = 0;   // the path rows written so far stay valid, but there is no previous leaf
             leaf = -1;
-            if (level == kCoordBits) return -1;
-            pend_level = level + 1;
-            pend_node = (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node);
+            if (done) return -1;   // more levels than the coordinates hold
+            pend_level = level;
+            pend_node = node;
             return kPending;
         }
         levels = level;
