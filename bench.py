@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the octree rendering hot path on one MI355X.
 
-Workload "sparse512_sh16" (BASELINE.json configs[2] and [3]): a seeded sparse octree with a 512^3
+Workload "sparse512_sh16" (the headline configuration of this benchmark): a seeded sparse octree with a 512^3
 finest grid refined only near the surface of a union of spheres, SH16 leaf records (49 floats).
   forward  : one step renders 8 poses of 800x800 pixels with step_size 5e-4 and
              sigma_thresh = stop_thresh = 1e-2 through VolumeRenderer.render_persp, all poses in
@@ -55,11 +55,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-bwd", action="store_true", help="skip the forward+backward leg")
     ap.add_argument("--no-query", action="store_true", help="skip the point-query leg")
-    ap.add_argument("--no-large", action="store_true", help="skip the depth-10 SH25 NDC leg (BASELINE configs[4])")
+    ap.add_argument("--no-large", action="store_true", help="skip the depth-10 SH25 NDC leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (rays would shard "
-              "trivially; see DESIGN.md), run with --gpus 1", file=sys.stderr)
+              "trivially across GPUs), run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
@@ -233,7 +233,7 @@ def main():
         tree.data.grad = None
         log(f"[bench] fwd+bwd {fwd_bwd}")
 
-    # ---------------------------------------------------------------- point queries (configs[1])
+    # ---------------------------------------------------------------- point queries (dense 128^3 SH9 tree)
     query = None
     if not args.no_query:
         qtree = synth.dense_tree(6, "SH9", seed=0, sigma="lognormal", coeff_std=0.5, zero_fraction=0.5).to(dev)
@@ -277,7 +277,7 @@ def main():
         del qtree, pts, go, leaves
         log(f"[bench] query {query}")
 
-    # ---------------------------------------------------------------- depth-10 SH25 tree, NDC (configs[4])
+    # ---------------------------------------------------------------- depth-10 SH25 tree, NDC camera
     large = None
     free_bytes, _ = torch.cuda.mem_get_info()
     if not args.no_large and free_bytes > 100 * 2 ** 30:

@@ -176,7 +176,7 @@ def test_full_size_render_properties(gpu):
 
 
 def test_config5_depth10_sh25_ndc_against_the_oracle(gpu, oracle_mod):
-    """BASELINE config 5 at full size: depth-10 octree (42 M leaves, 13.5 GB of SH25 records, more than
+    """The largest benchmark configuration at full size: depth-10 octree (42 M leaves, 13.5 GB of SH25 records, more than
     2^31 elements), forward-facing NDC camera 1008x756.  One whole image, its visit counts, its
     gradient and a million point queries are compared with the CPU oracle."""
     free, _ = torch.cuda.mem_get_info()

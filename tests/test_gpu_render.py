@@ -35,7 +35,7 @@ def render_both(gpu, oracle_mod, tree, rays, opt, generic=0):
 
 @pytest.mark.parametrize("generic", [0, 1])
 def test_config1_rgba_forward_backward(gpu, oracle_mod, generic):
-    """BASELINE config 1: dense 16^3 RGBA tree, 4096 sphere rays, step 1e-3, white background."""
+    """The smallest benchmark configuration: dense 16^3 RGBA tree, 4096 sphere rays, step 1e-3, white background."""
     tree = synth.dense_tree(3, "RGBA", seed=0)
     rays = synth.sphere_rays(4096, seed=0)
     opt = options(tree, step_size=1e-3, background_brightness=1.0)
