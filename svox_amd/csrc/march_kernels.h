@@ -1,14 +1,13 @@
 // march_kernels.h -- ray marching through the leaves of the N^3 tree: forward rendering, its
-// backward pass and the visit counters (reference: svox/csrc/rt_kernel.cu:189-477, 717-844).
+// backward pass, the squared-error gradient / Hessian diagonal, the dense-grid weight render and
+// the visit counters (reference: svox/csrc/rt_kernel.cu:189-1003).
 //
-// Every kernel exists in two flavours that compute the same numbers:
-//   GenericPolicy<T>   any branching factor, scalar type, data format, component range, softplus,
-//                      weight accumulation; the reference's floating-point walk from the root for
-//                      every sample.
+// The tree kernels exist in two flavours that compute the same numbers:
+//   GenericPolicy<T>   any branching factor, scalar type, data format, component range, softplus;
+//                      the reference's floating-point walk from the root for every sample.
 //   OctreePolicy<FMT,D> fp32 octree with the default options (SH with D in {1,4,9,16,25}, or RGBA
 //                      with 3 colours): integer-coordinate walk restarted from the previous path
-//                      (OctreeCursor), record length and basis size known at compile time so the
-//                      basis, the colour accumulators and the dot products live in registers.
+//                      (OctreeCursor), record length and basis size known at compile time.
 #pragma once
 
 #include "basis.h"
@@ -93,7 +92,7 @@ __device__ __forceinline__ void maybe_world2ndc(const SvoxRenderOptions& opt, T*
 }
 
 // Ray sources.  The rays of a launch are numbered 0 .. total()-1 ("items"); a wavefront owns the
-// `per_wave` consecutive items starting at blockIdx.x * per_wave and feeds them to its 64 lanes.
+// `per_wave` consecutive items of chunk chunk_of_block(blockIdx.x) and feeds them to its 64 lanes.
 //   Batch: item i is ray i.
 //   Image: items are numbered so that 64 consecutive items are one 8x8 pixel tile and 256
 //          consecutive items one 16x16 block (four tiles), image after image: the rays a wavefront
@@ -489,9 +488,10 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
 //   refill    lanes whose ray has ended take the next rays of the wavefront's range (ranked by
 //             ballot among the idle lanes) once `refill_at` lanes are idle: rays differ wildly in
 //             length, and a finished lane does not wait for the longest ray of the wavefront;
-//   walk      every live lane advances its ray by up to kQueue leaves and remembers (leaf, step
-//             length) of each: the next position depends only on the tree, not on the leaf's
-//             contents, so this phase waits for child-table reads only;
+//   walk      kQueue turns; in a turn every live lane advances its ray by one leaf and remembers
+//             (leaf, step length), or, if the descent needs more than kSeekBudget child reads,
+//             goes on with it in its next turn.  The next position depends only on the tree, not
+//             on the leaf's contents, so this phase waits for child-table reads only;
 //   sigma     the densities of the remembered leaves are fetched together (kQueue loads in flight);
 //   shade     the leaves with sigma > sigma_thresh of all lanes form one list, and the wavefront
 //             evaluates their colours together (shade_entries), all 64 lanes busy whatever the
