@@ -422,6 +422,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_generic_kernel(T
 }
 
 constexpr int kQueue = 4;  // leaves a lane walks ahead before the wavefront shades them
+static_assert(kQueue <= 4, "ShadeShared::who packs the queue slot into two bits");
 
 // Shade list shared by the wavefront: the (lane, slot) pairs of one round whose leaf has to be
 // shaded, compacted so that consecutive lanes can take consecutive entries.  kRows: the basis of
