@@ -206,6 +206,102 @@ class N3Tree(nn.Module):
     def shrink(self, data_format, data_dim=None, remap=None):
         self.expand(data_format, data_dim, remap)
 
+    # ------------------------------------------------------------------ frontier (nodes whose cells are all leaves)
+    @property
+    def _frontier(self):
+        """Indices of the live nodes all of whose cells are leaves (svox/svox.py:621-633)."""
+        if self._last_frontier is None:
+            n_int = self.n_internal
+            all_leaves = (self.child[:n_int] == 0).reshape(n_int, -1).all(dim=1)
+            live = self.parent_depth[:n_int, 0] != -1
+            self._last_frontier = (all_leaves & live).nonzero(as_tuple=False).reshape(-1)
+        return self._last_frontier
+
+    @property
+    def n_frontier(self):
+        return self._frontier.shape[0]
+
+    @property
+    def frontier_depth(self):
+        """Depth of every frontier node, (n_frontier,)."""
+        return self.parent_depth[self._frontier, 1]
+
+    def reduce_frontier(self, op=torch.mean, dim=None, grad=False):
+        """Apply `op(x, dim=1)` to the (n_frontier, N^3, data_dim) block of child-leaf records of the
+        frontier nodes; `dim` selects data channels first; `grad` keeps the result differentiable
+        with respect to `data` (svox/svox.py:491-530)."""
+        source = self.data if grad else self.data.data
+        block = source[self._frontier].view(-1, self.N ** 3, self.data_dim)
+        if dim is not None:
+            block = block[..., dim]
+        return op(block, dim=1)
+
+    def max_frontier(self, dim=None, grad=False):
+        """reduce_frontier with the maximum over the children (svox/svox.py:532-548)."""
+        return self.reduce_frontier(op=lambda x, dim: torch.max(x, dim=dim)[0], dim=dim, grad=grad)
+
+    def diam_frontier(self, dim=None, grad=False, scale=1.0):
+        """Largest distance between the records of any two children of each frontier node
+        (svox/svox.py:550-580)."""
+        def diameter(x, dim):
+            if x.ndim == 2:
+                x = x[:, :, None]
+            pairwise = torch.cdist(x * scale, x * scale)          # (B, N^3, N^3)
+            return pairwise.reshape(x.shape[0], -1).max(dim=1)[0]
+        return self.reduce_frontier(op=diameter, dim=dim, grad=grad)
+
+    def merge(self, frontier_sel=None, op=torch.mean):
+        """Collapse the selected frontier nodes (default all) into leaves of their parents: the
+        parent cell takes `op` over the N^3 child records (the first result if `op` returns a
+        tuple, as torch.max does), the node is marked free (child and parent link -1) and
+        shrink_to_fit() reclaims it later.  Returns False if nothing was selected
+        (svox/svox.py:436-475)."""
+        if self._lock_tree_structure:
+            raise RuntimeError("Tree locked")
+        if self.n_internal - int(self._n_free.item()) <= 1:
+            raise RuntimeError("Cannot merge root node")
+        nodes = self._frontier if frontier_sel is None else self._frontier[frontier_sel]
+        nodes = nodes.reshape(-1)
+        nodes = nodes[nodes != 0]           # the root has no parent cell to fall back into
+        if nodes.numel() == 0:
+            return False
+        with torch.no_grad():
+            merged = op(self.data.data[nodes].view(-1, self.N ** 3, self.data_dim), dim=1)
+            if isinstance(merged, tuple):
+                merged = merged[0]
+            parent_cells = tuple(self._unpack_index(self.parent_depth[nodes, 0].long()).T)
+            self.data.data[parent_cells] = merged
+            self.child[parent_cells] = 0
+            self.parent_depth[nodes] = -1
+            self.child[nodes] = -1
+            self._n_free += nodes.shape[0]
+        self._invalidate()
+        return True
+
+    # ------------------------------------------------------------------ dense grids
+    @classmethod
+    def from_grid(cls, grid, *args, **kwargs):
+        """Tree with the resolution of the (D, D, D, data_dim) grid `grid`, D a power of two, holding
+        the grid's values (svox/svox.py:868-883).  The tree must live on a GPU (`device=`)."""
+        D = grid.shape[0]
+        assert grid.ndim == 4 and grid.shape[1] == D and grid.shape[2] == D, \
+            "Grid must be a 4D array with first 3 dims equal"
+        log_d = int(math.log2(D))
+        assert 2 ** log_d == D, "Grid size must be power of 2"
+        kwargs["init_refine"] = log_d - 1
+        kwargs.setdefault("data_dim", grid.shape[-1])
+        tree = cls(*args, **kwargs)
+        tree.set_grid(grid)
+        return tree
+
+    def set_grid(self, grid):
+        """Write grid[i, j, k] into the leaf at the centre of grid cell (i, j, k)
+        (svox/svox.py:885-897)."""
+        D = grid.shape[0]
+        assert grid.ndim == 4 and grid.shape[1] == D and grid.shape[2] == D and grid.shape[-1] == self.data_dim
+        centres = gen_grid(D).reshape(-1, 3).to(device=self.data.device, dtype=self.data.dtype)
+        self[LocalIndex(centres)] = grid.reshape(-1, self.data_dim).to(device=self.data.device, dtype=self.data.dtype)
+
     # ------------------------------------------------------------------ structure
     def refine(self, repeats=1, sel=None):
         """Split every selected leaf into N^3 children (respecting depth_limit).
@@ -588,3 +684,9 @@ def gen_grid(D):
     c = (torch.arange(D) + 0.5) / D
     X, Y, Z = torch.meshgrid(c, c, c, indexing="ij")
     return torch.stack([X, Y, Z], -1)
+
+
+def gen_grid(D):
+    """Centres of a D^3 grid over [0, 1]^3, (D, D, D, 3) in xyz order (svox/svox.py:1163-1173)."""
+    axis = (torch.arange(D) + 0.5) / D
+    return torch.stack(torch.meshgrid(axis, axis, axis, indexing="ij"), dim=-1)

@@ -148,3 +148,32 @@ def test_errors_mirror_reference_checks(gpu):
         C.query_vertical(tree._spec(), torch.rand(3, 4, device=gpu).T)
     with pytest.raises(RuntimeError, match="scalar type"):
         C.query_vertical(tree._spec(), torch.rand(4, 3, device=gpu, dtype=torch.float64))
+
+
+def test_from_grid_and_merge_on_the_gpu(gpu, oracle_mod):
+    """from_grid / set_grid write every grid cell into its leaf (svox/svox.py:868-897); a tree with
+    merged (freed) nodes still queries and renders like the oracle."""
+    g = torch.Generator().manual_seed(11)
+    grid = torch.rand(16, 16, 16, 4, generator=g)
+    grid[..., -1] *= 6
+    tree = svox.N3Tree.from_grid(grid, data_format="RGBA", device=gpu)
+    assert tree.n_leaves == 16 ** 3
+    from svox_amd.tree import gen_grid
+    centres = gen_grid(16).reshape(-1, 3).to(gpu)
+    assert torch.equal(tree(centres, world=False).detach().cpu(), grid.reshape(-1, 4))
+    # merge half of the frontier nodes: their node rows become free (-1) inside the table
+    sel = torch.arange(0, tree.n_frontier, 2)
+    assert tree.merge(sel)
+    tree.check_integrity()
+    host = tree.clone(device="cpu")
+    ot = oracle_mod.Tree.from_n3tree(host)
+    pts = torch.rand(5000, 3, generator=g)
+    ref_vals, ref_ids = oracle_mod.query_vertical(ot, pts)
+    vals, ids = tree(pts.to(gpu), want_node_ids=True)
+    assert np.array_equal(ids.cpu().numpy(), ref_ids) and np.array_equal(vals.detach().cpu().numpy(), ref_vals)
+    rays = synth.sphere_rays(2000, seed=3)
+    from util import options, rays_spec
+    opt = options(host, step_size=1e-3)
+    ref = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    out = C.volume_render(tree._spec(), rays_spec(rays, gpu), opt)
+    assert np.array_equal(out.cpu().numpy(), ref)

@@ -217,3 +217,47 @@ def test_generators_are_seeded():
     assert torch.equal(r1.origins, r2.origins) and torch.allclose((r1.origins - 0.5).norm(dim=1), torch.full((10,), 2.0))
     noise = synth.shell_tree(depth=6, data_format="SH1", seed=2, geometry="noise")
     assert noise.check_integrity() and noise.info["occupied_leaves"] > 0
+
+
+def test_frontier_reductions_and_merge():
+    """merge() undoes refine() on frontier nodes; reductions see the N^3 child records
+    (svox/svox.py:436-580)."""
+    tree = svox.N3Tree(N=2, data_format="RGBA", init_refine=1)                 # 1 + 8 nodes, 64 leaves
+    g = torch.Generator().manual_seed(0)
+    tree.data.data.copy_(torch.rand(tree.data.shape, generator=g))
+    assert tree.n_frontier == 8 and (tree.frontier_depth == 1).all()
+    block = tree.data.data[tree._frontier].view(8, 8, 4)
+    assert torch.equal(tree.reduce_frontier(torch.mean), block.mean(dim=1))
+    assert torch.equal(tree.max_frontier(dim=-1), block[..., -1].max(dim=1)[0])
+    diam = tree.diam_frontier()
+    brute = torch.stack([torch.cdist(b, b).max() for b in block])
+    assert torch.allclose(diam, brute)
+    out = tree.reduce_frontier(torch.mean, grad=True)
+    out.sum().backward()
+    assert tree.data.grad is not None and tree.data.grad[1:].abs().sum() > 0
+    tree.data.grad = None
+    # merge three of the eight frontier nodes with max
+    picked = tree._frontier[torch.tensor([0, 3, 5])]
+    want = tree.data.data[picked].view(3, 8, 4).max(dim=1)[0]
+    parents = tuple(tree._unpack_index(tree.parent_depth[picked, 0].long()).T)
+    assert tree.merge(torch.tensor([0, 3, 5]), op=torch.max)
+    assert torch.equal(tree.data.data[parents], want)
+    assert (tree.child[parents] == 0).all() and (tree.child[picked] == -1).all()
+    assert tree.n_leaves == 64 - 3 * 8 + 3 and tree.n_frontier == 5
+    tree.check_integrity()
+    assert tree.shrink_to_fit() and tree.capacity == 6
+    tree.check_integrity()
+    assert tree.n_leaves == 43
+    # merging everything that is left leaves the root alone
+    assert tree.merge()
+    tree.shrink_to_fit()
+    assert tree.capacity == 1 and tree.n_leaves == 8
+    with pytest.raises(RuntimeError, match="Cannot merge root"):
+        tree.merge()
+
+
+def test_gen_grid_centres():
+    from svox_amd.tree import gen_grid
+    grid = gen_grid(4)
+    assert grid.shape == (4, 4, 4, 3)
+    assert torch.allclose(grid[1, 2, 3], torch.tensor([0.375, 0.625, 0.875]))
