@@ -147,17 +147,30 @@ struct ImageSource {
     int per_wave;           // 64 (one 8x8 tile) or 256 (one 16x16 block)
     int refill_at;          // idle lanes that trigger taking new rays
     int xcd_group;          // see chunk_of_block
+    int run;                // > 0: the images advance together, `run` 16x16 blocks at a time
     __device__ __forceinline__ int64_t total() const {
-        return (int64_t)n_images * blocks16_of(cam.width) * blocks16_of(cam.height) * 256;
+        const int64_t per_image = (int64_t)blocks16_of(cam.width) * blocks16_of(cam.height);
+        const int64_t padded = run > 0 ? (per_image + run - 1) / run * run : per_image;
+        return (int64_t)n_images * padded * 256;
     }
     __device__ __forceinline__ int64_t fetch_item(int64_t i, const SvoxRenderOptions& opt, const T* offset,
                                                   const T* scaling, T* origin, T* dir, T* vdir) const {
         const int nbx = blocks16_of(cam.width), nby = blocks16_of(cam.height);
         const int64_t block = i >> 8;
         const int within = (int)(i & 255);
-        const int image = (int)(block / (nbx * nby));
-        if (image >= n_images) return -1;
-        const int b = (int)(block - (int64_t)image * (nbx * nby));
+        int image, b;
+        if (run > 0) {
+            // runs of `run` blocks, image after image, then the next run of every image
+            const int64_t r = block / run;
+            const int64_t round = r / n_images;
+            image = (int)(r - round * n_images);
+            b = (int)(round * run + (block - r * run));
+            if (b >= nbx * nby) return -1;
+        } else {
+            image = (int)(block / (nbx * nby));
+            if (image >= n_images) return -1;
+            b = (int)(block - (int64_t)image * (nbx * nby));
+        }
         const int by = b / nbx, bx = b - by * nbx;
         const int sub = within >> 6, pos = within & 63;
         const int ix = bx * 16 + (sub & 1) * 8 + (pos & 7);

@@ -152,7 +152,8 @@ int check_camera(const SvoxCameraSpec* cam, int n_images = 1, int64_t pose_strid
     if (cam->width < 0 || cam->height < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative image size");
     if (n_images < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative image count");
     if (n_images > 1 && pose_stride < 12) return fail(SVOX_ERR_BAD_SHAPE, "pose_stride must be >= 12 scalars");
-    const double tiles = 4.0 * blocks16_of(cam->width) * blocks16_of(cam->height) * (n_images > 0 ? n_images : 1);
+    // (+ 64: multi-image launches pad every image to a whole number of block runs)
+    const double tiles = 4.0 * ((double)blocks16_of(cam->width) * blocks16_of(cam->height) + 64.0) * (n_images > 0 ? n_images : 1);
     if (tiles >= 2147483647.0) return fail(SVOX_ERR_BAD_SHAPE, "too many pixels for one launch");
     return SVOX_OK;
 }
@@ -233,12 +234,19 @@ ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pos
     s.cam.height = cam->height;
     s.n_images = n_images;
     s.pose_stride = pose_stride;
-    const int64_t total = (int64_t)n_images * blocks16_of(cam->width) * blocks16_of(cam->height) * 256;
     // image tiles are coherent (rays of a tile end together) and only part of an image hits the
     // tree: one tile per wavefront keeps the busy tiles spread over the whole GPU
     s.per_wave = 64;
     s.refill_at = pick_refill();
     s.xcd_group = pick_xcd_group();
+    s.run = 0;
+    if (n_images > 1) {
+        static const int forced = [] {
+            const char* e = getenv("SVOX_IMAGE_RUN");
+            return e ? atoi(e) : -1;
+        }();
+        s.run = forced >= 0 ? forced : 4;
+    }
     return s;
 }
 
@@ -246,7 +254,9 @@ template <typename T>
 int64_t total_items_of(const BatchSource<T>& s) { return s.rays.n_rays; }
 template <typename T>
 int64_t total_items_of(const ImageSource<T>& s) {
-    return (int64_t)s.n_images * blocks16_of(s.cam.width) * blocks16_of(s.cam.height) * 256;
+    const int64_t per_image = (int64_t)blocks16_of(s.cam.width) * blocks16_of(s.cam.height);
+    const int64_t padded = s.run > 0 ? (per_image + s.run - 1) / s.run * s.run : per_image;
+    return (int64_t)s.n_images * padded * 256;
 }
 
 unsigned blocks_for(int64_t items, int per_block) { return (unsigned)((items + per_block - 1) / per_block); }
