@@ -591,30 +591,21 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         }
 
         // ---- walk
+        // slot q holds the leaf found in turn q, or -1 (no live ray, or a descent still under way)
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            q_leaf[q] = 0;
-            q_dt[q] = 0.0f;
-        }
-        int n = 0;
         bool broken = false;
 #pragma unroll
-        for (int turn = 0; turn < kQueue; ++turn) {
-            if (active && !broken && n < kQueue && r.t < r.tmax) {
+        for (int q = 0; q < kQueue; ++q) {
+            q_leaf[q] = -1;
+            q_dt[q] = 0.0f;
+            if (active && !broken && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
-#pragma unroll
-                    for (int q = 0; q < kQueue; ++q) {
-                        if (n == q) {
-                            q_leaf[q] = (int32_t)v.leaf;
-                            q_dt[q] = delta_t;
-                        }
-                    }
+                    q_leaf[q] = (int32_t)v.leaf;
+                    q_dt[q] = delta_t;
                     advance(r, delta_t);
-                    n += 1;
                 } else if (v.leaf != OctreeCursor::kPending) {
                     broken = true;   // malformed tree: the ray ends here
                 }
@@ -624,12 +615,12 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         float q_sigma[kQueue];
 #pragma unroll
         for (int q = 0; q < kQueue; ++q)
-            q_sigma[q] = q < n ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+            q_sigma[q] = q_leaf[q] >= 0 ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
         // ---- shade list
         int n_entries = 0;
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
-            const bool want = q < n && q_sigma[q] > sigma_thresh;
+            const bool want = q_leaf[q] >= 0 && q_sigma[q] > sigma_thresh;
             const unsigned long long m = __ballot(want);
             if (want) {
                 const int e = n_entries + rank_in(m);
@@ -646,7 +637,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
             bool stopped = false;
 #pragma unroll
             for (int q = 0; q < kQueue; ++q) {
-                if (q < n && !stopped && q_sigma[q] > sigma_thresh) {
+                if (q_leaf[q] >= 0 && !stopped && q_sigma[q] > sigma_thresh) {
                     const float att = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
                     const float weight = light * (1.0f - att);
                     const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
@@ -886,30 +877,21 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         }
 
         // ---- walk
+        // slot q holds the leaf found in turn q, or -1 (no live ray, or a descent still under way)
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            q_leaf[q] = 0;
-            q_dt[q] = 0.0f;
-        }
-        int n = 0;
         bool broken = false;
 #pragma unroll
-        for (int turn = 0; turn < kQueue; ++turn) {
-            if (active && !broken && n < kQueue && r.t < r.tmax) {
+        for (int q = 0; q < kQueue; ++q) {
+            q_leaf[q] = -1;
+            q_dt[q] = 0.0f;
+            if (active && !broken && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
-#pragma unroll
-                    for (int q = 0; q < kQueue; ++q) {
-                        if (n == q) {
-                            q_leaf[q] = (int32_t)v.leaf;
-                            q_dt[q] = delta_t;
-                        }
-                    }
+                    q_leaf[q] = (int32_t)v.leaf;
+                    q_dt[q] = delta_t;
                     advance(r, delta_t);
-                    n += 1;
                 } else if (v.leaf != OctreeCursor::kPending) {
                     broken = true;   // malformed tree: the ray ends here
                 }
@@ -919,12 +901,12 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         float q_sigma[kQueue];
 #pragma unroll
         for (int q = 0; q < kQueue; ++q)
-            q_sigma[q] = q < n ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+            q_sigma[q] = q_leaf[q] >= 0 ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
         // ---- shade list
         int n_entries = 0;
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
-            const bool want = q < n && q_sigma[q] > 0.0f;
+            const bool want = q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
             const unsigned long long m = __ballot(want);
             if (want) {
                 const int e = n_entries + rank_in(m);
@@ -942,7 +924,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             bool emit = false;
             float tmp2[3] = {0.f, 0.f, 0.f};
             float g_sigma = 0.f;
-            if (active && q < n && q_sigma[q] > 0.0f) {
+            if (active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f) {
                 const float att = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
                 const float weight = light * (1.0f - att);
                 const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
@@ -1259,30 +1241,21 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         }
 
         // ---- walk
+        // slot q holds the leaf found in turn q, or -1 (no live ray, or a descent still under way)
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            q_leaf[q] = 0;
-            q_dt[q] = 0.0f;
-        }
-        int n = 0;
         bool broken = false;
 #pragma unroll
-        for (int turn = 0; turn < kQueue; ++turn) {
-            if (active && !broken && n < kQueue && r.t < r.tmax) {
+        for (int q = 0; q < kQueue; ++q) {
+            q_leaf[q] = -1;
+            q_dt[q] = 0.0f;
+            if (active && !broken && r.t < r.tmax) {
                 float delta_t;
                 const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
                 if (v.leaf >= 0) {
-#pragma unroll
-                    for (int q = 0; q < kQueue; ++q) {
-                        if (n == q) {
-                            q_leaf[q] = (int32_t)v.leaf;
-                            q_dt[q] = delta_t;
-                        }
-                    }
+                    q_leaf[q] = (int32_t)v.leaf;
+                    q_dt[q] = delta_t;
                     advance(r, delta_t);
-                    n += 1;
                 } else if (v.leaf != OctreeCursor::kPending) {
                     broken = true;   // malformed tree: the ray ends here
                 }
@@ -1292,12 +1265,12 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         float q_sigma[kQueue];
 #pragma unroll
         for (int q = 0; q < kQueue; ++q)
-            q_sigma[q] = q < n ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+            q_sigma[q] = q_leaf[q] >= 0 ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
         // ---- shade list
         int n_entries = 0;
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
-            const bool want = q < n && q_sigma[q] > 0.0f;
+            const bool want = q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
             const unsigned long long m = __ballot(want);
             if (want) {
                 const int e = n_entries + rank_in(m);
@@ -1315,7 +1288,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
             bool emit = false;
             float gci[3] = {0.f, 0.f, 0.f};
             float g_sigma = 0.f, h_sigma = 0.f;
-            if (active && q < n && q_sigma[q] > 0.0f) {
+            if (active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f) {
                 const float att = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
                 const float weight = light * (1.0f - att);
                 const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
