@@ -650,16 +650,17 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                         else
                             atomicAdd(tr.weight_accum + q_leaf[q], weight);
                     }
-                    if (light <= stop_thresh) {
-                        const float scale = (float)(1.0 / (1.0 - (double)light));
-#pragma unroll
-                        for (int c = 0; c < 3; ++c) acc[c] *= scale;
-                        stopped = true;
-                    }
+                    if (light <= stop_thresh) stopped = true;
                 }
             }
             if (stopped || broken || !(r.t < r.tmax)) {
-                if (!stopped) {
+                if (stopped) {
+                    // rt_kernel.cu:306-313: rescale and leave without the background (done here, once
+                    // per round, with the transmittance the ray stopped at)
+                    const float scale = (float)(1.0 / (1.0 - (double)light));
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) acc[c] *= scale;
+                } else {
 #pragma unroll
                     for (int c = 0; c < 3; ++c) acc[c] = fma_(light, bg, acc[c]);
                 }

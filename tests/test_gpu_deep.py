@@ -47,7 +47,7 @@ def test_deep_tree_render(gpu, oracle_mod, levels, fmt):
         assert stats["samples"] == ref_stats["samples"] and stats["levels"] == ref_stats["levels"]
     # gradients on fewer rays: thousands of rays adding into under a hundred leaves would make the
     # fp32 summation order (sequential in the oracle, atomics here) the largest term of the comparison
-    m = 1000
+    m = 300
     sub = svox.Rays(rays.origins[:m].contiguous(), rays.dirs[:m].contiguous(), rays.viewdirs[:m].contiguous())
     rs = rays_spec(sub, gpu)
     go = torch.randn(m, 3, generator=torch.Generator().manual_seed(1))
@@ -79,8 +79,8 @@ def test_deep_tree_queries(gpu, oracle_mod, levels):
     vals, ids = dev(pts.to(gpu), want_node_ids=True)
     assert np.array_equal(ids.cpu().numpy(), ref_ids)
     assert np.array_equal(vals.detach().cpu().numpy(), ref_vals)
-    go = torch.randn(n, tree.data_dim, generator=g)
+    # small integers: thousands of them add up exactly in fp32, whatever the order of the atomics
+    go = torch.randint(-8, 9, (n, tree.data_dim), generator=g).float()
     want = oracle_mod.query_vertical_backward(ot, pts, go)
     got = C.query_vertical_backward(dev._spec(), pts.to(gpu), go.to(gpu)).cpu().numpy()
-    err, ok = grad_close(got, want)
-    assert ok, err
+    assert np.array_equal(got, want)
