@@ -1,5 +1,6 @@
 """Helpers shared by the tests."""
 import copy
+import os
 
 import numpy as np
 import torch
@@ -53,6 +54,8 @@ def grad_close(got, ref, rel=1e-4):
     ref = np.asarray(ref, dtype=np.float64)
     floor = np.abs(ref).max() * 1e-3
     err = np.abs(got - ref) / np.maximum(np.abs(ref), floor if floor > 0 else 1.0)
+    if os.environ.get("SVOX_TEST_VERBOSE"):
+        print(f"[grad_close] worst relative error {float(err.max()):.3e} (limit {rel:.0e})", flush=True)
     return float(err.max()), err.max() <= rel
 
 
