@@ -497,6 +497,78 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
     }
 }
 
+// ---- phases of a round shared by the octree kernels --------------------------------------------
+// Refill: once `refill_at` lanes are idle and the wavefront's range [next, end) is not used up, the
+// idle lanes take the next items, ranked by ballot.  Returns kRoundRefilled (look again), kRoundDone
+// (every lane idle, range used up) or kRoundWork.
+enum RoundState { kRoundWork, kRoundRefilled, kRoundDone };
+template <class Start>
+__device__ __forceinline__ RoundState refill_lanes(bool active, int64_t& next, int64_t end, int refill_at,
+                                                   Start&& start) {
+    const unsigned long long idle = __ballot(!active);
+    const int n_idle = __popcll(idle);
+    if (next < end && n_idle >= refill_at) {
+        if (!active) {
+            const int64_t item = next + rank_in(idle);
+            if (item < end) start(item);
+        }
+        next += n_idle;
+        return kRoundRefilled;
+    }
+    return n_idle == kMarchThreads ? kRoundDone : kRoundWork;
+}
+
+// Walk: kQueue turns; slot q receives the leaf found in turn q and its step length, or -1 (no live
+// ray, or a descent still under way).  `broken` reports a malformed tree: the ray ends there.
+__device__ __forceinline__ void walk_turns(const TreeDev<float>& tr, RayState<float>& r, OctreeCursor& cur,
+                                           float step, bool active, bool& broken, int32_t* q_leaf, float* q_dt,
+                                           int* reads) {
+    broken = false;
+#pragma unroll
+    for (int q = 0; q < kQueue; ++q) {
+        q_leaf[q] = -1;
+        q_dt[q] = 0.0f;
+        if (active && !broken && r.t < r.tmax) {
+            float delta_t;
+            const Visit v = step_octree(tr, r, cur, step, &delta_t, reads);
+            if (v.leaf >= 0) {
+                q_leaf[q] = (int32_t)v.leaf;
+                q_dt[q] = delta_t;
+                advance(r, delta_t);
+            } else if (v.leaf != OctreeCursor::kPending) {
+                broken = true;
+            }
+        }
+    }
+}
+
+// Sigma: the densities of the queued leaves, fetched together (the last scalar of each record).
+template <int K>
+__device__ __forceinline__ void fetch_sigma(const float* __restrict__ data, const int32_t* q_leaf, float* q_sigma) {
+#pragma unroll
+    for (int q = 0; q < kQueue; ++q) q_sigma[q] = q_leaf[q] >= 0 ? data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+}
+
+// Shade list: the (lane, slot) pairs with sigma > thresh, compacted by ballot and prefix count.
+// Returns the number of entries.
+template <class Shared>
+__device__ __forceinline__ int build_shade_list(Shared& sh, const int32_t* q_leaf, const float* q_sigma,
+                                                float thresh, int lane) {
+    int n_entries = 0;
+#pragma unroll
+    for (int q = 0; q < kQueue; ++q) {
+        const bool want = q_leaf[q] >= 0 && q_sigma[q] > thresh;
+        const unsigned long long m = __ballot(want);
+        if (want) {
+            const int e = n_entries + rank_in(m);
+            sh.leaf[e] = q_leaf[q];
+            sh.who[e] = (uint8_t)(lane | (q << 6));
+        }
+        n_entries += __popcll(m);
+    }
+    return n_entries;
+}
+
 // trace_ray, octree flavour: a persistent wavefront working in rounds.
 //
 //   refill    lanes whose ray has ended take the next rays of the wavefront's range (ranked by
@@ -574,61 +646,23 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
 
     while (true) {
         if constexpr (kRefill) {
-            // ---- refill
-            const unsigned long long idle = __ballot(!active);
-            const int n_idle = __popcll(idle);
-            if (next < end && n_idle >= src.refill_at) {
-                if (!active) {
-                    const int64_t item = next + rank_in(idle);
-                    if (item < end) start(item);
-                }
-                next += n_idle;
-                continue;
-            }
-            if (n_idle == kMarchThreads) break;
+            const RoundState state = refill_lanes(active, next, end, src.refill_at, start);
+            if (state == kRoundRefilled) continue;
+            if (state == kRoundDone) break;
         } else {
             if (!__any(active)) break;
         }
 
         // ---- walk
-        // slot q holds the leaf found in turn q, or -1 (no live ray, or a descent still under way)
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-        bool broken = false;
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            q_leaf[q] = -1;
-            q_dt[q] = 0.0f;
-            if (active && !broken && r.t < r.tmax) {
-                float delta_t;
-                const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
-                if (v.leaf >= 0) {
-                    q_leaf[q] = (int32_t)v.leaf;
-                    q_dt[q] = delta_t;
-                    advance(r, delta_t);
-                } else if (v.leaf != OctreeCursor::kPending) {
-                    broken = true;   // malformed tree: the ray ends here
-                }
-            }
-        }
+        bool broken;
+        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt, &reads);
         // ---- sigma
         float q_sigma[kQueue];
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q)
-            q_sigma[q] = q_leaf[q] >= 0 ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
         // ---- shade list
-        int n_entries = 0;
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            const bool want = q_leaf[q] >= 0 && q_sigma[q] > sigma_thresh;
-            const unsigned long long m = __ballot(want);
-            if (want) {
-                const int e = n_entries + rank_in(m);
-                sh.leaf[e] = q_leaf[q];
-                sh.who[e] = (uint8_t)(lane | (q << 6));
-            }
-            n_entries += __popcll(m);
-        }
+        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, sigma_thresh, lane);
         __syncthreads();   // one wavefront per block: list and basis rows are visible to every lane
         shade_entries<P, false>(tr.data, sh, n_entries, lane);
         __syncthreads();
@@ -861,61 +895,23 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 
     while (true) {
         if constexpr (kRefill) {
-            // ---- refill
-            const unsigned long long idle = __ballot(!active);
-            const int n_idle = __popcll(idle);
-            if (next < end && n_idle >= src.refill_at) {
-                if (!active) {
-                    const int64_t item = next + rank_in(idle);
-                    if (item < end) start(item);
-                }
-                next += n_idle;
-                continue;
-            }
-            if (n_idle == kMarchThreads) break;
+            const RoundState state = refill_lanes(active, next, end, src.refill_at, start);
+            if (state == kRoundRefilled) continue;
+            if (state == kRoundDone) break;
         } else {
             if (!__any(active)) break;
         }
 
         // ---- walk
-        // slot q holds the leaf found in turn q, or -1 (no live ray, or a descent still under way)
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-        bool broken = false;
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            q_leaf[q] = -1;
-            q_dt[q] = 0.0f;
-            if (active && !broken && r.t < r.tmax) {
-                float delta_t;
-                const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
-                if (v.leaf >= 0) {
-                    q_leaf[q] = (int32_t)v.leaf;
-                    q_dt[q] = delta_t;
-                    advance(r, delta_t);
-                } else if (v.leaf != OctreeCursor::kPending) {
-                    broken = true;   // malformed tree: the ray ends here
-                }
-            }
-        }
+        bool broken;
+        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt, &reads);
         // ---- sigma
         float q_sigma[kQueue];
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q)
-            q_sigma[q] = q_leaf[q] >= 0 ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
         // ---- shade list
-        int n_entries = 0;
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            const bool want = q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
-            const unsigned long long m = __ballot(want);
-            if (want) {
-                const int e = n_entries + rank_in(m);
-                sh.leaf[e] = q_leaf[q];
-                sh.who[e] = (uint8_t)(lane | (q << 6));
-            }
-            n_entries += __popcll(m);
-        }
+        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane);
         __syncthreads();
         shade_entries<P, true>(tr.data, sh, n_entries, lane);
         __syncthreads();
@@ -1225,61 +1221,23 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
 
     while (true) {
         if constexpr (kRefill) {
-            // ---- refill
-            const unsigned long long idle = __ballot(!active);
-            const int n_idle = __popcll(idle);
-            if (next < end && n_idle >= src.refill_at) {
-                if (!active) {
-                    const int64_t item = next + rank_in(idle);
-                    if (item < end) start(item);
-                }
-                next += n_idle;
-                continue;
-            }
-            if (n_idle == kMarchThreads) break;
+            const RoundState state = refill_lanes(active, next, end, src.refill_at, start);
+            if (state == kRoundRefilled) continue;
+            if (state == kRoundDone) break;
         } else {
             if (!__any(active)) break;
         }
 
         // ---- walk
-        // slot q holds the leaf found in turn q, or -1 (no live ray, or a descent still under way)
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
-        bool broken = false;
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            q_leaf[q] = -1;
-            q_dt[q] = 0.0f;
-            if (active && !broken && r.t < r.tmax) {
-                float delta_t;
-                const Visit v = step_octree(tr, r, cur, step, &delta_t, &reads);
-                if (v.leaf >= 0) {
-                    q_leaf[q] = (int32_t)v.leaf;
-                    q_dt[q] = delta_t;
-                    advance(r, delta_t);
-                } else if (v.leaf != OctreeCursor::kPending) {
-                    broken = true;   // malformed tree: the ray ends here
-                }
-            }
-        }
+        bool broken;
+        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt, &reads);
         // ---- sigma
         float q_sigma[kQueue];
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q)
-            q_sigma[q] = q_leaf[q] >= 0 ? tr.data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
+        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
         // ---- shade list
-        int n_entries = 0;
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            const bool want = q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
-            const unsigned long long m = __ballot(want);
-            if (want) {
-                const int e = n_entries + rank_in(m);
-                sh.leaf[e] = q_leaf[q];
-                sh.who[e] = (uint8_t)(lane | (q << 6));
-            }
-            n_entries += __popcll(m);
-        }
+        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane);
         __syncthreads();
         shade_entries<P, true>(tr.data, sh, n_entries, lane);
         __syncthreads();
