@@ -223,7 +223,7 @@ def main():
         bbytes = backward_bytes(train_stats, B, K, 36 + 12, data_bytes)
         fwd_bwd = {
             "value": round(B / (tb_ms * 1e-3) / 1e6, 3), "unit": "Mrays/s", "rays": B,
-            "ms_per_step": round(tb_ms, 3), "includes": "forward + backward (zero-fill, 2 marches, atomics) + SGD update",
+            "ms_per_step": round(tb_ms, 3), "includes": "forward + backward (zero-fill, march + replay from a 768 B/ray workspace, atomics) + SGD update",
             "backward_ms": round(bwd_ms, 3),
             "backward_algorithmic_gbs": round(bbytes / (bwd_ms * 1e-3) / 1e9, 2),
             "backward_frac_of_peak": round(bbytes / (bwd_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 5),

@@ -180,6 +180,24 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
                                 const SvoxRenderOptions* opt, const void* grad_output,
                                 void* grad_data_out, int32_t accumulate, void* stream);
 
+/* No counterpart in the reference.  svox_volume_render_backward with a workspace in device memory
+ * (8-byte aligned, any contents, overwritten): while the first of the two marches of a ray passes
+ * the leaves with sigma > 0, the kernel notes in the workspace what the second march needs of them
+ * (24 bytes per leaf, in chunks of 384 bytes = 15 leaves and a link); a ray whose notes fit is not
+ * marched a second time, the others are.  The first n_rays chunks are the rays' own; the rest of
+ * the workspace is shared out among the wavefronts for rays with more than 15 such leaves, so the
+ * workspace holds workspace_bytes / 384 chunks and is useful from n_rays chunks on.
+ * The gradient is the one svox_volume_render_backward gives (the same terms; the order of the
+ * atomic additions differs from call to call either way).  Without a workspace (NULL, or fewer
+ * than n_rays chunks), for fp64 trees and wherever the generic kernels run, the call is
+ * svox_volume_render_backward.  svox_volume_render_backward_workspace_bytes gives the size that
+ * holds `records_per_ray` leaves per ray on average (rounded up to whole chunks). */
+int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                                   const SvoxRenderOptions* opt, const void* grad_output,
+                                   void* grad_data_out, int32_t accumulate, void* workspace,
+                                   int64_t workspace_bytes, void* stream);
+int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray);
+
 /* volume_render_image_backward(TreeSpec&, CameraSpec&, RenderOptions&, grad_output);
  * rt_kernel.cu:1085-1109.  grad_output (H, W, out_dim). */
 int svox_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,

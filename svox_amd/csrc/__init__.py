@@ -368,18 +368,37 @@ def _check_grad(grad_output, shape, dtype):
         raise RuntimeError(f"grad_output must have shape {tuple(shape)}, got {tuple(grad_output.shape)}")
 
 
-def volume_render_backward(tree, rays, opt, grad_output):
-    """zeros_like(tree.data) + scatter; rt_kernel.cu:1059-1083"""
+# Leaves per ray (on average) the backward's workspace has room for, and the most memory it may take.
+BACKWARD_RECORDS_PER_RAY = 30
+BACKWARD_WORKSPACE_LIMIT = 1 << 30
+
+
+def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
+    """zeros_like(tree.data) + scatter; rt_kernel.cu:1059-1083.
+
+    workspace: let the kernel note, during the first march, the leaves the second march needs, so
+    that a ray whose notes fit is marched once (fp32 octrees; room for BACKWARD_RECORDS_PER_RAY
+    leaves per ray on average, at most BACKWARD_WORKSPACE_LIMIT bytes, from torch's allocator).
+    The gradient is the same."""
     spec = _pack_tree(tree)
     rspec = _pack_rays(rays, tree.data.dtype)
     od = _render_out_dim(spec, opt)
     _check_grad(grad_output, (rspec.n_rays, od), tree.data.dtype)
     grad = torch.empty_like(tree.data)
     copt = opt._pack()
+    ws, ws_bytes = None, 0
+    if workspace and rspec.n_rays > 0 and tree.data.dtype == torch.float32:
+        size_of = _abi.load_library().svox_volume_render_backward_workspace_bytes
+        per_ray = int(BACKWARD_RECORDS_PER_RAY)
+        while per_ray > 0 and size_of(rspec.n_rays, per_ray) > BACKWARD_WORKSPACE_LIMIT:
+            per_ray -= 15
+        ws_bytes = int(size_of(rspec.n_rays, per_ray)) if per_ray > 0 else 0
+        if ws_bytes > 0:
+            ws = torch.empty(ws_bytes // 8, dtype=torch.float64, device=tree.data.device)
     with torch.cuda.device(tree.data.device):
-        _call("svox_volume_render_backward", ctypes.byref(spec), ctypes.byref(rspec),
+        _call("svox_volume_render_backward_ws", ctypes.byref(spec), ctypes.byref(rspec),
               ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
-              _stream(tree.data.device))
+              ws.data_ptr() if ws is not None else None, ws_bytes, _stream(tree.data.device))
     return grad
 
 

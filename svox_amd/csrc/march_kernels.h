@@ -17,6 +17,13 @@ namespace svox {
 
 constexpr int kMarchThreads = 64;  // one wavefront per block: finished tiles free their slot at once
 
+// Orders the LDS traffic of the block's single wavefront: what a lane wrote before is read by
+// any lane after.  The hardware keeps a wavefront's LDS operations in order; this keeps the compiler
+// from moving them across and waits for the LDS counter only.  (__syncthreads would also wait for
+// every outstanding global load, store and atomic of the wavefront -- the gradient atomics, which
+// nothing here has to wait for.)
+__device__ __forceinline__ void wave_lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
 // ------------------------------------------------------------------------------------------------
 // ray sources
 // ------------------------------------------------------------------------------------------------
@@ -549,15 +556,15 @@ __device__ __forceinline__ void fetch_sigma(const float* __restrict__ data, cons
     for (int q = 0; q < kQueue; ++q) q_sigma[q] = q_leaf[q] >= 0 ? data[(int64_t)q_leaf[q] * K + (K - 1)] : 0.0f;
 }
 
-// Shade list: the (lane, slot) pairs with sigma > thresh, compacted by ballot and prefix count.
-// Returns the number of entries.
+// Shade list: the (lane, slot) pairs with sigma > thresh, compacted by ballot and prefix count
+// (`skip`: none of this lane's).  Returns the number of entries.
 template <class Shared>
 __device__ __forceinline__ int build_shade_list(Shared& sh, const int32_t* q_leaf, const float* q_sigma,
-                                                float thresh, int lane) {
+                                                float thresh, int lane, bool skip = false) {
     int n_entries = 0;
 #pragma unroll
     for (int q = 0; q < kQueue; ++q) {
-        const bool want = q_leaf[q] >= 0 && q_sigma[q] > thresh;
+        const bool want = !skip && q_leaf[q] >= 0 && q_sigma[q] > thresh;
         const unsigned long long m = __ballot(want);
         if (want) {
             const int e = n_entries + rank_in(m);
@@ -663,9 +670,9 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);
         // ---- shade list
         const int n_entries = build_shade_list(sh, q_leaf, q_sigma, sigma_thresh, lane);
-        __syncthreads();   // one wavefront per block: list and basis rows are visible to every lane
+        wave_lds_sync();   // list and view directions are visible to every lane
         shade_entries<P, false>(tr.data, sh, n_entries, lane);
-        __syncthreads();
+        wave_lds_sync();
         // ---- composite
         if (active) {
             bool stopped = false;
@@ -838,11 +845,74 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
 // summed first, so that leaf receives one atomic per element instead of one per ray.  The per-term
 // products are the reference's; only the order in which they are added up differs.
 // Both marches test sigma > 0 and never stop early (rt_kernel.cu:377, 441).
-template <class P, class Source, bool kRefill>
+// Adds the gradient records of one queue slot.  A record is the K-long vector
+// (basis[i] * tmp2[c] for the colour coefficients, g_sigma last) of a lane whose `emit` is set, to
+// be added at leaf `leaf`.  The records of the slot are listed in LDS (in parts of ShadeShared that
+// are dead by now: the shade list and the slot's colours), and the wavefront adds the n * K
+// scalars of the list flat, element f of the list from lane f mod 64: every atomic instruction
+// covers 64 consecutive scalars of at most 64 / K + 2 records, whatever K is.
+template <class P, int D>
+__device__ __forceinline__ void emit_records(ShadeShared<D, true>& sh, int q, bool emit, int32_t leaf,
+                                             const float* tmp2, float g_sigma, int lane,
+                                             float* __restrict__ grad_data) {
+    constexpr int K = P::kRecord;
+    const unsigned long long todo = __ballot(emit);
+    const int n = __popcll(todo);
+    if (n == 0) return;
+    float* list_t = sh.colour + q * (kMarchThreads * 3);          // [record][channel]
+    float* list_gs = (float*)(sh.leaf + kMarchThreads);            // [record]
+    if (emit) {
+        const int rec = rank_in(todo);
+        sh.leaf[rec] = leaf;
+        sh.who[rec] = (uint8_t)lane;
+        list_gs[rec] = g_sigma;
+        list_t[rec * 3] = tmp2[0];
+        list_t[rec * 3 + 1] = tmp2[1];
+        list_t[rec * 3 + 2] = tmp2[2];
+    }
+    wave_lds_sync();
+    const int total = n * K;
+    for (int f = lane; f < total; f += kMarchThreads) {
+        const int rec = f / K, e = f - rec * K;
+        float val;
+        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+            val = e < 3 ? list_t[rec * 3 + e] : list_gs[rec];
+        } else {
+            if (e < 3 * D) {
+                const int c = e / D;
+                val = sh.basis[sh.who[rec] * D + (e - c * D)] * list_t[rec * 3 + c];
+            } else {
+                val = list_gs[rec];
+            }
+        }
+        atomicAdd(grad_data + (int64_t)sh.leaf[rec] * K + e, val);
+    }
+    wave_lds_sync();
+}
+
+// Workspace of the replaying backward: chunks of kChunkRecords records of 3 float2 (leaf and step
+// length, attenuation and first sigmoid, the other two sigmoids) followed by one float2 whose x
+// holds the index of the ray's next chunk.  Ray number i starts in chunk i; further chunks come
+// from a part of the workspace that belongs to the wavefront (no atomics: the lanes that need a
+// chunk in the same step are ranked by ballot).
+constexpr int kChunkRecords = 15;
+constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
+struct ReplaySpace {
+    float2* base;          // chunk c starts at base + c * kChunkFloat2
+    int64_t first_shared;  // chunks [0, first_shared) are the rays' first chunks
+    int32_t per_block;     // chunks of the shared part that belong to one block
+};
+
+// kReplay: during march 1 a lane notes, for every leaf with sigma > 0, what march 2 needs of it; if
+// the notes fit into the workspace, march 2 does not walk the tree again but replays them (a ray
+// with no such leaf is finished on the spot), otherwise it marches as without a workspace.  The
+// duration of a launch is set by its longest rays: halving their second march is what this buys.
+template <class P, class Source, bool kRefill, bool kReplay>
 __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<float> tr, Source src,
                                                                         SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
-                                                                        float* __restrict__ grad_data) {
+                                                                        float* __restrict__ grad_data,
+                                                                        ReplaySpace ws) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
@@ -859,10 +929,20 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     const int64_t total = src.total();
     const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
+    enum { kMarch1 = 0, kMarch2 = 1, kReplaying = 2 };
     RayState<float> r;
     float go[3] = {0.f, 0.f, 0.f};
     float light = 1.0f, accum = 0.0f, tmin = 0.0f;
-    bool active = false, second = false;
+    bool active = false;
+    int phase = kMarch1;
+    // notes of march 1: total count, the chunk being written / read and the position in it
+    int rec_count = 0, rec_next = 0, rec_pos = 0;
+    int32_t rec_link = 0;              // replay: index of the chunk after rec_chunk
+    bool rec_lost = false;             // the workspace ran out: this ray marches twice
+    float2* rec_first = ws.base;
+    float2* rec_chunk = ws.base;
+    int64_t shared_next = ws.first_shared + (int64_t)blockIdx.x * ws.per_block;   // wavefront-uniform
+    const int64_t shared_end = shared_next + ws.per_block;
     int reads = 0;
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
@@ -885,7 +965,14 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             accum = 0.0f;
             tmin = r.t;
             cur.restart();
-            second = false;
+            phase = kMarch1;
+            if constexpr (kReplay) {
+                rec_count = 0;
+                rec_pos = 0;
+                rec_lost = false;
+                rec_first = ws.base + slot * kChunkFloat2;
+                rec_chunk = rec_first;
+            }
             active = true;
         }
     };
@@ -902,35 +989,83 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             if (!__any(active)) break;
         }
 
-        // ---- walk
+        // ---- walk (lanes that replay their notes do not walk)
+        const bool replaying = kReplay && phase == kReplaying;
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
         bool broken;
-        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt, &reads);
-        // ---- sigma
         float q_sigma[kQueue];
-        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
-        // ---- shade list
-        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane);
-        __syncthreads();
-        shade_entries<P, true>(tr.data, sh, n_entries, lane);
-        __syncthreads();
+        const bool any_walk = !kReplay || __any(active && !replaying);
+        if (any_walk) {
+            walk_turns(tr, r, cur, step, active && !replaying, broken, q_leaf, q_dt, &reads);
+            // ---- sigma
+            fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+        } else {
+            // every lane left replays: a round without the tree
+            broken = false;
+#pragma unroll
+            for (int q = 0; q < kQueue; ++q) {
+                q_leaf[q] = -1;
+                q_dt[q] = 0.0f;
+                q_sigma[q] = 0.0f;
+            }
+        }
+        // ---- replayed leaves: the next kQueue notes take the slots; q_sigma holds their attenuation.
+        // Their loads are in flight together with the density loads of the walking lanes.
+        if constexpr (kReplay) {
+            if (active && replaying) {
+#pragma unroll
+                for (int q = 0; q < kQueue; ++q) {
+                    if (rec_next + q < rec_count) {
+                        if (rec_pos == kChunkRecords) {
+                            // the link was read when this chunk was entered: no load to wait for here
+                            rec_chunk = ws.base + (int64_t)rec_link * kChunkFloat2;
+                            rec_link = __float_as_int(rec_chunk[kChunkRecords * 3].x);
+                            rec_pos = 0;
+                        }
+                        const float2* e = rec_chunk + rec_pos * 3;
+                        const float2 a = e[0], b = e[1], c = e[2];
+                        rec_pos += 1;
+                        q_leaf[q] = __float_as_int(a.x);
+                        q_dt[q] = a.y;
+                        q_sigma[q] = b.x;
+                        float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+                        s[0] = b.y;
+                        s[1] = c.x;
+                        s[2] = c.y;
+                    }
+                }
+            }
+        }
+        // ---- shade list (walking lanes only)
+        const int n_entries = any_walk ? build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane, replaying) : 0;
+        wave_lds_sync();
+        if (n_entries > 0) shade_entries<P, true>(tr.data, sh, n_entries, lane);
+        wave_lds_sync();
         // ---- composite and emit, slot by slot
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
-            bool emit = false;
+            bool emit = false, note = false;
             float tmp2[3] = {0.f, 0.f, 0.f};
-            float g_sigma = 0.f;
-            if (active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f) {
-                const float att = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
+            float g_sigma = 0.f, note_att = 0.f;
+            float note_s[3] = {0.f, 0.f, 0.f};
+            if (active && q_leaf[q] >= 0 && (replaying || q_sigma[q] > 0.0f)) {
+                const float att = replaying ? q_sigma[q] : expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
                 const float weight = light * (1.0f - att);
                 const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
                 float total_color = 0.0f;
 #pragma unroll
                 for (int c = 0; c < 3; ++c) total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
                 light *= att;
-                if (!second) {
+                if (phase == kMarch1) {
                     accum = fma_(weight, total_color, accum);
+                    if constexpr (kReplay) {
+                        note = true;
+                        note_att = att;
+                        note_s[0] = s[0];
+                        note_s[1] = s[1];
+                        note_s[2] = s[2];
+                    }
                 } else {
 #pragma unroll
                     for (int c = 0; c < 3; ++c) {
@@ -946,50 +1081,60 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                     emit = true;
                 }
             }
-            unsigned long long todo = __ballot(emit);
-            while (todo) {
-                const int leader = __ffsll((long long)todo) - 1;
-                const int32_t leaf_l = __builtin_amdgcn_readlane(q_leaf[q], leader);
-                const unsigned long long same = __ballot(emit && q_leaf[q] == leaf_l);
-                todo &= ~same;
-                float* g = grad_data + (int64_t)leaf_l * K;
-#pragma unroll
-                for (int e0 = 0; e0 < K; e0 += 64) {
-                    const int e = e0 + lane;
-                    float val = 0.0f;
-                    unsigned long long members = same;
-                    while (members) {
-                        const int k = __ffsll((long long)members) - 1;
-                        members &= members - 1;
-                        const float t0 = read_lane(tmp2[0], k);
-                        const float t1 = read_lane(tmp2[1], k);
-                        const float t2 = read_lane(tmp2[2], k);
-                        const float gs = read_lane(g_sigma, k);
-                        float term;
-                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                            term = e == 0 ? t0 : e == 1 ? t1 : e == 2 ? t2 : gs;
+            if constexpr (kReplay) {
+                // lanes whose chunk is full take the next chunks of the wavefront's share, in lane order
+                const bool need = note && !rec_lost && rec_pos == kChunkRecords;
+                const unsigned long long m = __ballot(need);
+                if (m) {
+                    const int64_t mine = shared_next + rank_in(m);
+                    if (need) {
+                        if (mine < shared_end) {
+                            rec_chunk[kChunkRecords * 3] = make_float2(__int_as_float((int32_t)mine), 0.0f);
+                            rec_chunk = ws.base + mine * kChunkFloat2;
+                            rec_pos = 0;
                         } else {
-                            const int c = e / D;
-                            const float b = e < 3 * D ? sh.basis[k * D + (e - c * D)] : 0.0f;
-                            const float tc = c == 0 ? t0 : c == 1 ? t1 : t2;
-                            term = e < 3 * D ? b * tc : gs;
+                            rec_lost = true;
                         }
-                        val += term;
                     }
-                    if (e < K) atomicAdd(g + e, val);
+                    shared_next += __popcll(m);
+                }
+                if (note) {
+                    if (!rec_lost) {
+                        float2* e = rec_chunk + rec_pos * 3;
+                        e[0] = make_float2(__int_as_float(q_leaf[q]), q_dt[q]);
+                        e[1] = make_float2(note_att, note_s[0]);
+                        e[2] = make_float2(note_s[1], note_s[2]);
+                        rec_pos += 1;
+                    }
+                    rec_count += 1;
                 }
             }
+            emit_records<P, D>(sh, q, emit, q_leaf[q], tmp2, g_sigma, lane, grad_data);
         }
         // ---- end of a march
-        if (active && (broken || !(r.t < r.tmax))) {
-            if (!second && !broken) {
-                const float total_grad = (go[0] + go[1]) + go[2];
-                accum = fma_(light * bg, total_grad, accum);
-                light = 1.0f;
-                r.t = tmin;
-                second = true;
-            } else {
-                active = false;
+        if (active) {
+            if (replaying) {
+                rec_next += kQueue;
+                if (rec_next >= rec_count) active = false;
+            } else if (broken || !(r.t < r.tmax)) {
+                if (phase == kMarch1 && !broken) {
+                    const float total_grad = (go[0] + go[1]) + go[2];
+                    accum = fma_(light * bg, total_grad, accum);
+                    light = 1.0f;
+                    if (kReplay && !rec_lost) {
+                        phase = kReplaying;
+                        rec_next = 0;
+                        rec_pos = 0;
+                        rec_chunk = rec_first;
+                        rec_link = __float_as_int(rec_first[kChunkRecords * 3].x);   // garbage if there is none
+                        if (rec_count == 0) active = false;   // no leaf with sigma > 0: nothing to add
+                    } else {
+                        phase = kMarch2;
+                        r.t = tmin;
+                    }
+                } else {
+                    active = false;
+                }
             }
         }
     }
@@ -1238,9 +1383,9 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);
         // ---- shade list
         const int n_entries = build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane);
-        __syncthreads();
+        wave_lds_sync();
         shade_entries<P, true>(tr.data, sh, n_entries, lane);
-        __syncthreads();
+        wave_lds_sync();
         // ---- composite and emit, slot by slot
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {

@@ -300,23 +300,36 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
                        dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (T*)out);
 }
 
+constexpr int64_t kChunkBytes = (int64_t)kChunkFloat2 * 8;   // 384: 15 records and a link
+
 template <class Source, typename T>
 void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, int out_dim,
-                     const void* grad_out, void* grad_data, hipStream_t stream) {
+                     const void* grad_out, void* grad_data, void* workspace, int64_t workspace_bytes,
+                     int64_t n_slots, hipStream_t stream) {
     const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
-            if (src.per_wave > kMarchThreads) {
-                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, true>), dim3(blocks),
-                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                           src, *opt, (const float*)grad_out, (float*)grad_data));
-            } else {
-                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, false>), dim3(blocks),
-                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                           src, *opt, (const float*)grad_out, (float*)grad_data));
+            // every ray owns one chunk; what is left of the workspace is dealt out to the blocks
+            ReplaySpace ws{nullptr, 0, 0};
+            const int64_t chunks = workspace ? workspace_bytes / kChunkBytes : 0;
+            if (n_slots > 0 && chunks >= n_slots && chunks < 0x7fffffffll && ((uintptr_t)workspace & 7u) == 0) {
+                ws.base = (float2*)workspace;
+                ws.first_shared = n_slots;
+                ws.per_block = (int32_t)((chunks - n_slots) / blocks);
             }
+#define SVOX_LAUNCH_BACKWARD(REFILL, REPLAY)                                                                     \
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, REFILL, REPLAY>), dim3(blocks), \
+                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), src,       \
+                                               *opt, (const float*)grad_out, (float*)grad_data, ws))
+            const bool refill = src.per_wave > kMarchThreads;
+            if (ws.base) {
+                if (refill) { SVOX_LAUNCH_BACKWARD(true, true); } else { SVOX_LAUNCH_BACKWARD(false, true); }
+            } else {
+                if (refill) { SVOX_LAUNCH_BACKWARD(true, false); } else { SVOX_LAUNCH_BACKWARD(false, false); }
+            }
+#undef SVOX_LAUNCH_BACKWARD
             return;
         }
     }
@@ -518,6 +531,19 @@ int svox_volume_render_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam
 
 int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
                                 const void* grad_output, void* grad_data_out, int32_t accumulate, void* stream) {
+    return svox_volume_render_backward_ws(tree, rays, opt, grad_output, grad_data_out, accumulate, nullptr, 0,
+                                          stream);
+}
+
+int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray) {
+    if (n_rays <= 0 || records_per_ray <= 0) return 0;
+    const int64_t chunks_per_ray = (records_per_ray + kChunkRecords - 1) / kChunkRecords;
+    return n_rays * chunks_per_ray * kChunkBytes;
+}
+
+int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
+                                   const void* grad_output, void* grad_data_out, int32_t accumulate,
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
     int od;
     int rc = check_render(tree, opt, &od);
     if (rc) return rc;
@@ -530,12 +556,14 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
     }
     if (rays->n_rays == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
+    if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
     if (tree->dtype == SVOX_F32)
         launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays, true), opt, od, grad_output,
-                                                   grad_data_out, (hipStream_t)stream);
+                                                   grad_data_out, workspace, workspace_bytes, rays->n_rays,
+                                                   (hipStream_t)stream);
     else
         launch_backward<BatchSource<double>, double>(tree, batch_source<double>(rays, true), opt, od, grad_output,
-                                                     grad_data_out, (hipStream_t)stream);
+                                                     grad_data_out, nullptr, 0, 0, (hipStream_t)stream);
     return check_launch("volume_render_backward");
 }
 
@@ -557,11 +585,11 @@ int svox_volume_render_images_backward(const SvoxTreeSpec* tree, const SvoxCamer
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
     if (tree->dtype == SVOX_F32) {
         const auto src = image_source<float>(cam, n_images, pose_stride);
-        launch_backward<ImageSource<float>, float>(tree, src, opt, od, grad_output, grad_data_out,
+        launch_backward<ImageSource<float>, float>(tree, src, opt, od, grad_output, grad_data_out, nullptr, 0, 0,
                                                    (hipStream_t)stream);
     } else {
         const auto src = image_source<double>(cam, n_images, pose_stride);
-        launch_backward<ImageSource<double>, double>(tree, src, opt, od, grad_output, grad_data_out,
+        launch_backward<ImageSource<double>, double>(tree, src, opt, od, grad_output, grad_data_out, nullptr, 0, 0,
                                                      (hipStream_t)stream);
     }
     return check_launch("volume_render_image_backward");

@@ -305,3 +305,24 @@ def test_pathological_rays_end_and_match_the_oracle(gpu, oracle_mod, fmt):
         assert np.array_equal(np.isfinite(grad), finite)
         err, ok = grad_close(np.where(finite, grad, 0.0), np.where(finite, ref_grad, 0.0))
         assert ok, err
+
+
+@pytest.mark.parametrize("fmt", ["SH9", "RGBA"])
+def test_backward_workspace_sizes(gpu, oracle_mod, fmt, monkeypatch):
+    """The backward with a workspace (march 2 replayed from notes of march 1) for shares of the
+    workspace that hold none, some and all of the rays' leaves, and without a workspace: the same
+    gradient as the oracle's every time."""
+    tree = synth.shell_tree(depth=6, n_spheres=6, data_format=fmt, seed=9, sigma_range=(2.0, 20.0))
+    rays = synth.sphere_rays(6000, seed=4)
+    opt = options(tree, step_size=1e-3)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    go = torch.randn(6000, 3, generator=torch.Generator().manual_seed(5))
+    want, stats = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go, want_stats=True)
+    assert stats["samples_bwd_pos"] > 8 * 6000          # many rays have more than 4 and 8 such leaves
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    for per_ray in (0, 15, 30, 90):      # no workspace; first chunks only; some / plenty of shared chunks
+        monkeypatch.setattr(C, "BACKWARD_RECORDS_PER_RAY", per_ray)
+        got = C.volume_render_backward(dev._spec(), rs, opt, go.to(gpu), workspace=per_ray > 0).cpu().numpy()
+        err, ok = grad_close(got, want)
+        assert ok, (per_ray, err)
