@@ -370,7 +370,7 @@ def _check_grad(grad_output, shape, dtype):
 
 # Leaves per ray (on average) the backward's workspace has room for, and the most memory it may take.
 BACKWARD_RECORDS_PER_RAY = 30
-BACKWARD_WORKSPACE_LIMIT = 1 << 30
+BACKWARD_WORKSPACE_LIMIT = 4 << 30
 
 
 def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
