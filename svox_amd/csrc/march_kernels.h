@@ -10,6 +10,8 @@
 //                      (OctreeCursor), record length and basis size known at compile time.
 #pragma once
 
+#include <cstddef>
+
 #include "basis.h"
 #include "tree_walk.h"
 
@@ -845,50 +847,75 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
 // summed first, so that leaf receives one atomic per element instead of one per ray.  The per-term
 // products are the reference's; only the order in which they are added up differs.
 // Both marches test sigma > 0 and never stop early (rt_kernel.cu:377, 441).
-// Adds the gradient records of one queue slot.  A record is the K-long vector
-// (basis[i] * tmp2[c] for the colour coefficients, g_sigma last) of a lane whose `emit` is set, to
-// be added at leaf `leaf`.  The records of the slot are listed in LDS (in parts of ShadeShared that
-// are dead by now: the shade list and the slot's colours), and the wavefront adds the n * K
-// scalars of the list flat, element f of the list from lane f mod 64: every atomic instruction
-// covers 64 consecutive scalars of at most 64 / K + 2 records, whatever K is.
+// Gradient records of a round.  A record is the K-long vector (basis[i] * tmp2[c] for the colour
+// coefficients, g_sigma last) of a lane, to be added at a leaf.  The records of the queue slots are
+// collected in LDS -- in the shade list's storage, which is dead once the colours are evaluated --
+// and added together: the n * K scalars of the list flat, scalar f from lane f mod 64, so that every
+// atomic instruction covers 64 consecutive scalars whatever K is.  The list is flushed when it is
+// full and at the end of the round.
+constexpr int kEmitCap = 60;   // 60 * (leaf 4 + g_sigma 4 + tmp2 12 + owner 1) = 1260 of 1280 bytes
 template <class P, int D>
-__device__ __forceinline__ void emit_records(ShadeShared<D, true>& sh, int q, bool emit, int32_t leaf,
-                                             const float* tmp2, float g_sigma, int lane,
-                                             float* __restrict__ grad_data) {
-    constexpr int K = P::kRecord;
-    const unsigned long long todo = __ballot(emit);
-    const int n = __popcll(todo);
-    if (n == 0) return;
-    float* list_t = sh.colour + q * (kMarchThreads * 3);          // [record][channel]
-    float* list_gs = (float*)(sh.leaf + kMarchThreads);            // [record]
-    if (emit) {
-        const int rec = rank_in(todo);
-        sh.leaf[rec] = leaf;
-        sh.who[rec] = (uint8_t)lane;
-        list_gs[rec] = g_sigma;
-        list_t[rec * 3] = tmp2[0];
-        list_t[rec * 3 + 1] = tmp2[1];
-        list_t[rec * 3 + 2] = tmp2[2];
-    }
-    wave_lds_sync();
-    const int total = n * K;
-    for (int f = lane; f < total; f += kMarchThreads) {
-        const int rec = f / K, e = f - rec * K;
-        float val;
-        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-            val = e < 3 ? list_t[rec * 3 + e] : list_gs[rec];
-        } else {
-            if (e < 3 * D) {
-                const int c = e / D;
-                val = sh.basis[sh.who[rec] * D + (e - c * D)] * list_t[rec * 3 + c];
+struct RecordList {
+    static constexpr int K = P::kRecord;
+    ShadeShared<D, true>& sh;
+    float* grad_data;
+    int lane;
+    int n = 0;   // wavefront-uniform
+
+    __device__ __forceinline__ int32_t* leaves() const { return sh.leaf; }
+    __device__ __forceinline__ float* g_sigmas() const { return (float*)(sh.leaf + kEmitCap); }
+    __device__ __forceinline__ float* tmp2s() const { return (float*)(sh.leaf + 2 * kEmitCap); }
+    __device__ __forceinline__ uint8_t* owners() const { return (uint8_t*)(sh.leaf + 5 * kEmitCap); }
+
+    __device__ __forceinline__ void flush() {
+        if (n == 0) return;
+        wave_lds_sync();
+        const int total = n * K;
+        for (int f = lane; f < total; f += kMarchThreads) {
+            const int rec = f / K, e = f - rec * K;
+            float val;
+            if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                val = e < 3 ? tmp2s()[rec * 3 + e] : g_sigmas()[rec];
             } else {
-                val = list_gs[rec];
+                if (e < 3 * D) {
+                    const int c = e / D;
+                    val = sh.basis[owners()[rec] * D + (e - c * D)] * tmp2s()[rec * 3 + c];
+                } else {
+                    val = g_sigmas()[rec];
+                }
             }
+            atomicAdd(grad_data + (int64_t)leaves()[rec] * K + e, val);
         }
-        atomicAdd(grad_data + (int64_t)sh.leaf[rec] * K + e, val);
+        wave_lds_sync();
+        n = 0;
     }
-    wave_lds_sync();
-}
+
+    // the record of every lane with `emit` set joins the list (in lane order)
+    __device__ __forceinline__ void append(bool emit, int32_t leaf, const float* tmp2, float g_sigma) {
+        unsigned long long todo = __ballot(emit);
+        while (todo) {
+            if (n == kEmitCap) flush();
+            const bool pending = (todo >> lane) & 1ull;
+            const int slot = n + rank_in(todo);
+            const bool take = pending && slot < kEmitCap;
+            if (take) {
+                leaves()[slot] = leaf;
+                owners()[slot] = (uint8_t)lane;
+                g_sigmas()[slot] = g_sigma;
+                tmp2s()[slot * 3] = tmp2[0];
+                tmp2s()[slot * 3 + 1] = tmp2[1];
+                tmp2s()[slot * 3 + 2] = tmp2[2];
+            }
+            const unsigned long long taken = __ballot(take);
+            n += __popcll(taken);
+            todo &= ~taken;
+        }
+    }
+};
+static_assert(5 * kEmitCap * 4 + kEmitCap <= kQueue * kMarchThreads * 5, "record list exceeds the shade list");
+using ShadeSharedProbe = ShadeShared<1, true>;
+static_assert(offsetof(ShadeSharedProbe, who) == sizeof(int32_t) * kQueue * kMarchThreads,
+              "the record list runs from ShadeShared::leaf into ShadeShared::who");
 
 // Workspace of the replaying backward: chunks of kChunkRecords records of 3 float2 (leaf and step
 // length, attenuation and first sigmoid, the other two sigmoids) followed by one float2 whose x
@@ -1042,7 +1069,8 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         wave_lds_sync();
         if (n_entries > 0) shade_entries<P, true>(tr.data, sh, n_entries, lane);
         wave_lds_sync();
-        // ---- composite and emit, slot by slot
+        // ---- composite slot by slot; the gradient records of the round are added together
+        RecordList<P, D> records{sh, grad_data, lane};
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
             bool emit = false, note = false;
@@ -1109,8 +1137,9 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                     rec_count += 1;
                 }
             }
-            emit_records<P, D>(sh, q, emit, q_leaf[q], tmp2, g_sigma, lane, grad_data);
+            records.append(emit, q_leaf[q], tmp2, g_sigma);
         }
+        records.flush();
         // ---- end of a march
         if (active) {
             if (replaying) {
