@@ -326,3 +326,39 @@ def test_backward_workspace_sizes(gpu, oracle_mod, fmt, monkeypatch):
         got = C.volume_render_backward(dev._spec(), rs, opt, go.to(gpu), workspace=per_ray > 0).cpu().numpy()
         err, ok = grad_close(got, want)
         assert ok, (per_ray, err)
+
+
+def test_backward_workspace_argument_handling(gpu, oracle_mod):
+    """The C entry point with workspaces it cannot use (misaligned, too small for one chunk per ray)
+    gives the plain backward's result; a negative size is an error."""
+    import ctypes
+    from svox_amd.csrc import _abi
+    tree = synth.shell_tree(depth=5, n_spheres=4, data_format="SH4", seed=2, sigma_range=(2.0, 20.0))
+    rays = synth.sphere_rays(1000, seed=1)
+    opt = options(tree, step_size=1e-3)
+    go = torch.randn(1000, 3, generator=torch.Generator().manual_seed(5))
+    want = oracle_mod.volume_render_backward(oracle_mod.Tree.from_n3tree(tree), rays.origins, rays.dirs, rays.viewdirs,
+                                             opt, go)
+    dev = on_gpu(tree, gpu)
+    lib = _abi.load_library()
+    spec = C._pack_tree(dev._spec())
+    rs_obj = rays_spec(rays, gpu)
+    rs = C._pack_rays(rs_obj, torch.float32)
+    copt = opt._pack()
+    go_d = go.to(gpu)
+    buf = torch.empty(1000 * 384 + 64, dtype=torch.uint8, device=gpu)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    cases = [(buf.data_ptr() + 4, 1000 * 384), (buf.data_ptr(), 999 * 384), (buf.data_ptr(), 1000 * 384), (None, 0)]
+    for ptr, nbytes in cases:
+        grad = torch.full_like(dev.data.data, 7.0)
+        rc = lib.svox_volume_render_backward_ws(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), go_d.data_ptr(),
+                                                grad.data_ptr(), 0, ptr, nbytes, stream)
+        assert rc == 0, lib.svox_last_error()
+        err, ok = grad_close(grad.cpu().numpy(), want)
+        assert ok, (nbytes, err)
+    grad = torch.empty_like(dev.data.data)
+    rc = lib.svox_volume_render_backward_ws(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), go_d.data_ptr(),
+                                            grad.data_ptr(), 0, buf.data_ptr(), -1, stream)
+    assert rc < 0 and b"workspace" in lib.svox_last_error()
+    assert lib.svox_volume_render_backward_workspace_bytes(1000, 30) == 1000 * 2 * 384
+    assert lib.svox_volume_render_backward_workspace_bytes(0, 30) == 0
