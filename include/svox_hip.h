@@ -198,6 +198,13 @@ int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec*
                                    int64_t workspace_bytes, void* stream);
 int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray);
 
+/* The same for svox_volume_render_images_backward: one ray per pixel, n_rays = n_images * H * W. */
+int svox_volume_render_images_backward_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                                          int32_t n_images, int64_t pose_stride,
+                                          const SvoxRenderOptions* opt, const void* grad_output,
+                                          void* grad_data_out, int32_t accumulate, void* workspace,
+                                          int64_t workspace_bytes, void* stream);
+
 /* volume_render_image_backward(TreeSpec&, CameraSpec&, RenderOptions&, grad_output);
  * rt_kernel.cu:1085-1109.  grad_output (H, W, out_dim). */
 int svox_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,

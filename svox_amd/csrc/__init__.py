@@ -346,8 +346,8 @@ def volume_render_images(tree, cam, opt):
     return out
 
 
-def volume_render_images_backward(tree, cam, opt, grad_output):
-    """zeros_like(tree.data) + scatter for volume_render_images."""
+def volume_render_images_backward(tree, cam, opt, grad_output, workspace=True):
+    """zeros_like(tree.data) + scatter for volume_render_images (workspace: see volume_render_backward)."""
     spec = _pack_tree(tree)
     cspec = _pack_camera(cam, tree.data.dtype, batched=True)
     n, stride = int(cam.c2w.shape[0]), int(cam.c2w.shape[1]) * 4
@@ -355,9 +355,11 @@ def volume_render_images_backward(tree, cam, opt, grad_output):
     _check_grad(grad_output, (n, cspec.height, cspec.width, od), tree.data.dtype)
     grad = torch.empty_like(tree.data)
     copt = opt._pack()
+    ws, ws_bytes = _backward_workspace(tree, n * cspec.height * cspec.width) if workspace else (None, 0)
     with torch.cuda.device(tree.data.device):
-        _call("svox_volume_render_images_backward", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
-              ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0, _stream(tree.data.device))
+        _call("svox_volume_render_images_backward_ws", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
+              ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
+              ws.data_ptr() if ws is not None else None, ws_bytes, _stream(tree.data.device))
     return grad
 
 
@@ -373,6 +375,20 @@ BACKWARD_RECORDS_PER_RAY = 30
 BACKWARD_WORKSPACE_LIMIT = 4 << 30
 
 
+def _backward_workspace(tree, n_rays):
+    """(tensor, bytes) of the backward's workspace for n_rays rays, or (None, 0)."""
+    if n_rays <= 0 or tree.data.dtype != torch.float32:
+        return None, 0
+    size_of = _abi.load_library().svox_volume_render_backward_workspace_bytes
+    per_ray = int(BACKWARD_RECORDS_PER_RAY)
+    while per_ray > 0 and size_of(n_rays, per_ray) > BACKWARD_WORKSPACE_LIMIT:
+        per_ray -= 15
+    nbytes = int(size_of(n_rays, per_ray)) if per_ray > 0 else 0
+    if nbytes <= 0:
+        return None, 0
+    return torch.empty(nbytes // 8, dtype=torch.float64, device=tree.data.device), nbytes
+
+
 def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
     """zeros_like(tree.data) + scatter; rt_kernel.cu:1059-1083.
 
@@ -386,15 +402,7 @@ def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
     _check_grad(grad_output, (rspec.n_rays, od), tree.data.dtype)
     grad = torch.empty_like(tree.data)
     copt = opt._pack()
-    ws, ws_bytes = None, 0
-    if workspace and rspec.n_rays > 0 and tree.data.dtype == torch.float32:
-        size_of = _abi.load_library().svox_volume_render_backward_workspace_bytes
-        per_ray = int(BACKWARD_RECORDS_PER_RAY)
-        while per_ray > 0 and size_of(rspec.n_rays, per_ray) > BACKWARD_WORKSPACE_LIMIT:
-            per_ray -= 15
-        ws_bytes = int(size_of(rspec.n_rays, per_ray)) if per_ray > 0 else 0
-        if ws_bytes > 0:
-            ws = torch.empty(ws_bytes // 8, dtype=torch.float64, device=tree.data.device)
+    ws, ws_bytes = _backward_workspace(tree, rspec.n_rays) if workspace else (None, 0)
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_backward_ws", ctypes.byref(spec), ctypes.byref(rspec),
               ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
@@ -402,18 +410,19 @@ def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
     return grad
 
 
-def volume_render_image_backward(tree, cam, opt, grad_output):
-    """zeros_like(tree.data) + scatter; rt_kernel.cu:1085-1109"""
+def volume_render_image_backward(tree, cam, opt, grad_output, workspace=True):
+    """zeros_like(tree.data) + scatter; rt_kernel.cu:1085-1109 (workspace: see volume_render_backward)"""
     spec = _pack_tree(tree)
     cspec = _pack_camera(cam, tree.data.dtype)
     od = _render_out_dim(spec, opt)
     _check_grad(grad_output, (cspec.height, cspec.width, od), tree.data.dtype)
     grad = torch.empty_like(tree.data)
     copt = opt._pack()
+    ws, ws_bytes = _backward_workspace(tree, cspec.height * cspec.width) if workspace else (None, 0)
     with torch.cuda.device(tree.data.device):
-        _call("svox_volume_render_image_backward", ctypes.byref(spec), ctypes.byref(cspec),
+        _call("svox_volume_render_images_backward_ws", ctypes.byref(spec), ctypes.byref(cspec), 1, 12,
               ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
-              _stream(tree.data.device))
+              ws.data_ptr() if ws is not None else None, ws_bytes, _stream(tree.data.device))
     return grad
 
 

@@ -121,6 +121,9 @@ SIGNATURES = {
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int32, c_void_p, c_int64,
                        c_void_p]),
     "svox_volume_render_backward_workspace_bytes": (c_int64, [c_int64, c_int32]),
+    "svox_volume_render_images_backward_ws": (
+        ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), c_int32, c_int64, P(RenderOptionsC), c_void_p, c_void_p, c_int32,
+                       c_void_p, c_int64, c_void_p]),
     "svox_volume_render_image_backward": (
         ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int32, c_void_p]),
     "svox_se_grad": (

@@ -571,6 +571,14 @@ int svox_volume_render_images_backward(const SvoxTreeSpec* tree, const SvoxCamer
                                        int64_t pose_stride, const SvoxRenderOptions* opt,
                                        const void* grad_output, void* grad_data_out, int32_t accumulate,
                                        void* stream) {
+    return svox_volume_render_images_backward_ws(tree, cam, n_images, pose_stride, opt, grad_output, grad_data_out,
+                                                 accumulate, nullptr, 0, stream);
+}
+
+int svox_volume_render_images_backward_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
+                                          int64_t pose_stride, const SvoxRenderOptions* opt,
+                                          const void* grad_output, void* grad_data_out, int32_t accumulate,
+                                          void* workspace, int64_t workspace_bytes, void* stream) {
     int od;
     int rc = check_render(tree, opt, &od);
     if (rc) return rc;
@@ -583,9 +591,11 @@ int svox_volume_render_images_backward(const SvoxTreeSpec* tree, const SvoxCamer
     }
     if (cam->width == 0 || cam->height == 0 || n_images == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
+    if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
     if (tree->dtype == SVOX_F32) {
         const auto src = image_source<float>(cam, n_images, pose_stride);
-        launch_backward<ImageSource<float>, float>(tree, src, opt, od, grad_output, grad_data_out, nullptr, 0, 0,
+        launch_backward<ImageSource<float>, float>(tree, src, opt, od, grad_output, grad_data_out, workspace,
+                                                   workspace_bytes, (int64_t)n_images * cam->width * cam->height,
                                                    (hipStream_t)stream);
     } else {
         const auto src = image_source<double>(cam, n_images, pose_stride);

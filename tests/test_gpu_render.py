@@ -115,6 +115,10 @@ def test_image_render_and_backward(gpu, oracle_mod, ndc):
     grad = C.volume_render_image_backward(dev._spec(), cam, opt, go.to(gpu))
     err, ok = grad_close(grad.cpu().numpy(), ref_grad)
     assert ok, err
+    # the same without a workspace (the second march walks the tree again)
+    grad = C.volume_render_image_backward(dev._spec(), cam, opt, go.to(gpu), workspace=False)
+    err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+    assert ok, err
     # the batch kernels on the oracle's pixel rays give the same picture
     ro, rd, rv = oracle_mod.image_rays(oracle_mod.Tree.from_n3tree(tree), c2w, fx, fx, W, H, opt)
     assert np.isfinite(rd).all()
