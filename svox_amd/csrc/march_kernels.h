@@ -240,7 +240,7 @@ struct Visit {
     int levels;
 };
 
-// Child entries one lane reads per turn of the octree walk (OctreeCursor::seek).  A lane that needs
+// Child entries one lane reads per turn of the octree walk (OctreeCursor::seek_flat).  A lane that needs
 // more (its ray crossed the boundary of a large cell and has to descend many levels) goes on in its
 // next turn, so that the other lanes of the wavefront do not wait for it: measured, the lanes need
 // 2.0 entries per leaf on average, but the slowest lane of a wavefront 4.8.  (Budgets of 1 and 3, and
@@ -263,44 +263,44 @@ __device__ __forceinline__ Visit step_generic(const TreeDev<T>& tr, const RaySta
     return v;
 }
 
-// The same sample for an fp32 octree: integer walk resumed from the previous path.
-__device__ __forceinline__ Visit step_octree(const TreeDev<float>& tr, const RayState<float>& r,
-                                             OctreeCursor& cur, float step_size, float* delta_t,
-                                             int* reads) {
+// One turn of the octree walk for the whole wavefront, written flat: the lanes with `go` take one
+// sample (slot_leaf, slot_dt) and advance, or keep a descent pending (slot_leaf -1); the others run
+// the same instructions without effect.  `broken`: the tree is malformed, the ray ends here.
+__device__ __forceinline__ void walk_turn_flat(const TreeDev<float>& tr, RayState<float>& r, OctreeCursor& cur,
+                                               float step_size, bool go, bool& broken, int32_t& slot_leaf,
+                                               float& slot_dt) {
     float pc[3];
 #pragma unroll
     for (int j = 0; j < 3; ++j) pc[j] = clamp01(fma_(r.t, r.d[j], r.o[j]));
-    Visit v;
-    const int32_t leaf = cur.seek<kSeekBudget>(tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]),
-                                               cell_coord(pc[1]), cell_coord(pc[2]));
-    if (leaf == OctreeCursor::kPending) {   // the descent goes on in the lane's next turn
-        v.leaf = OctreeCursor::kPending;
-        v.levels = 0;
-        *delta_t = 0.0f;
-        return v;
-    }
-    float inv_cube;  // 2^-levels: dividing by the power of two 2^levels is this multiplication
+    int32_t leaf = cur.seek_flat<kSeekBudget>(go, tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]),
+                                              cell_coord(pc[1]), cell_coord(pc[2]));
+    // 2^levels and 2^-levels: dividing by the power of two is the multiplication by its reciprocal
+    const float cube = __uint_as_float((uint32_t)(127 + cur.levels) << 23);
+    float inv_cube = __uint_as_float((uint32_t)(127 - cur.levels) << 23);
     float local[3];
-    if (leaf >= 0) {
-        v.leaf = leaf;
-        v.levels = cur.levels;
-        const float cube = __uint_as_float((uint32_t)(127 + cur.levels) << 23);
-        inv_cube = __uint_as_float((uint32_t)(127 - cur.levels) << 23);
 #pragma unroll
-        for (int j = 0; j < 3; ++j) local[j] = leaf_local(pc[j], cube);
-    } else {
-        // more levels than the integer coordinates hold (or a broken tree): floating-point walk
-        float cube;
+    for (int j = 0; j < 3; ++j) local[j] = leaf_local(pc[j], cube);
+    const bool deep = leaf == -1;
+    if (__any(deep)) {
+        if (deep) {
+            // more levels than the integer coordinates hold (or a broken tree): floating-point walk
+            float cube_f;
+            int levels_f;
 #pragma unroll
-        for (int j = 0; j < 3; ++j) local[j] = pc[j];
-        v.leaf = descend_generic<float>(tr.child, tr.capacity, 2, local, &cube, &v.levels);
-        *reads += v.levels;
-        inv_cube = 1.0f / cube;
+            for (int j = 0; j < 3; ++j) local[j] = pc[j];
+            leaf = (int32_t)descend_generic<float>(tr.child, tr.capacity, 2, local, &cube_f, &levels_f);
+            inv_cube = 1.0f / cube_f;
+            broken = broken || leaf < 0;
+        }
     }
     float s0, s1;
     dda_unit(local, r.inv, &s0, &s1);
-    *delta_t = (s1 - s0) * inv_cube + step_size;
-    return v;
+    const float delta_t = (s1 - s0) * inv_cube + step_size;
+    const bool ok = leaf >= 0;
+    slot_leaf = ok ? leaf : -1;
+    slot_dt = ok ? delta_t : 0.0f;
+    const float t_next = r.t + delta_t;
+    r.t = ok ? (t_next > r.t ? t_next : r.tmax) : r.t;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -530,24 +530,14 @@ __device__ __forceinline__ RoundState refill_lanes(bool active, int64_t& next, i
 // Walk: kQueue turns; slot q receives the leaf found in turn q and its step length, or -1 (no live
 // ray, or a descent still under way).  `broken` reports a malformed tree: the ray ends there.
 __device__ __forceinline__ void walk_turns(const TreeDev<float>& tr, RayState<float>& r, OctreeCursor& cur,
-                                           float step, bool active, bool& broken, int32_t* q_leaf, float* q_dt,
-                                           int* reads) {
+                                           float step, bool active, bool& broken, int32_t* q_leaf, float* q_dt) {
     broken = false;
 #pragma unroll
     for (int q = 0; q < kQueue; ++q) {
+        const bool go = active && !broken && r.t < r.tmax;
         q_leaf[q] = -1;
         q_dt[q] = 0.0f;
-        if (active && !broken && r.t < r.tmax) {
-            float delta_t;
-            const Visit v = step_octree(tr, r, cur, step, &delta_t, reads);
-            if (v.leaf >= 0) {
-                q_leaf[q] = (int32_t)v.leaf;
-                q_dt[q] = delta_t;
-                advance(r, delta_t);
-            } else if (v.leaf != OctreeCursor::kPending) {
-                broken = true;
-            }
-        }
+        if (__any(go)) walk_turn_flat(tr, r, cur, step, go, broken, q_leaf[q], q_dt[q]);
     }
 }
 
@@ -624,7 +614,6 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     float light = 1.0f;
     int64_t slot = -1;
     bool active = false;
-    int reads = 0;
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
@@ -666,7 +655,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
         bool broken;
-        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt, &reads);
+        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt);
         // ---- sigma
         float q_sigma[kQueue];
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);
@@ -970,7 +959,6 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     float2* rec_chunk = ws.base;
     int64_t shared_next = ws.first_shared + (int64_t)blockIdx.x * ws.per_block;   // wavefront-uniform
     const int64_t shared_end = shared_next + ws.per_block;
-    int reads = 0;
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
@@ -1024,7 +1012,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         float q_sigma[kQueue];
         const bool any_walk = !kReplay || __any(active && !replaying);
         if (any_walk) {
-            walk_turns(tr, r, cur, step, active && !replaying, broken, q_leaf, q_dt, &reads);
+            walk_turns(tr, r, cur, step, active && !replaying, broken, q_leaf, q_dt);
             // ---- sigma
             fetch_sigma<K>(tr.data, q_leaf, q_sigma);
         } else {
@@ -1356,7 +1344,6 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
     float light = 1.0f, light1 = 1.0f, tmin = 0.0f;
     int64_t slot = -1;
     bool active = false, second = false;
-    int reads = 0;
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
@@ -1406,7 +1393,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
         bool broken;
-        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt, &reads);
+        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt);
         // ---- sigma
         float q_sigma[kQueue];
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);

@@ -203,64 +203,58 @@ struct OctreeCursor {
         pend_level = 0;
     }
 
+    static constexpr int32_t kIdle = -3;
+
     // Finds the leaf of the point with integer coordinates (nx, ny, nz), reading at most kBudget
     // child entries.  Returns the leaf cell index; kPending if the budget ran out (call again with
     // the same point to go on); -1 if the tree has more levels than the coordinates hold (`levels`
     // becomes 0).  The budget bounds how long the lanes of a wavefront wait for the one lane that
     // has to descend many levels: that lane continues in its next turn instead.
     // Node ids read from the table are clamped into [0, capacity): a malformed tree yields a wrong
-    // leaf, never an access outside the table.
+    // leaf, never an access outside the table.  The table is smaller than 4 GiB (checked on the
+    // host): a 32-bit byte offset from the uniform base lets the load use the scalar-base form.
+    //
+    // The bookkeeping is written as selects: every lane runs every instruction (in a wavefront that
+    // costs nothing more than running it for one lane) and only the table reads sit under a
+    // condition.  `go`: this lane searches; a lane that does not keeps its state and returns kIdle.
     template <int kBudget>
-    __device__ __forceinline__ int32_t seek(const int32_t* __restrict__ child, int32_t last_node,
-                                            uint32_t nx, uint32_t ny, uint32_t nz) {
-        int level = 1;
-        int32_t node = 0;
-        if (pend_level > 0) {
-            level = pend_level;
-            node = pend_node;
-        } else if (levels > 0) {
-            const uint32_t diff = (ix ^ nx) | (iy ^ ny) | (iz ^ nz);
-            // first level at which the two points fall into different cells
-            const int first_diff = diff ? (kCoordBits - 31 + __builtin_clz(diff)) : kCoordBits + 1;
-            ix = nx; iy = ny; iz = nz;
-            if (first_diff > levels) return leaf;  // still inside the previous leaf
-            level = first_diff < kPathLevels ? first_diff : kPathLevels;
-            node = path[(level - 1) * stride];
-        } else {
-            ix = nx; iy = ny; iz = nz;
-        }
-        // kBudget reads, written out one after the other: no loop bookkeeping between them
-        int32_t cell = 0, skip = 1;
-        bool done = false;
+    __device__ __forceinline__ int32_t seek_flat(bool go, const int32_t* __restrict__ child, int32_t last_node,
+                                                 uint32_t nx, uint32_t ny, uint32_t nz) {
+        const bool pending = pend_level > 0;
+        const bool have = levels > 0;
+        const uint32_t diff = (ix ^ nx) | (iy ^ ny) | (iz ^ nz);
+        const int first_diff = diff ? (kCoordBits - 31 + __builtin_clz(diff)) : kCoordBits + 1;
+        const bool same = !pending && have && first_diff > levels;   // still inside the previous leaf
+        const int from = first_diff < kPathLevels ? first_diff : kPathLevels;
+        const int32_t remembered = path[(from - 1) * stride];   // a row of the array for every lane
+        int level = pending ? pend_level : (have ? from : 1);
+        int32_t node = pending ? pend_node : (have ? remembered : 0);
+        const bool moved = go && !pending;
+        ix = moved ? nx : ix;
+        iy = moved ? ny : iy;
+        iz = moved ? nz : iz;
+        const bool search = go && !same;
+        bool want = search;
+        int32_t cell = 0, skip = 0;
 #pragma unroll
         for (int it = 0; it < kBudget; ++it) {
-            if (!done) {
+            if (want) {
                 path[((level <= kPathLevels ? level : kPathLevels + 1) - 1) * stride] = node;
                 cell = (node << 3) | cell_at(nx, ny, nz, level);
-                // the table is smaller than 4 GiB (checked on the host): a 32-bit byte offset from the
-                // uniform base lets the load use the scalar-base addressing form
                 skip = *(const int32_t*)((const char*)child + ((uint32_t)cell << 2));
-                if (skip == 0 || level == kCoordBits) {
-                    done = true;
-                } else {
-                    // a negative or too large id (malformed tree) wraps / clamps to the last node
-                    node = (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node);
-                    level += 1;
-                }
             }
+            want = want && skip != 0 && level != kCoordBits;
+            node = want ? (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node) : node;
+            level = want ? level + 1 : level;
         }
-        pend_level = 0;
-        if (skip != 0) {
-            levels = 0;   // the path rows written so far stay valid, but there is no previous leaf
-            leaf = -1;
-            if (done) return -1;   // more levels than the coordinates hold
-            pend_level = level;
-            pend_node = node;
-            return kPending;
-        }
-        levels = level;
-        leaf = cell;
-        return cell;
+        // want: the budget ran out; skip == 0: found; else more levels than the coordinates hold
+        const bool found = search && skip == 0;
+        const bool open = search && skip != 0;
+        pend_level = go ? (want ? level : 0) : pend_level;
+        pend_node = want ? node : pend_node;
+        levels = found ? level : (open ? 0 : levels);
+        leaf = found ? cell : (open ? -1 : leaf);
+        return !go ? kIdle : (want ? kPending : leaf);
     }
 };
 

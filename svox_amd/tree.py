@@ -680,13 +680,6 @@ class WeightAccumulator:
 
 
 def gen_grid(D):
-    """Centres of a D^3 grid over [0, 1]^3, shape (D, D, D, 3)."""
-    c = (torch.arange(D) + 0.5) / D
-    X, Y, Z = torch.meshgrid(c, c, c, indexing="ij")
-    return torch.stack([X, Y, Z], -1)
-
-
-def gen_grid(D):
     """Centres of a D^3 grid over [0, 1]^3, (D, D, D, 3) in xyz order (svox/svox.py:1163-1173)."""
     axis = (torch.arange(D) + 0.5) / D
     return torch.stack(torch.meshgrid(axis, axis, axis, indexing="ij"), dim=-1)
