@@ -29,10 +29,11 @@ __device__ __forceinline__ double floor_(double a) { return __builtin_floor(a); 
 // exact steps.  At most 1 ulp from the true value on [-87, 88.72]; 0 below -87 (so no subnormal
 // is ever produced), +inf above 88.7228.  Only fma/mul/add/round-to-nearest are used, so the
 // result does not depend on the math library or on the machine.
-__device__ __forceinline__ float expf_fixed(float x) {
-    if (!(x == x)) return x;
-    if (x < -87.0f) return 0.0f;
-    if (x > 88.72283f) return __builtin_inff();
+__device__ __forceinline__ float expf_fixed(float x0) {
+    // without branches: the polynomial runs on an argument inside the range (any, where x0 is
+    // outside or NaN) and the special results are selected afterwards
+    const bool low = x0 < -87.0f, high = x0 > 88.72283f, nan = !(x0 == x0);
+    const float x = (low || high || nan) ? 0.0f : x0;
     const float n = __builtin_rintf(x * 1.44269504088896341f);
     float r = fma_(n, -0.693145751953125f, x);
     r = fma_(n, -1.428606765330187045e-06f, r);
@@ -49,7 +50,8 @@ __device__ __forceinline__ float expf_fixed(float x) {
     const int n1 = ni >> 1, n2 = ni - n1;
     const float s1 = __uint_as_float((uint32_t)(n1 + 127) << 23);
     const float s2 = __uint_as_float((uint32_t)(n2 + 127) << 23);
-    return (y * s1) * s2;
+    const float e = (y * s1) * s2;
+    return nan ? x0 : (low ? 0.0f : (high ? __builtin_inff() : e));
 }
 
 // expf applied to a scalar_t argument (the reference calls expf in double builds too)

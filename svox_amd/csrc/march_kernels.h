@@ -489,6 +489,10 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
             s = sigmoid_(rec[c]);
         } else {
             const float* co = rec + c * D;
+            // the coefficients are asked for first: the basis is evaluated while they arrive
+            float cv[D];
+#pragma unroll
+            for (int i = 0; i < D; ++i) cv[i] = co[i];
             float b[D];
             if constexpr (kRows) {
 #pragma unroll
@@ -499,7 +503,7 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
             }
             float tmp = 0.0f;
 #pragma unroll
-            for (int i = 0; i < D; ++i) tmp = fma_(b[i], co[i], tmp);
+            for (int i = 0; i < D; ++i) tmp = fma_(b[i], cv[i], tmp);
             s = sigmoid_(tmp);
         }
         sh.colour[(slot * kMarchThreads + owner) * 3 + c] = s;
@@ -661,30 +665,41 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);
         // ---- shade list
         const int n_entries = build_shade_list(sh, q_leaf, q_sigma, sigma_thresh, lane);
-        wave_lds_sync();   // list and view directions are visible to every lane
-        shade_entries<P, false>(tr.data, sh, n_entries, lane);
-        wave_lds_sync();
-        // ---- composite
-        if (active) {
-            bool stopped = false;
+        bool stopped = false;
+        if (n_entries > 0) {   // most rounds of a ray pass through empty space: nothing to shade
+            wave_lds_sync();   // list and view directions are visible to every lane
+            shade_entries<P, false>(tr.data, sh, n_entries, lane);
+            wave_lds_sync();
+            // ---- composite
+            // the attenuations and padded colours of the four slots do not depend on one another: they
+            // are evaluated side by side, and only the products with the transmittance form a chain
+            float q_att[kQueue], q_rgb[kQueue][3];
 #pragma unroll
             for (int q = 0; q < kQueue; ++q) {
-                if (q_leaf[q] >= 0 && !stopped && q_sigma[q] > sigma_thresh) {
-                    const float att = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
-                    const float weight = light * (1.0f - att);
-                    const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+                q_att[q] = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
+                const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
 #pragma unroll
-                    for (int c = 0; c < 3; ++c) acc[c] = fma_(weight, fma_(s[c], d_rgb_pad, -pad), acc[c]);
-                    light *= att;
-                    if constexpr (kAccum) {
+                for (int c = 0; c < 3; ++c) q_rgb[q][c] = fma_(s[c], d_rgb_pad, -pad);
+            }
+#pragma unroll
+            for (int q = 0; q < kQueue; ++q) {
+                const bool take = active && q_leaf[q] >= 0 && !stopped && q_sigma[q] > sigma_thresh;
+                const float weight = light * (1.0f - q_att[q]);
+#pragma unroll
+                for (int c = 0; c < 3; ++c) acc[c] = take ? fma_(weight, q_rgb[q][c], acc[c]) : acc[c];
+                light = take ? light * q_att[q] : light;
+                if constexpr (kAccum) {
+                    if (take) {
                         if (tr.weight_accum_max)
                             atomic_max_float(tr.weight_accum + q_leaf[q], weight);
                         else
                             atomicAdd(tr.weight_accum + q_leaf[q], weight);
                     }
-                    if (light <= stop_thresh) stopped = true;
                 }
+                stopped = stopped || (take && light <= stop_thresh);
             }
+        }
+        if (active) {
             if (stopped || broken || !(r.t < r.tmax)) {
                 if (stopped) {
                     // rt_kernel.cu:306-313: rescale and leave without the background (done here, once
