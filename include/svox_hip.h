@@ -122,7 +122,9 @@ const char* svox_last_error(void);
 const char* svox_status_string(int status);
 
 /* Debugging aid without a counterpart in the reference.  Bit 0: route every call to the generic
- * kernels (any N, any dtype) even where a specialised octree kernel exists. */
+ * kernels (any N, any dtype) even where a specialised octree kernel exists.  Bit 1: ray batches of
+ * any size run the way batches of 512 Ki rays and more do (several 64-ray chunks per wavefront, idle
+ * lanes refilled), so that small test batches reach those kernels. */
 void svox_set_debug_flags(int flags);
 
 /* query_vertical(TreeSpec&, Tensor indices) -> (values, node_ids); svox/csrc/svox_kernel.cu:120-143.

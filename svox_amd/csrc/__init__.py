@@ -520,5 +520,5 @@ def volume_render_stats(tree, rays_or_cam, opt):
 
 
 def set_debug_flags(flags):
-    """bit 0: route every call to the generic kernels"""
+    """bit 0: route every call to the generic kernels; bit 1: small ray batches run like large ones"""
     _abi.load_library().svox_set_debug_flags(int(flags))

@@ -18,7 +18,7 @@ namespace {
 using namespace svox;
 
 thread_local char g_error[512] = "";
-int g_debug_flags = 0;  // bit 0: always take the generic kernels
+int g_debug_flags = 0;  // bit 0: always take the generic kernels; bit 1: small batches run like large ones
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -188,7 +188,7 @@ int pick_per_wave(int64_t total_items, bool backward) {
         return e ? atoi(e) : 0;
     }();
     if (forced == 64 || forced == 128 || forced == 256 || forced == 512 || forced == 1024) return forced;
-    if (total_items < (int64_t)64 * 1024 * 8) return 64;
+    if (total_items < (int64_t)64 * 1024 * 8 && !(g_debug_flags & 2)) return 64;
     return backward ? 512 : 256;
 }
 
@@ -221,8 +221,18 @@ BatchSource<T> batch_source(const SvoxRaysSpec* rays, bool backward = false) {
     s.per_wave = pick_per_wave(rays->n_rays, backward);
     s.refill_at = pick_refill();
     s.xcd_group = 1;
+    s.n_waves = 0;
     return s;
 }
+
+// The persistent kernels deal the rays of a batch out over their wavefronts (BatchSource::n_waves).
+template <typename T>
+BatchSource<T> dealt_out(BatchSource<T> s, unsigned n_waves) {
+    if (s.per_wave > kMarchThreads && (s.per_wave & (s.per_wave - 1)) == 0) s.n_waves = n_waves;
+    return s;
+}
+template <typename T>
+ImageSource<T> dealt_out(const ImageSource<T>& s, unsigned) { return s; }
 
 template <typename T>
 ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pose_stride) {
@@ -279,9 +289,10 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
+            const Source dealt = dealt_out(src, blocks);
 #define SVOX_LAUNCH_FORWARD(ACCUM, REFILL)                                                                     \
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, ACCUM, REFILL>), dim3(blocks), \
-                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), src,     \
+                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), dealt,   \
                                                *opt, (float*)out))
             const bool refill = src.per_wave > kMarchThreads;
             if (tree->weight_accum) {
@@ -311,6 +322,7 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
+            const Source dealt = dealt_out(src, blocks);
             // every ray owns one chunk; what is left of the workspace is dealt out to the blocks
             ReplaySpace ws{nullptr, 0, 0};
             const int64_t chunks = workspace ? workspace_bytes / kChunkBytes : 0;
@@ -321,7 +333,7 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
             }
 #define SVOX_LAUNCH_BACKWARD(REFILL, REPLAY)                                                                     \
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, REFILL, REPLAY>), dim3(blocks), \
-                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), src,       \
+                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), dealt,     \
                                                *opt, (const float*)grad_out, (float*)grad_data, ws))
             const bool refill = src.per_wave > kMarchThreads;
             if (ws.base) {
@@ -351,10 +363,11 @@ void launch_se_grad(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
+            const Source dealt = dealt_out(src, blocks);
             if (src.per_wave > kMarchThreads) {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source, true>), dim3(blocks),
                                                            dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
-                                                           src, *opt, (const float*)color_ref, (float*)color_out,
+                                                           dealt, *opt, (const float*)color_ref, (float*)color_out,
                                                            (float*)grad, (float*)hess));
             } else {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source, false>), dim3(blocks),

@@ -366,3 +366,42 @@ def test_backward_workspace_argument_handling(gpu, oracle_mod):
     assert rc < 0 and b"workspace" in lib.svox_last_error()
     assert lib.svox_volume_render_backward_workspace_bytes(1000, 30) == 1000 * 2 * 384
     assert lib.svox_volume_render_backward_workspace_bytes(0, 30) == 0
+
+
+@pytest.mark.parametrize("order", ["random", "image"])
+@pytest.mark.parametrize("fmt", ["SH9", "RGBA"])
+def test_persistent_batch_kernels_on_a_small_batch(gpu, oracle_mod, fmt, order):
+    """The kernels large batches run in (several 64-ray chunks per wavefront, dealt out over the
+    wavefronts, idle lanes refilled) on a batch small enough for the oracle: unrelated rays, and the
+    rays of an image row by row with a ragged end."""
+    tree = synth.shell_tree(depth=6, n_spheres=6, data_format=fmt, seed=23, sigma_range=(20.0, 200.0))
+    if order == "random":
+        rays = synth.sphere_rays(5000 + 37, seed=9)
+    else:
+        c2w = synth.orbit_poses(1, seed=6, radius=2.4)[0]
+        rays = svox.VolumeRenderer.persp_rays(c2w, 83, 61, 75.0)    # 5063 rays, not a multiple of 64
+    rays = svox.Rays(rays.origins.contiguous(), rays.dirs.contiguous(), rays.dirs.clone())
+    opt = options(tree, step_size=1e-3, fast=True)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    ref = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    go = torch.randn(ref.shape, generator=torch.Generator().manual_seed(8)) * 1e-2
+    ref_grad = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    colors = torch.rand(ref.shape, generator=torch.Generator().manual_seed(4))
+    ref_se = oracle_mod.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, colors, opt)
+    dev = on_gpu(tree, gpu)
+    C.set_debug_flags(2)
+    try:
+        out = C.volume_render(dev._spec(), rays_spec(rays, gpu), opt)
+        grads = [C.volume_render_backward(dev._spec(), rays_spec(rays, gpu), opt, go.to(gpu), workspace=w)
+                 for w in (True, False)]
+        se = C.se_grad(dev._spec(), rays_spec(rays, gpu), colors.to(gpu), opt)
+    finally:
+        C.set_debug_flags(0)
+    assert np.array_equal(out.cpu().numpy(), ref)
+    for grad in grads:
+        err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+        assert ok, err
+    assert np.array_equal(se[0].cpu().numpy(), ref_se[0])
+    for got, want in zip(se[1:], ref_se[1:]):
+        err, ok = grad_close(got.cpu().numpy(), want)
+        assert ok, err
