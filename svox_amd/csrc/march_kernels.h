@@ -1087,6 +1087,20 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         wave_lds_sync();
         // ---- composite slot by slot; the gradient records of the round are added together
         RecordList<P, D> records{sh, grad_data, lane};
+        // what does not depend on the transmittance is evaluated for the four slots side by side
+        float q_att[kQueue], q_total[kQueue], q_s[kQueue][3];
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            q_att[q] = replaying ? q_sigma[q] : expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
+            const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+            float total_color = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                q_s[q][c] = s[c];
+                total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+            }
+            q_total[q] = total_color;
+        }
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
             bool emit = false, note = false;
@@ -1094,12 +1108,10 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             float g_sigma = 0.f, note_att = 0.f;
             float note_s[3] = {0.f, 0.f, 0.f};
             if (active && q_leaf[q] >= 0 && (replaying || q_sigma[q] > 0.0f)) {
-                const float att = replaying ? q_sigma[q] : expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
+                const float att = q_att[q];
                 const float weight = light * (1.0f - att);
-                const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
-                float total_color = 0.0f;
-#pragma unroll
-                for (int c = 0; c < 3; ++c) total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+                const float* s = q_s[q];
+                const float total_color = q_total[q];
                 light *= att;
                 if (phase == kMarch1) {
                     accum = fma_(weight, total_color, accum);

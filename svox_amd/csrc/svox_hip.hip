@@ -161,6 +161,7 @@ int check_camera(const SvoxCameraSpec* cam, int n_images = 1, int64_t pose_strid
 int check_rays(const SvoxRaysSpec* rays) {
     if (!rays) return fail(SVOX_ERR_NULL_POINTER, "rays spec is NULL");
     if (rays->n_rays < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative ray count");
+    if (rays->n_rays >= (1ll << 36)) return fail(SVOX_ERR_BAD_SHAPE, "too many rays for one launch");
     if (rays->n_rays > 0 && (!rays->origins || !rays->dirs || !rays->vdirs))
         return fail(SVOX_ERR_NULL_POINTER, "rays.origins / dirs / vdirs is NULL");
     return SVOX_OK;
