@@ -183,12 +183,14 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
                                 void* grad_data_out, int32_t accumulate, void* stream);
 
 /* No counterpart in the reference.  svox_volume_render_backward with a workspace in device memory
- * (8-byte aligned, any contents, overwritten): while the first of the two marches of a ray passes
+ * (16-byte aligned, any contents, overwritten): while the first of the two marches of a ray passes
  * the leaves with sigma > 0, the kernel notes in the workspace what the second march needs of them
  * (24 bytes per leaf, in chunks of 384 bytes = 15 leaves and a link); a ray whose notes fit is not
  * marched a second time, the others are.  The first n_rays chunks are the rays' own; the rest of
- * the workspace is shared out among the wavefronts for rays with more than 15 such leaves, so the
- * workspace holds workspace_bytes / 384 chunks and is useful from n_rays chunks on.
+ * the workspace is shared out among the wavefronts for rays with more than 15 such leaves; its last
+ * 256 bytes hold a counter through which the wavefronts of a large batch share out the second half
+ * of the rays as they run out of work.  So the workspace holds (workspace_bytes - 256) / 384 chunks
+ * and is useful from n_rays chunks on.
  * The gradient is the one svox_volume_render_backward gives (the same terms; the order of the
  * atomic additions differs from call to call either way).  Without a workspace (NULL, or fewer
  * than n_rays chunks), for fp64 trees and wherever the generic kernels run, the call is
@@ -198,6 +200,28 @@ int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec*
                                    const SvoxRenderOptions* opt, const void* grad_output,
                                    void* grad_data_out, int32_t accumulate, void* workspace,
                                    int64_t workspace_bytes, void* stream);
+
+/* No counterpart in the reference: the pair a training step calls instead of svox_volume_render and
+ * svox_volume_render_backward when it runs both on the same rays (what an autograd function keeps
+ * between its forward and its backward).  svox_volume_render_noted gives the output of
+ * svox_volume_render and, in the same march, leaves in the workspace the notes of every leaf with
+ * sigma > 0 of every ray (the whole ray, also behind the point where the rendering stops early).
+ * svox_volume_render_backward_noted, called with the same tree, rays, options and workspace, gives
+ * the gradient of svox_volume_render_backward without walking the tree: it replays the notes twice.
+ * A ray whose notes did not fit is marched twice as in svox_volume_render_backward; so is every ray
+ * if the workspace does not carry the stamp (ray count, tree->data, rays->origins, step size,
+ * sigma_thresh) the first call left.  The caller must not change tree->data, the rays or the
+ * workspace between the two calls.  Workspace as for svox_volume_render_backward_ws (same size
+ * function).  Where notes cannot be taken (fp64 or generic kernels, a weight accumulator, a negative
+ * sigma_thresh, a workspace with fewer than n_rays chunks) the two calls are svox_volume_render and
+ * svox_volume_render_backward_ws. */
+int svox_volume_render_noted(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                             const SvoxRenderOptions* opt, void* out, void* workspace,
+                             int64_t workspace_bytes, void* stream);
+int svox_volume_render_backward_noted(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                                      const SvoxRenderOptions* opt, const void* grad_output,
+                                      void* grad_data_out, int32_t accumulate, void* workspace,
+                                      int64_t workspace_bytes, void* stream);
 int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray);
 
 /* The same for svox_volume_render_images_backward: one ray per pixel, n_rays = n_images * H * W. */

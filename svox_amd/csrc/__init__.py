@@ -410,6 +410,41 @@ def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
     return grad
 
 
+def volume_render_noted(tree, rays, opt):
+    """(out, notes): volume_render, which in the same march leaves in `notes` (a workspace tensor, or
+    None where the library cannot take notes) what volume_render_backward_noted needs of the rays.
+    No counterpart in the reference: it is what an autograd function keeps between forward and
+    backward."""
+    spec = _pack_tree(tree, rays.origins.dtype if isinstance(rays.origins, torch.Tensor) else None)
+    rspec = _pack_rays(rays, tree.data.dtype)
+    od = _render_out_dim(spec, opt)
+    out = torch.empty((rspec.n_rays, od), dtype=rays.origins.dtype, device=rays.origins.device)
+    copt = opt._pack()
+    ws, ws_bytes = _backward_workspace(tree, rspec.n_rays)
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_noted", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),
+              out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, _stream(tree.data.device))
+    return out, ws
+
+
+def volume_render_backward_noted(tree, rays, opt, grad_output, notes):
+    """volume_render_backward from the notes volume_render_noted left for the same tree, rays and
+    options (notes None: volume_render_backward).  tree.data must not have changed in between."""
+    if notes is None:
+        return volume_render_backward(tree, rays, opt, grad_output)
+    spec = _pack_tree(tree)
+    rspec = _pack_rays(rays, tree.data.dtype)
+    od = _render_out_dim(spec, opt)
+    _check_grad(grad_output, (rspec.n_rays, od), tree.data.dtype)
+    grad = torch.empty_like(tree.data)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_backward_noted", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),
+              grad_output.data_ptr(), grad.data_ptr(), 0, notes.data_ptr(), notes.numel() * notes.element_size(),
+              _stream(tree.data.device))
+    return grad
+
+
 def volume_render_image_backward(tree, cam, opt, grad_output, workspace=True):
     """zeros_like(tree.data) + scatter; rt_kernel.cu:1085-1109 (workspace: see volume_render_backward)"""
     spec = _pack_tree(tree)

@@ -124,10 +124,15 @@ struct BatchSource {
     // out like this every wavefront gets its share whatever the order, at 2-3 % for a shuffled batch
     // (groups of four keep the reads of the rays in whole 48-byte pieces; single rays cost 14 %).
     int64_t n_waves;
-    __device__ __forceinline__ int64_t total() const { return n_waves > 0 ? n_waves * per_wave : rays.n_rays; }
+    // items from `pool_first` on (0: none) are not dealt out: they are ray numbers, handed to whichever
+    // wavefront asks next (see WorkPool)
+    int64_t pool_first;
+    __device__ __forceinline__ int64_t total() const {
+        return pool_first > 0 ? pool_first : (n_waves > 0 ? n_waves * per_wave : rays.n_rays);
+    }
     __device__ __forceinline__ int64_t fetch_item(int64_t i, const SvoxRenderOptions&, const T* offset,
                                                   const T* scaling, T* origin, T* dir, T* vdir) const {
-        if (n_waves > 0) {
+        if (n_waves > 0 && (pool_first == 0 || i < pool_first)) {
             const int shift = __builtin_ctz((unsigned)per_wave);
             const int64_t j = i & (per_wave - 1), w = i >> shift;
             i = ((((j >> 2) * n_waves + w) << 2) | (j & 3));
@@ -544,6 +549,47 @@ __device__ __forceinline__ RoundState refill_lanes(bool active, int64_t& next, i
     return n_idle == kMarchThreads ? kRoundDone : kRoundWork;
 }
 
+// The second half of a large batch is not owned by any wavefront: a wavefront that has used up its
+// own range takes the next 64 rays of the pool (one atomic add by lane 0 per 64 rays).  All
+// wavefronts of such a launch are resident from its start to its end, and the rays of a range differ
+// widely in length; without the pool the first wavefront of a 1M-ray backward launch was done after
+// 550 us, the median after 850 us and the last after 1250 us.
+struct WorkPool {
+    unsigned long long* taken;   // rays handed out so far (zero when the launch starts); null: no pool
+    int64_t first, end;          // the pool's rays
+};
+
+template <class Start>
+__device__ __forceinline__ RoundState refill_lanes(bool active, int64_t& next, int64_t& end, int refill_at,
+                                                   Start&& start, const WorkPool& pool, bool& pool_empty) {
+    const unsigned long long idle = __ballot(!active);
+    const int n_idle = __popcll(idle);
+    if (n_idle >= refill_at) {
+        if (next >= end && !pool_empty) {
+            unsigned long long t = 0;
+            if (threadIdx.x == 0) t = atomicAdd(pool.taken, (unsigned long long)kMarchThreads);
+            const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)t);
+            const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(t >> 32));
+            const int64_t base = pool.first + (int64_t)(((unsigned long long)hi << 32) | lo);
+            if (base >= pool.end) {
+                pool_empty = true;
+            } else {
+                next = base;
+                end = base + kMarchThreads < pool.end ? base + kMarchThreads : pool.end;
+            }
+        }
+        if (next < end) {
+            if (!active) {
+                const int64_t item = next + rank_in(idle);
+                if (item < end) start(item);
+            }
+            next += n_idle;
+            return kRoundRefilled;
+        }
+    }
+    return n_idle == kMarchThreads ? kRoundDone : kRoundWork;
+}
+
 // Walk: kQueue turns; slot q receives the leaf found in turn q and its step length, or -1 (no live
 // ray, or a descent still under way).  `broken` reports a malformed tree: the ray ends there.
 __device__ __forceinline__ void walk_turns(const TreeDev<float>& tr, RayState<float>& r, OctreeCursor& cur,
@@ -939,24 +985,48 @@ static_assert(offsetof(ShadeSharedProbe, who) == sizeof(int32_t) * kQueue * kMar
 // holds the index of the ray's next chunk.  Ray number i starts in chunk i; further chunks come
 // from a part of the workspace that belongs to the wavefront (no atomics: the lanes that need a
 // chunk in the same step are ranked by ballot).
-constexpr int kChunkRecords = 15;
-constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
 struct ReplaySpace {
     float2* base;          // chunk c starts at base + c * kChunkFloat2
     int64_t first_shared;  // chunks [0, first_shared) are the rays' first chunks
     int32_t per_block;     // chunks of the shared part that belong to one block
+    WorkPool pool;         // its counter lives in the workspace as well
+    // kForwardNoted writes `stamp` (what the notes belong to) to stamp_at; replay_backward_kernel uses
+    // the notes only if it finds its own stamp there
+    unsigned long long* stamp_at;
+    unsigned long long stamp[4];
+    // one bit per ray (ray i: bit i % 64 of word i / 64).  replay_backward_kernel sets the bits of the
+    // rays it could not do from their notes; a launch of render_backward_kernel that is given the
+    // bitmap as `only` does those rays and no others
+    unsigned long long* undone;
+    const unsigned long long* only;
 };
+
+// What a launch of render_backward_kernel does:
+//   kBackwardPlain   both marches walk the tree;
+//   kBackwardReplay  march 1 leaves notes in the workspace, march 2 replays them;
+//   kForwardNoted    march 1 only: it renders the ray (the output of render_forward_kernel, thresholds
+//                    and early stop included) and leaves the notes and their count in the workspace,
+//                    for replay_backward_kernel.
+enum BackwardMode { kBackwardPlain = 0, kBackwardReplay = 1, kForwardNoted = 2 };
+
+// Head of a ray's notes, kept in the spare floats of its first chunk (after the 15 records): the
+// link to the next chunk, the number of notes (-1: they did not fit; 0 also for a ray that misses
+// the tree) and the ray's delta_scale (rt_kernel.cu:228).
+constexpr int kChunkRecords = 15;
+constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
+constexpr int kHeadFloat2 = kChunkRecords * 3;          // float2 index of {link, count}, then {delta_scale, -}
 
 // kReplay: during march 1 a lane notes, for every leaf with sigma > 0, what march 2 needs of it; if
 // the notes fit into the workspace, march 2 does not walk the tree again but replays them (a ray
 // with no such leaf is finished on the spot), otherwise it marches as without a workspace.  The
 // duration of a launch is set by its longest rays: halving their second march is what this buys.
-template <class P, class Source, bool kRefill, bool kReplay>
+template <class P, class Source, bool kRefill, int kMode>
 __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<float> tr, Source src,
                                                                         SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
                                                                         float* __restrict__ grad_data,
-                                                                        ReplaySpace ws) {
+                                                                        ReplaySpace ws, float* __restrict__ out) {
+    constexpr bool kReplay = kMode != kBackwardPlain;
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
@@ -968,15 +1038,26 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     const float pad = opt.rgb_padding;
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     const float step = opt.step_size;
+    const float sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
 
     int64_t next = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)src.per_wave;
     const int64_t total = src.total();
-    const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
+    int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
+    bool pool_empty = !(kRefill && kReplay && ws.pool.taken != nullptr);
+
+    if constexpr (kMode == kForwardNoted) {
+        if (blockIdx.x == 0 && lane < 4) ws.stamp_at[lane] = ws.stamp[lane];
+    }
 
     enum { kMarch1 = 0, kMarch2 = 1, kReplaying = 2 };
     RayState<float> r;
     float go[3] = {0.f, 0.f, 0.f};
     float light = 1.0f, accum = 0.0f, tmin = 0.0f;
+    // kForwardNoted: the rendered colour, composited as render_forward_kernel does
+    float acc[3] = {0.f, 0.f, 0.f};
+    float light_f = 1.0f;
+    bool stopped_f = false;
+    int64_t out_slot = 0;
     bool active = false;
     int phase = kMarch1;
     // notes of march 1: total count, the chunk being written / read and the position in it
@@ -993,6 +1074,8 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     // takes ray `item` into this lane if it hits the tree
     auto start = [&](int64_t item) {
         float origin[3], dir[3], vdir[3];
+        // (with a bitmap the items are ray numbers: such a launch does not deal its rays out)
+        if (ws.only && !((ws.only[item >> 6] >> (item & 63)) & 1ull)) return;
         const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
         if (slot >= 0 && setup_ray(r, origin, dir, scaling)) {
             if constexpr (P::kFormat == SVOX_FORMAT_SH) {
@@ -1001,14 +1084,22 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
-            go[0] = grad_out[slot * 3];
-            go[1] = grad_out[slot * 3 + 1];
-            go[2] = grad_out[slot * 3 + 2];
+            if constexpr (kMode == kForwardNoted) {
+                acc[0] = acc[1] = acc[2] = 0.0f;
+                light_f = 1.0f;
+                stopped_f = false;
+                out_slot = slot;
+            } else {
+                go[0] = grad_out[slot * 3];
+                go[1] = grad_out[slot * 3 + 1];
+                go[2] = grad_out[slot * 3 + 2];
+            }
             light = 1.0f;
             accum = 0.0f;
             tmin = r.t;
             cur.restart();
             phase = kMarch1;
+            active = true;
             if constexpr (kReplay) {
                 rec_count = 0;
                 rec_pos = 0;
@@ -1016,7 +1107,11 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                 rec_first = ws.base + slot * kChunkFloat2;
                 rec_chunk = rec_first;
             }
-            active = true;
+        } else if (kMode == kForwardNoted && slot >= 0) {
+            out[slot * 3] = bg;
+            out[slot * 3 + 1] = bg;
+            out[slot * 3 + 2] = bg;
+            ws.base[slot * kChunkFloat2 + kHeadFloat2] = make_float2(0.0f, __int_as_float(0));   // no notes
         }
     };
     if constexpr (!kRefill) {
@@ -1025,7 +1120,22 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 
     while (true) {
         if constexpr (kRefill) {
-            const RoundState state = refill_lanes(active, next, end, src.refill_at, start);
+            if (ws.only) {
+                // skip the 64-ray words of the bitmap in which no ray is left to do, 64 words at a time
+                while (next < end) {
+                    const int64_t word = next >> 6, last_word = (end - 1) >> 6;
+                    const bool some = word + lane <= last_word && ws.only[word + lane] != 0ull;
+                    const unsigned long long nz = __ballot(some);
+                    if (nz == 0ull) {
+                        next = (word + kMarchThreads) << 6;
+                        continue;
+                    }
+                    const int64_t first = (word + __builtin_ctzll(nz)) << 6;
+                    if (first > next) next = first;
+                    break;
+                }
+            }
+            const RoundState state = refill_lanes(active, next, end, src.refill_at, start, ws.pool, pool_empty);
             if (state == kRoundRefilled) continue;
             if (state == kRoundDone) break;
         } else {
@@ -1053,7 +1163,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                 q_sigma[q] = 0.0f;
             }
         }
-        // ---- replayed leaves: the next kQueue notes take the slots; q_sigma holds their attenuation.
+        // ---- replayed leaves: the next kQueue notes take the slots.
         // Their loads are in flight together with the density loads of the walking lanes.
         if constexpr (kReplay) {
             if (active && replaying) {
@@ -1063,7 +1173,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                         if (rec_pos == kChunkRecords) {
                             // the link was read when this chunk was entered: no load to wait for here
                             rec_chunk = ws.base + (int64_t)rec_link * kChunkFloat2;
-                            rec_link = __float_as_int(rec_chunk[kChunkRecords * 3].x);
+                            rec_link = __float_as_int(rec_chunk[kHeadFloat2].x);
                             rec_pos = 0;
                         }
                         const float2* e = rec_chunk + rec_pos * 3;
@@ -1091,7 +1201,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         float q_att[kQueue], q_total[kQueue], q_s[kQueue][3];
 #pragma unroll
         for (int q = 0; q < kQueue; ++q) {
-            q_att[q] = replaying ? q_sigma[q] : expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
+            q_att[q] = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
             const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
             float total_color = 0.0f;
 #pragma unroll
@@ -1105,7 +1215,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         for (int q = 0; q < kQueue; ++q) {
             bool emit = false, note = false;
             float tmp2[3] = {0.f, 0.f, 0.f};
-            float g_sigma = 0.f, note_att = 0.f;
+            float g_sigma = 0.f;
             float note_s[3] = {0.f, 0.f, 0.f};
             if (active && q_leaf[q] >= 0 && (replaying || q_sigma[q] > 0.0f)) {
                 const float att = q_att[q];
@@ -1113,11 +1223,21 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                 const float* s = q_s[q];
                 const float total_color = q_total[q];
                 light *= att;
+                if constexpr (kMode == kForwardNoted) {
+                    // rt_kernel.cu:278-313 on this leaf, as render_forward_kernel composes it
+                    if (!stopped_f && q_sigma[q] > sigma_thresh) {
+                        const float att_f = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
+                        const float weight_f = light_f * (1.0f - att_f);
+#pragma unroll
+                        for (int c = 0; c < 3; ++c) acc[c] = fma_(weight_f, fma_(s[c], d_rgb_pad, -pad), acc[c]);
+                        light_f *= att_f;
+                        if (light_f <= stop_thresh) stopped_f = true;
+                    }
+                }
                 if (phase == kMarch1) {
                     accum = fma_(weight, total_color, accum);
                     if constexpr (kReplay) {
                         note = true;
-                        note_att = att;
                         note_s[0] = s[0];
                         note_s[1] = s[1];
                         note_s[2] = s[2];
@@ -1145,7 +1265,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                     const int64_t mine = shared_next + rank_in(m);
                     if (need) {
                         if (mine < shared_end) {
-                            rec_chunk[kChunkRecords * 3] = make_float2(__int_as_float((int32_t)mine), 0.0f);
+                            rec_chunk[kHeadFloat2] = make_float2(__int_as_float((int32_t)mine), 0.0f);
                             rec_chunk = ws.base + mine * kChunkFloat2;
                             rec_pos = 0;
                         } else {
@@ -1158,7 +1278,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                     if (!rec_lost) {
                         float2* e = rec_chunk + rec_pos * 3;
                         e[0] = make_float2(__int_as_float(q_leaf[q]), q_dt[q]);
-                        e[1] = make_float2(note_att, note_s[0]);
+                        e[1] = make_float2(q_sigma[q], note_s[0]);
                         e[2] = make_float2(note_s[1], note_s[2]);
                         rec_pos += 1;
                     }
@@ -1173,6 +1293,24 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             if (replaying) {
                 rec_next += kQueue;
                 if (rec_next >= rec_count) active = false;
+            } else if (kMode == kForwardNoted && (broken || !(r.t < r.tmax))) {
+                // the ray's colour (rt_kernel.cu:306-319) and the count of its notes
+                if (stopped_f) {
+                    const float scale = (float)(1.0 / (1.0 - (double)light_f));
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) acc[c] *= scale;
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) acc[c] = fma_(light_f, bg, acc[c]);
+                }
+                out[out_slot * 3] = acc[0];
+                out[out_slot * 3 + 1] = acc[1];
+                out[out_slot * 3 + 2] = acc[2];
+                // the head of the notes: the count beside the link (written when the first chunk filled
+                // up), then delta_scale
+                ((float*)(rec_first + kHeadFloat2))[1] = __int_as_float(rec_lost || broken ? -1 : rec_count);
+                rec_first[kHeadFloat2 + 1] = make_float2(r.dscale, 0.0f);
+                active = false;
             } else if (broken || !(r.t < r.tmax)) {
                 if (phase == kMarch1 && !broken) {
                     const float total_grad = (go[0] + go[1]) + go[2];
@@ -1183,7 +1321,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                         rec_next = 0;
                         rec_pos = 0;
                         rec_chunk = rec_first;
-                        rec_link = __float_as_int(rec_first[kChunkRecords * 3].x);   // garbage if there is none
+                        rec_link = __float_as_int(rec_first[kHeadFloat2].x);   // garbage if there is none
                         if (rec_count == 0) active = false;   // no leaf with sigma > 0: nothing to add
                     } else {
                         phase = kMarch2;
@@ -1195,6 +1333,139 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             }
         }
     }
+}
+
+// The backward pass from the notes render_backward_kernel<kForwardNoted> left: one lane per ray, no
+// tree walk.  The notes of a ray (leaf, step length, sigma, the three sigmoids of every leaf with
+// sigma > 0) are read twice, five at a time: first for the sum the reference's first march forms
+// (rt_kernel.cu:358-419), then for the gradient records of its second march (:421-475), which the
+// wavefront adds together as render_backward_kernel does.  A ray whose notes are incomplete, or every
+// ray if the workspace carries another stamp, is left to a launch of render_backward_kernel with the
+// bitmap this kernel writes (one word per wavefront).
+constexpr int kReplayGroup = 5;
+static_assert(kChunkRecords % kReplayGroup == 0, "a group of notes never straddles two chunks");
+
+template <class P>
+__global__ __launch_bounds__(kMarchThreads) void replay_backward_kernel(RayBatch<float> rays, SvoxRenderOptions opt,
+                                                                        const float* __restrict__ grad_out,
+                                                                        float* __restrict__ grad_data,
+                                                                        ReplaySpace ws) {
+    constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
+    __shared__ ShadeShared<D, true> sh;
+    const int lane = threadIdx.x;
+    const int64_t ray = blockIdx.x * (int64_t)kMarchThreads + lane;
+    const bool stamped = ws.stamp_at[0] == ws.stamp[0] && ws.stamp_at[1] == ws.stamp[1] &&
+                         ws.stamp_at[2] == ws.stamp[2] && ws.stamp_at[3] == ws.stamp[3];
+    const float2* first = ws.base + ray * kChunkFloat2;
+    int count = 0;
+    int32_t first_link = 0;
+    float dscale = 0.0f;
+    if (ray < rays.n_rays) {
+        const float2 head = first[kHeadFloat2], tail = first[kHeadFloat2 + 1];
+        first_link = __float_as_int(head.x);
+        count = stamped ? __float_as_int(head.y) : -1;
+        dscale = tail.x;
+    }
+    const unsigned long long undone = __ballot(count < 0);
+    if (lane == 0) ws.undone[blockIdx.x] = undone;
+    const bool work = count > 0;
+    if (!__any(work)) return;
+
+    const float bg = opt.background_brightness;
+    const float pad = opt.rgb_padding;
+    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
+    float go[3] = {0.f, 0.f, 0.f};
+    if (work) {
+        if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+            const float vdir[3] = {rays.vdirs[ray * 3], rays.vdirs[ray * 3 + 1], rays.vdirs[ray * 3 + 2]};
+            float basis[D];
+            sh_basis<float>(P::kBasis, vdir, basis);
+#pragma unroll
+            for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
+        }
+        go[0] = grad_out[ray * 3];
+        go[1] = grad_out[ray * 3 + 1];
+        go[2] = grad_out[ray * 3 + 2];
+    }
+    wave_lds_sync();   // the basis rows are read by other lanes when the records are added
+
+    float light = 1.0f, accum = 0.0f;
+    RecordList<P, D> records{sh, grad_data, lane};
+    struct Group {
+        float2 note[kReplayGroup][3];
+    };
+#pragma unroll 1
+    for (int pass = 0; pass < 2; ++pass) {
+        const float2* chunk = first;
+        int32_t link = first_link;
+        int pos = 0;
+        // asks for the group of notes that starts at note `base` (the loads are waited for where the
+        // group is worked on: meanwhile the group before it is)
+        auto fetch = [&](Group& g, int base) {
+            if (work && base < count) {
+                if (pos == kChunkRecords) {
+                    chunk = ws.base + (int64_t)link * kChunkFloat2;
+                    link = __float_as_int(chunk[kHeadFloat2].x);
+                    pos = 0;
+                }
+#pragma unroll
+                for (int k = 0; k < kReplayGroup; ++k) {
+#pragma unroll
+                    for (int j = 0; j < 3; ++j) g.note[k][j] = chunk[(pos + k) * 3 + j];
+                }
+                pos += kReplayGroup;
+            }
+        };
+        auto work_on = [&](const Group& g, int base) {
+#pragma unroll
+            for (int k = 0; k < kReplayGroup; ++k) {
+                const bool have = work && base + k < count;
+                const int32_t leaf = __float_as_int(g.note[k][0].x);
+                const float dt = g.note[k][0].y, sigma = g.note[k][1].x;
+                const float s[3] = {g.note[k][1].y, g.note[k][2].x, g.note[k][2].y};
+                float tmp2[3] = {0.f, 0.f, 0.f};
+                float g_sigma = 0.0f;
+                if (have) {
+                    const float att = expf_fixed(-dt * sigma * dscale);
+                    const float weight = light * (1.0f - att);
+                    float total_color = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+                    light *= att;
+                    if (pass == 0) {
+                        accum = fma_(weight, total_color, accum);
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < 3; ++c) {
+                            if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                                tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
+                            } else {
+                                tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)go[c] *
+                                                  (double)d_rgb_pad);
+                            }
+                        }
+                        accum = fma_(-weight, total_color, accum);
+                        g_sigma = dt * dscale * fma_(total_color, light, -accum);
+                    }
+                }
+                if (pass == 1) records.append(have, leaf, tmp2, g_sigma);
+            }
+        };
+        Group a, b;
+        fetch(a, 0);
+        for (int base = 0; __any(work && base < count); base += 2 * kReplayGroup) {
+            fetch(b, base + kReplayGroup);
+            work_on(a, base);
+            fetch(a, base + 2 * kReplayGroup);
+            work_on(b, base + kReplayGroup);
+        }
+        if (pass == 0) {
+            const float total_grad = (go[0] + go[1]) + go[2];
+            accum = fma_(light * bg, total_grad, accum);
+            light = 1.0f;
+        }
+    }
+    records.flush();
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -223,6 +223,7 @@ BatchSource<T> batch_source(const SvoxRaysSpec* rays, bool backward = false) {
     s.refill_at = pick_refill();
     s.xcd_group = 1;
     s.n_waves = 0;
+    s.pool_first = 0;
     return s;
 }
 
@@ -234,6 +235,22 @@ BatchSource<T> dealt_out(BatchSource<T> s, unsigned n_waves) {
 }
 template <typename T>
 ImageSource<T> dealt_out(const ImageSource<T>& s, unsigned) { return s; }
+
+// Work pool of a large batch: the wavefronts keep the first half of their rays and the second half
+// of the batch becomes a pool (WorkPool) whose counter the caller's workspace holds.
+constexpr int64_t kPoolBytes = 256;
+template <typename T>
+bool share_out(BatchSource<T>& s, unsigned n_waves, WorkPool* pool) {
+    if (s.n_waves == 0 || s.per_wave < 2 * kMarchThreads) return false;
+    s.per_wave /= 2;
+    s.pool_first = (int64_t)n_waves * s.per_wave;
+    if (s.pool_first >= s.rays.n_rays) return false;
+    pool->first = s.pool_first;
+    pool->end = s.rays.n_rays;
+    return true;
+}
+template <typename T>
+bool share_out(ImageSource<T>&, unsigned, WorkPool*) { return false; }
 
 template <typename T>
 ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pose_stride) {
@@ -314,33 +331,76 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
 
 constexpr int64_t kChunkBytes = (int64_t)kChunkFloat2 * 8;   // 384: 15 records and a link
 
+// What the notes in a workspace belong to (ReplaySpace::stamp).
+struct NoteStamp {
+    unsigned long long word[4];
+};
+NoteStamp stamp_of(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt) {
+    NoteStamp st;
+    uint32_t step_bits, thresh_bits;
+    memcpy(&step_bits, &opt->step_size, 4);
+    memcpy(&thresh_bits, &opt->sigma_thresh, 4);
+    st.word[0] = 0x73766f786e6f7465ull ^ (unsigned long long)rays->n_rays;
+    st.word[1] = (unsigned long long)(uintptr_t)tree->data;
+    st.word[2] = (unsigned long long)(uintptr_t)rays->origins;
+    st.word[3] = ((unsigned long long)thresh_bits << 32) | step_bits;
+    return st;
+}
+
+// The workspace of the replaying kernels: chunks of notes, then one bit per ray (rays left undone by
+// replay_backward_kernel), then 256 bytes with the counter of the work pool (first 16 bytes, cleared
+// before every launch) and the stamp of the notes (from byte 64 on).
+constexpr int64_t kStampOffset = 64;
+int64_t bitmap_bytes(int64_t n_slots) { return ((n_slots + 63) / 64 * 8 + 15) / 16 * 16; }
+bool carve_workspace(void* workspace, int64_t workspace_bytes, int64_t n_slots, unsigned blocks, ReplaySpace* ws) {
+    *ws = ReplaySpace{nullptr, 0, 0, {nullptr, 0, 0}, nullptr, {0, 0, 0, 0}, nullptr, nullptr};
+    const int64_t chunks = workspace && n_slots > 0
+                               ? (workspace_bytes - kPoolBytes - bitmap_bytes(n_slots)) / kChunkBytes : 0;
+    if (n_slots <= 0 || chunks < n_slots || chunks >= 0x7fffffffll || ((uintptr_t)workspace & 15u) != 0) return false;
+    ws->base = (float2*)workspace;
+    ws->first_shared = n_slots;
+    ws->per_block = (int32_t)((chunks - n_slots) / blocks);
+    ws->undone = (unsigned long long*)((char*)workspace + chunks * kChunkBytes);
+    ws->stamp_at = (unsigned long long*)((char*)ws->undone + bitmap_bytes(n_slots) + kStampOffset);
+    return true;
+}
+
+// mode: kBackwardPlain asks for the backward pass with whatever the workspace allows (replay if it is
+// large enough); kForwardNoted needs a usable workspace and the octree kernels, which noted_ok() tells
+// beforehand.
 template <class Source, typename T>
 void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, int out_dim,
                      const void* grad_out, void* grad_data, void* workspace, int64_t workspace_bytes,
-                     int64_t n_slots, hipStream_t stream) {
+                     int64_t n_slots, hipStream_t stream, int mode = kBackwardPlain, void* out = nullptr,
+                     const NoteStamp* stamp = nullptr) {
     const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
-            const Source dealt = dealt_out(src, blocks);
+            Source dealt = dealt_out(src, blocks);
             // every ray owns one chunk; what is left of the workspace is dealt out to the blocks
-            ReplaySpace ws{nullptr, 0, 0};
-            const int64_t chunks = workspace ? workspace_bytes / kChunkBytes : 0;
-            if (n_slots > 0 && chunks >= n_slots && chunks < 0x7fffffffll && ((uintptr_t)workspace & 7u) == 0) {
-                ws.base = (float2*)workspace;
-                ws.first_shared = n_slots;
-                ws.per_block = (int32_t)((chunks - n_slots) / blocks);
+            ReplaySpace ws;
+            if (carve_workspace(workspace, workspace_bytes, n_slots, blocks, &ws)) {
+                void* counter = (char*)ws.stamp_at - kStampOffset;
+                if (share_out(dealt, blocks, &ws.pool) && zero_fill(counter, 16, stream) == SVOX_OK)
+                    ws.pool.taken = (unsigned long long*)counter;
+                else
+                    dealt = dealt_out(src, blocks);
+                if (stamp) memcpy(ws.stamp, stamp->word, sizeof(ws.stamp));
+                if (mode == kBackwardPlain) mode = kBackwardReplay;
             }
-#define SVOX_LAUNCH_BACKWARD(REFILL, REPLAY)                                                                     \
-    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, REFILL, REPLAY>), dim3(blocks), \
-                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), dealt,     \
-                                               *opt, (const float*)grad_out, (float*)grad_data, ws))
+#define SVOX_LAUNCH_BACKWARD(REFILL, MODE)                                                                      \
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, REFILL, MODE>), dim3(blocks),  \
+                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), dealt,    \
+                                               *opt, (const float*)grad_out, (float*)grad_data, ws, (float*)out))
             const bool refill = src.per_wave > kMarchThreads;
-            if (ws.base) {
-                if (refill) { SVOX_LAUNCH_BACKWARD(true, true); } else { SVOX_LAUNCH_BACKWARD(false, true); }
+            if (mode == kBackwardReplay) {
+                if (refill) { SVOX_LAUNCH_BACKWARD(true, kBackwardReplay); } else { SVOX_LAUNCH_BACKWARD(false, kBackwardReplay); }
+            } else if (mode == kForwardNoted) {
+                if (refill) { SVOX_LAUNCH_BACKWARD(true, kForwardNoted); } else { SVOX_LAUNCH_BACKWARD(false, kForwardNoted); }
             } else {
-                if (refill) { SVOX_LAUNCH_BACKWARD(true, false); } else { SVOX_LAUNCH_BACKWARD(false, false); }
+                if (refill) { SVOX_LAUNCH_BACKWARD(true, kBackwardPlain); } else { SVOX_LAUNCH_BACKWARD(false, kBackwardPlain); }
             }
 #undef SVOX_LAUNCH_BACKWARD
             return;
@@ -501,6 +561,91 @@ int svox_calc_corners(const SvoxTreeSpec* tree, const int64_t* indexer, int64_t 
     return check_launch("calc_corners");
 }
 
+// Can a ray batch be rendered with notes (kForwardNoted / kBackwardNoted)?  The octree kernels, a forward
+// pass whose threshold does not admit leaves the backward pass ignores, no weight accumulator, and a
+// workspace with a chunk for every ray.
+// wavefronts that look after the rays replay_backward_kernel leaves undone (normally none)
+constexpr int kUndoneWaves = 256;
+
+static bool noted_ok(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt, void* workspace,
+              int64_t workspace_bytes) {
+    if (tree->dtype != SVOX_F32 || fast_basis(tree, opt) < 0 || tree->weight_accum) return false;
+    if (!(opt->sigma_thresh >= 0.0f)) return false;
+    ReplaySpace ws;
+    return carve_workspace(workspace, workspace_bytes, rays->n_rays, 1, &ws);
+}
+
+int svox_volume_render_noted(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
+                             void* out, void* workspace, int64_t workspace_bytes, void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    rc = check_rays(rays);
+    if (rc) return rc;
+    if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
+    if (rays->n_rays == 0) return SVOX_OK;
+    if (!out) return fail(SVOX_ERR_NULL_POINTER, "out is NULL");
+    if (!noted_ok(tree, rays, opt, workspace, workspace_bytes)) {
+        // no notes: a stamp left by an earlier call must not survive
+        return svox_volume_render(tree, rays, opt, out, stream);
+    }
+    const NoteStamp stamp = stamp_of(tree, rays, opt);
+    launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays, true), opt, od, nullptr, nullptr,
+                                               workspace, workspace_bytes, rays->n_rays, (hipStream_t)stream,
+                                               kForwardNoted, out, &stamp);
+    return check_launch("volume_render_noted");
+}
+
+int svox_volume_render_backward_noted(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                                      const SvoxRenderOptions* opt, const void* grad_output, void* grad_data_out,
+                                      int32_t accumulate, void* workspace, int64_t workspace_bytes, void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    rc = check_rays(rays);
+    if (rc) return rc;
+    if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
+    if (!noted_ok(tree, rays, opt, workspace, workspace_bytes))
+        return svox_volume_render_backward_ws(tree, rays, opt, grad_output, grad_data_out, accumulate, workspace,
+                                              workspace_bytes, stream);
+    if (!grad_data_out) return fail(SVOX_ERR_NULL_POINTER, "grad_data_out is NULL");
+    if (!accumulate) {
+        rc = zero_fill(grad_data_out, data_bytes(tree), (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    if (rays->n_rays == 0) return SVOX_OK;
+    if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
+    // the rays with complete notes from the notes; the others, marked in the bitmap, by two marches
+    const int D = fast_basis(tree, opt);
+    const unsigned words = blocks_for(rays->n_rays, kMarchThreads);
+    ReplaySpace ws;
+    carve_workspace(workspace, workspace_bytes, rays->n_rays, 1, &ws);
+    const NoteStamp stamp = stamp_of(tree, rays, opt);
+    memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
+    const BatchSource<float> all = batch_source<float>(rays, true);
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P>), dim3(words), dim3(kMarchThreads), 0,
+                                               (hipStream_t)stream, all.rays, *opt, (const float*)grad_output,
+                                               (float*)grad_data_out, ws));
+    rc = check_launch("volume_render_backward_noted");
+    if (rc) return rc;
+    BatchSource<float> rest = all;
+    rest.per_wave = (int)(((int64_t)words + kUndoneWaves - 1) / kUndoneWaves) * kMarchThreads;
+    ReplaySpace only = ReplaySpace{nullptr, 0, 0, {nullptr, 0, 0}, nullptr, {0, 0, 0, 0}, nullptr, ws.undone};
+    const unsigned blocks = blocks_for(rays->n_rays, rest.per_wave);
+    if (rest.per_wave > kMarchThreads) {
+        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, BatchSource<float>, true, kBackwardPlain>),
+                                                   dim3(blocks), dim3(kMarchThreads), 0, (hipStream_t)stream,
+                                                   make_tree<float>(tree), rest, *opt, (const float*)grad_output,
+                                                   (float*)grad_data_out, only, (float*)nullptr));
+    } else {
+        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, BatchSource<float>, false, kBackwardPlain>),
+                                                   dim3(blocks), dim3(kMarchThreads), 0, (hipStream_t)stream,
+                                                   make_tree<float>(tree), rest, *opt, (const float*)grad_output,
+                                                   (float*)grad_data_out, only, (float*)nullptr));
+    }
+    return check_launch("volume_render_backward_noted");
+}
+
 int svox_volume_render(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt, void* out,
                        void* stream) {
     int od;
@@ -552,7 +697,7 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
 int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray) {
     if (n_rays <= 0 || records_per_ray <= 0) return 0;
     const int64_t chunks_per_ray = (records_per_ray + kChunkRecords - 1) / kChunkRecords;
-    return n_rays * chunks_per_ray * kChunkBytes;
+    return n_rays * chunks_per_ray * kChunkBytes + bitmap_bytes(n_rays) + kPoolBytes;
 }
 
 int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,

@@ -34,20 +34,38 @@ def _make_camera_spec(c2w, width, height, fx, fy):
 
 class _VolumeRenderFunction(torch.autograd.Function):
     """svox/renderer.py:57-72.  The specs are kept on ctx as plain attributes, so the backward
-    pass sees the tree as it is when backward runs."""
+    pass sees the tree as it is when backward runs.
+
+    When a gradient will be asked for, the forward pass also leaves notes of the leaves it met
+    (volume_render_noted) and the backward pass works from them instead of marching through the tree
+    again.  The notes stand for the tree as it was: if tree.data or the rays were written to between
+    the two passes (their version counters tell), the backward pass marches as the reference does."""
 
     @staticmethod
     def forward(ctx, data, tree, rays, opt):
-        out = _C.volume_render(tree, rays, opt)
         ctx.tree, ctx.rays, ctx.opt = tree, rays, opt
-        return out
+        ctx.notes = None
+        if ctx.needs_input_grad[0]:
+            out, ctx.notes = _C.volume_render_noted(tree, rays, opt)
+            ctx.versions = _versions(tree, rays)
+            return out
+        return _C.volume_render(tree, rays, opt)
 
     @staticmethod
     def backward(ctx, grad_out):
         if not ctx.needs_input_grad[0]:
             return None, None, None, None
-        grad = _C.volume_render_backward(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous())
+        notes, ctx.notes = ctx.notes, None
+        if notes is not None and ctx.versions == _versions(ctx.tree, ctx.rays):
+            grad = _C.volume_render_backward_noted(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous(), notes)
+        else:
+            grad = _C.volume_render_backward(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous())
         return grad, None, None, None
+
+
+def _versions(tree, rays):
+    """Version counters of the tensors the notes of a forward pass depend on."""
+    return tuple(t._version for t in (tree.data, tree.child, rays.origins, rays.dirs, rays.vdirs))
 
 
 class _VolumeRenderImageFunction(torch.autograd.Function):

@@ -350,9 +350,11 @@ def test_backward_workspace_argument_handling(gpu, oracle_mod):
     rs = C._pack_rays(rs_obj, torch.float32)
     copt = opt._pack()
     go_d = go.to(gpu)
-    buf = torch.empty(1000 * 384 + 64, dtype=torch.uint8, device=gpu)
+    # 1000 chunks, 16 words of a bitmap (one bit per ray), 256 bytes for a counter and a stamp
+    enough = 1000 * 384 + 128 + 256
+    buf = torch.empty(enough + 64, dtype=torch.uint8, device=gpu)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    cases = [(buf.data_ptr() + 4, 1000 * 384), (buf.data_ptr(), 999 * 384), (buf.data_ptr(), 1000 * 384), (None, 0)]
+    cases = [(buf.data_ptr() + 4, enough), (buf.data_ptr(), enough - 1), (buf.data_ptr(), enough), (None, 0)]
     for ptr, nbytes in cases:
         grad = torch.full_like(dev.data.data, 7.0)
         rc = lib.svox_volume_render_backward_ws(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), go_d.data_ptr(),
@@ -364,7 +366,7 @@ def test_backward_workspace_argument_handling(gpu, oracle_mod):
     rc = lib.svox_volume_render_backward_ws(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), go_d.data_ptr(),
                                             grad.data_ptr(), 0, buf.data_ptr(), -1, stream)
     assert rc < 0 and b"workspace" in lib.svox_last_error()
-    assert lib.svox_volume_render_backward_workspace_bytes(1000, 30) == 1000 * 2 * 384
+    assert lib.svox_volume_render_backward_workspace_bytes(1000, 30) == 1000 * 2 * 384 + 128 + 256
     assert lib.svox_volume_render_backward_workspace_bytes(0, 30) == 0
 
 
@@ -405,3 +407,40 @@ def test_persistent_batch_kernels_on_a_small_batch(gpu, oracle_mod, fmt, order):
     for got, want in zip(se[1:], ref_se[1:]):
         err, ok = grad_close(got.cpu().numpy(), want)
         assert ok, err
+
+
+@pytest.mark.parametrize("persistent", [False, True])
+@pytest.mark.parametrize("fmt,fast", [("SH9", True), ("SH16", False), ("RGBA", True)])
+def test_noted_forward_and_backward_from_notes(gpu, oracle_mod, fmt, fast, persistent, monkeypatch):
+    """volume_render_noted gives volume_render's picture; volume_render_backward_noted gives the
+    gradient from its notes alone: with room for every ray's notes, with room for some (the others are
+    marched again), and with a workspace that carries another call's stamp."""
+    tree = synth.shell_tree(depth=6, n_spheres=6, data_format=fmt, seed=29, sigma_range=(20.0, 200.0))
+    rays = synth.sphere_rays(4000 + 21, seed=12)
+    o = rays.origins.clone()
+    o[:60] += 3.0                                   # these miss the cube
+    rays = svox.Rays(o.contiguous(), rays.dirs.contiguous(), rays.dirs.clone())
+    opt = options(tree, step_size=1e-3, fast=fast)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    ref = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    go = torch.randn(ref.shape, generator=torch.Generator().manual_seed(8)) * 1e-2
+    ref_grad = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    C.set_debug_flags(2 if persistent else 0)
+    try:
+        for per_ray in (30, 15):
+            monkeypatch.setattr(C, "BACKWARD_RECORDS_PER_RAY", per_ray)
+            out, notes = C.volume_render_noted(dev._spec(), rs, opt)
+            assert notes is not None
+            assert np.array_equal(out.cpu().numpy(), ref)
+            grad = C.volume_render_backward_noted(dev._spec(), rs, opt, go.to(gpu), notes)
+            err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+            assert ok, (per_ray, err)
+        # notes of other rays (another origins tensor): the stamp does not match, every ray is marched
+        other = svox.Rays(rays.origins.clone(), rays.dirs, rays.viewdirs)
+        grad = C.volume_render_backward_noted(dev._spec(), rays_spec(other, gpu), opt, go.to(gpu), notes)
+        err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+        assert ok, err
+    finally:
+        C.set_debug_flags(0)
