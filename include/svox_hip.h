@@ -187,10 +187,10 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
  * the leaves with sigma > 0, the kernel notes in the workspace what the second march needs of them
  * (24 bytes per leaf, in chunks of 384 bytes = 15 leaves and a link); a ray whose notes fit is not
  * marched a second time, the others are.  The first n_rays chunks are the rays' own; the rest of
- * the workspace is shared out among the wavefronts for rays with more than 15 such leaves; its last
- * 256 bytes hold a counter through which the wavefronts of a large batch share out the second half
- * of the rays as they run out of work.  So the workspace holds (workspace_bytes - 256) / 384 chunks
- * and is useful from n_rays chunks on.
+ * the workspace is shared out among the wavefronts for rays with more than 15 such leaves.  After
+ * the chunks come one bit per ray and 256 bytes of bookkeeping (used by the two calls below), so
+ * the workspace holds (workspace_bytes - 256 - 16 * ceil(n_rays / 128)) / 384 chunks and is useful
+ * from n_rays chunks on.
  * The gradient is the one svox_volume_render_backward gives (the same terms; the order of the
  * atomic additions differs from call to call either way).  Without a workspace (NULL, or fewer
  * than n_rays chunks), for fp64 trees and wherever the generic kernels run, the call is

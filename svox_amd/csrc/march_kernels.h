@@ -124,15 +124,10 @@ struct BatchSource {
     // out like this every wavefront gets its share whatever the order, at 2-3 % for a shuffled batch
     // (groups of four keep the reads of the rays in whole 48-byte pieces; single rays cost 14 %).
     int64_t n_waves;
-    // items from `pool_first` on (0: none) are not dealt out: they are ray numbers, handed to whichever
-    // wavefront asks next (see WorkPool)
-    int64_t pool_first;
-    __device__ __forceinline__ int64_t total() const {
-        return pool_first > 0 ? pool_first : (n_waves > 0 ? n_waves * per_wave : rays.n_rays);
-    }
+    __device__ __forceinline__ int64_t total() const { return n_waves > 0 ? n_waves * per_wave : rays.n_rays; }
     __device__ __forceinline__ int64_t fetch_item(int64_t i, const SvoxRenderOptions&, const T* offset,
                                                   const T* scaling, T* origin, T* dir, T* vdir) const {
-        if (n_waves > 0 && (pool_first == 0 || i < pool_first)) {
+        if (n_waves > 0) {
             const int shift = __builtin_ctz((unsigned)per_wave);
             const int64_t j = i & (per_wave - 1), w = i >> shift;
             i = ((((j >> 2) * n_waves + w) << 2) | (j & 3));
@@ -549,47 +544,6 @@ __device__ __forceinline__ RoundState refill_lanes(bool active, int64_t& next, i
     return n_idle == kMarchThreads ? kRoundDone : kRoundWork;
 }
 
-// The second half of a large batch is not owned by any wavefront: a wavefront that has used up its
-// own range takes the next 64 rays of the pool (one atomic add by lane 0 per 64 rays).  All
-// wavefronts of such a launch are resident from its start to its end, and the rays of a range differ
-// widely in length; without the pool the first wavefront of a 1M-ray backward launch was done after
-// 550 us, the median after 850 us and the last after 1250 us.
-struct WorkPool {
-    unsigned long long* taken;   // rays handed out so far (zero when the launch starts); null: no pool
-    int64_t first, end;          // the pool's rays
-};
-
-template <class Start>
-__device__ __forceinline__ RoundState refill_lanes(bool active, int64_t& next, int64_t& end, int refill_at,
-                                                   Start&& start, const WorkPool& pool, bool& pool_empty) {
-    const unsigned long long idle = __ballot(!active);
-    const int n_idle = __popcll(idle);
-    if (n_idle >= refill_at) {
-        if (next >= end && !pool_empty) {
-            unsigned long long t = 0;
-            if (threadIdx.x == 0) t = atomicAdd(pool.taken, (unsigned long long)kMarchThreads);
-            const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)t);
-            const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(t >> 32));
-            const int64_t base = pool.first + (int64_t)(((unsigned long long)hi << 32) | lo);
-            if (base >= pool.end) {
-                pool_empty = true;
-            } else {
-                next = base;
-                end = base + kMarchThreads < pool.end ? base + kMarchThreads : pool.end;
-            }
-        }
-        if (next < end) {
-            if (!active) {
-                const int64_t item = next + rank_in(idle);
-                if (item < end) start(item);
-            }
-            next += n_idle;
-            return kRoundRefilled;
-        }
-    }
-    return n_idle == kMarchThreads ? kRoundDone : kRoundWork;
-}
-
 // Walk: kQueue turns; slot q receives the leaf found in turn q and its step length, or -1 (no live
 // ray, or a descent still under way).  `broken` reports a malformed tree: the ray ends there.
 __device__ __forceinline__ void walk_turns(const TreeDev<float>& tr, RayState<float>& r, OctreeCursor& cur,
@@ -989,7 +943,6 @@ struct ReplaySpace {
     float2* base;          // chunk c starts at base + c * kChunkFloat2
     int64_t first_shared;  // chunks [0, first_shared) are the rays' first chunks
     int32_t per_block;     // chunks of the shared part that belong to one block
-    WorkPool pool;         // its counter lives in the workspace as well
     // kForwardNoted writes `stamp` (what the notes belong to) to stamp_at; replay_backward_kernel uses
     // the notes only if it finds its own stamp there
     unsigned long long* stamp_at;
@@ -1042,8 +995,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 
     int64_t next = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)src.per_wave;
     const int64_t total = src.total();
-    int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
-    bool pool_empty = !(kRefill && kReplay && ws.pool.taken != nullptr);
+    const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
     if constexpr (kMode == kForwardNoted) {
         if (blockIdx.x == 0 && lane < 4) ws.stamp_at[lane] = ws.stamp[lane];
@@ -1135,7 +1087,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                     break;
                 }
             }
-            const RoundState state = refill_lanes(active, next, end, src.refill_at, start, ws.pool, pool_empty);
+            const RoundState state = refill_lanes(active, next, end, src.refill_at, start);
             if (state == kRoundRefilled) continue;
             if (state == kRoundDone) break;
         } else {

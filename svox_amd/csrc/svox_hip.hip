@@ -223,7 +223,6 @@ BatchSource<T> batch_source(const SvoxRaysSpec* rays, bool backward = false) {
     s.refill_at = pick_refill();
     s.xcd_group = 1;
     s.n_waves = 0;
-    s.pool_first = 0;
     return s;
 }
 
@@ -236,21 +235,8 @@ BatchSource<T> dealt_out(BatchSource<T> s, unsigned n_waves) {
 template <typename T>
 ImageSource<T> dealt_out(const ImageSource<T>& s, unsigned) { return s; }
 
-// Work pool of a large batch: the wavefronts keep the first half of their rays and the second half
-// of the batch becomes a pool (WorkPool) whose counter the caller's workspace holds.
-constexpr int64_t kPoolBytes = 256;
-template <typename T>
-bool share_out(BatchSource<T>& s, unsigned n_waves, WorkPool* pool) {
-    if (s.n_waves == 0 || s.per_wave < 2 * kMarchThreads) return false;
-    s.per_wave /= 2;
-    s.pool_first = (int64_t)n_waves * s.per_wave;
-    if (s.pool_first >= s.rays.n_rays) return false;
-    pool->first = s.pool_first;
-    pool->end = s.rays.n_rays;
-    return true;
-}
-template <typename T>
-bool share_out(ImageSource<T>&, unsigned, WorkPool*) { return false; }
+// bytes after the chunks and the bitmap of a workspace: the stamp of the notes
+constexpr int64_t kTailBytes = 256;
 
 template <typename T>
 ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pose_stride) {
@@ -348,14 +334,13 @@ NoteStamp stamp_of(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const Svo
 }
 
 // The workspace of the replaying kernels: chunks of notes, then one bit per ray (rays left undone by
-// replay_backward_kernel), then 256 bytes with the counter of the work pool (first 16 bytes, cleared
-// before every launch) and the stamp of the notes (from byte 64 on).
-constexpr int64_t kStampOffset = 64;
+// replay_backward_kernel), then 256 bytes that hold the stamp of the notes.
+constexpr int64_t kStampOffset = 0;
 int64_t bitmap_bytes(int64_t n_slots) { return ((n_slots + 63) / 64 * 8 + 15) / 16 * 16; }
 bool carve_workspace(void* workspace, int64_t workspace_bytes, int64_t n_slots, unsigned blocks, ReplaySpace* ws) {
-    *ws = ReplaySpace{nullptr, 0, 0, {nullptr, 0, 0}, nullptr, {0, 0, 0, 0}, nullptr, nullptr};
+    *ws = ReplaySpace{nullptr, 0, 0, nullptr, {0, 0, 0, 0}, nullptr, nullptr};
     const int64_t chunks = workspace && n_slots > 0
-                               ? (workspace_bytes - kPoolBytes - bitmap_bytes(n_slots)) / kChunkBytes : 0;
+                               ? (workspace_bytes - kTailBytes - bitmap_bytes(n_slots)) / kChunkBytes : 0;
     if (n_slots <= 0 || chunks < n_slots || chunks >= 0x7fffffffll || ((uintptr_t)workspace & 15u) != 0) return false;
     ws->base = (float2*)workspace;
     ws->first_shared = n_slots;
@@ -378,15 +363,10 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
-            Source dealt = dealt_out(src, blocks);
+            const Source dealt = dealt_out(src, blocks);
             // every ray owns one chunk; what is left of the workspace is dealt out to the blocks
             ReplaySpace ws;
             if (carve_workspace(workspace, workspace_bytes, n_slots, blocks, &ws)) {
-                void* counter = (char*)ws.stamp_at - kStampOffset;
-                if (share_out(dealt, blocks, &ws.pool) && zero_fill(counter, 16, stream) == SVOX_OK)
-                    ws.pool.taken = (unsigned long long*)counter;
-                else
-                    dealt = dealt_out(src, blocks);
                 if (stamp) memcpy(ws.stamp, stamp->word, sizeof(ws.stamp));
                 if (mode == kBackwardPlain) mode = kBackwardReplay;
             }
@@ -630,7 +610,7 @@ int svox_volume_render_backward_noted(const SvoxTreeSpec* tree, const SvoxRaysSp
     if (rc) return rc;
     BatchSource<float> rest = all;
     rest.per_wave = (int)(((int64_t)words + kUndoneWaves - 1) / kUndoneWaves) * kMarchThreads;
-    ReplaySpace only = ReplaySpace{nullptr, 0, 0, {nullptr, 0, 0}, nullptr, {0, 0, 0, 0}, nullptr, ws.undone};
+    ReplaySpace only = ReplaySpace{nullptr, 0, 0, nullptr, {0, 0, 0, 0}, nullptr, ws.undone};
     const unsigned blocks = blocks_for(rays->n_rays, rest.per_wave);
     if (rest.per_wave > kMarchThreads) {
         SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, BatchSource<float>, true, kBackwardPlain>),
@@ -697,7 +677,7 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
 int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray) {
     if (n_rays <= 0 || records_per_ray <= 0) return 0;
     const int64_t chunks_per_ray = (records_per_ray + kChunkRecords - 1) / kChunkRecords;
-    return n_rays * chunks_per_ray * kChunkBytes + bitmap_bytes(n_rays) + kPoolBytes;
+    return n_rays * chunks_per_ray * kChunkBytes + bitmap_bytes(n_rays) + kTailBytes;
 }
 
 int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,

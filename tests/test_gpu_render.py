@@ -350,7 +350,7 @@ def test_backward_workspace_argument_handling(gpu, oracle_mod):
     rs = C._pack_rays(rs_obj, torch.float32)
     copt = opt._pack()
     go_d = go.to(gpu)
-    # 1000 chunks, 16 words of a bitmap (one bit per ray), 256 bytes for a counter and a stamp
+    # 1000 chunks, 16 words of a bitmap (one bit per ray), 256 bytes of bookkeeping
     enough = 1000 * 384 + 128 + 256
     buf = torch.empty(enough + 64, dtype=torch.uint8, device=gpu)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
