@@ -1144,102 +1144,106 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         }
         // ---- shade list (walking lanes only)
         const int n_entries = any_walk ? build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane, replaying) : 0;
-        wave_lds_sync();
-        if (n_entries > 0) shade_entries<P, true>(tr.data, sh, n_entries, lane);
-        wave_lds_sync();
-        // ---- composite slot by slot; the gradient records of the round are added together
-        RecordList<P, D> records{sh, grad_data, lane};
-        // what does not depend on the transmittance is evaluated for the four slots side by side
-        float q_att[kQueue], q_total[kQueue], q_s[kQueue][3];
+        // a round of kForwardNoted without a leaf to shade (most rounds of a ray pass through empty
+        // space) has nothing to compose and nothing to note
+        if (kMode != kForwardNoted || n_entries > 0) {
+            wave_lds_sync();
+            if (n_entries > 0) shade_entries<P, true>(tr.data, sh, n_entries, lane);
+            wave_lds_sync();
+            // ---- composite slot by slot; the gradient records of the round are added together
+            RecordList<P, D> records{sh, grad_data, lane};
+            // what does not depend on the transmittance is evaluated for the four slots side by side
+            float q_att[kQueue], q_total[kQueue], q_s[kQueue][3];
 #pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            q_att[q] = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
-            const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
-            float total_color = 0.0f;
+            for (int q = 0; q < kQueue; ++q) {
+                q_att[q] = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
+                const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+                float total_color = 0.0f;
 #pragma unroll
-            for (int c = 0; c < 3; ++c) {
-                q_s[q][c] = s[c];
-                total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
-            }
-            q_total[q] = total_color;
-        }
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            bool emit = false, note = false;
-            float tmp2[3] = {0.f, 0.f, 0.f};
-            float g_sigma = 0.f;
-            float note_s[3] = {0.f, 0.f, 0.f};
-            if (active && q_leaf[q] >= 0 && (replaying || q_sigma[q] > 0.0f)) {
-                const float att = q_att[q];
-                const float weight = light * (1.0f - att);
-                const float* s = q_s[q];
-                const float total_color = q_total[q];
-                light *= att;
-                if constexpr (kMode == kForwardNoted) {
-                    // rt_kernel.cu:278-313 on this leaf, as render_forward_kernel composes it
-                    if (!stopped_f && q_sigma[q] > sigma_thresh) {
-                        const float att_f = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
-                        const float weight_f = light_f * (1.0f - att_f);
-#pragma unroll
-                        for (int c = 0; c < 3; ++c) acc[c] = fma_(weight_f, fma_(s[c], d_rgb_pad, -pad), acc[c]);
-                        light_f *= att_f;
-                        if (light_f <= stop_thresh) stopped_f = true;
-                    }
+                for (int c = 0; c < 3; ++c) {
+                    q_s[q][c] = s[c];
+                    total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
                 }
-                if (phase == kMarch1) {
-                    accum = fma_(weight, total_color, accum);
-                    if constexpr (kReplay) {
-                        note = true;
-                        note_s[0] = s[0];
-                        note_s[1] = s[1];
-                        note_s[2] = s[2];
-                    }
-                } else {
+                q_total[q] = total_color;
+            }
 #pragma unroll
-                    for (int c = 0; c < 3; ++c) {
-                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                            tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
-                        } else {
-                            tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)go[c] *
-                                              (double)d_rgb_pad);
+            for (int q = 0; q < kQueue; ++q) {
+                bool emit = false, note = false;
+                float tmp2[3] = {0.f, 0.f, 0.f};
+                float g_sigma = 0.f;
+                float note_s[3] = {0.f, 0.f, 0.f};
+                if (active && q_leaf[q] >= 0 && (replaying || q_sigma[q] > 0.0f)) {
+                    const float att = q_att[q];
+                    const float weight = light * (1.0f - att);
+                    const float* s = q_s[q];
+                    const float total_color = q_total[q];
+                    light *= att;
+                    if constexpr (kMode == kForwardNoted) {
+                        // rt_kernel.cu:278-313 on this leaf, as render_forward_kernel composes it
+                        if (!stopped_f && q_sigma[q] > sigma_thresh) {
+                            const float att_f = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
+                            const float weight_f = light_f * (1.0f - att_f);
+#pragma unroll
+                            for (int c = 0; c < 3; ++c) acc[c] = fma_(weight_f, fma_(s[c], d_rgb_pad, -pad), acc[c]);
+                            light_f *= att_f;
+                            if (light_f <= stop_thresh) stopped_f = true;
                         }
                     }
-                    accum = fma_(-weight, total_color, accum);
-                    g_sigma = q_dt[q] * r.dscale * fma_(total_color, light, -accum);
-                    emit = true;
-                }
-            }
-            if constexpr (kReplay) {
-                // lanes whose chunk is full take the next chunks of the wavefront's share, in lane order
-                const bool need = note && !rec_lost && rec_pos == kChunkRecords;
-                const unsigned long long m = __ballot(need);
-                if (m) {
-                    const int64_t mine = shared_next + rank_in(m);
-                    if (need) {
-                        if (mine < shared_end) {
-                            rec_chunk[kHeadFloat2] = make_float2(__int_as_float((int32_t)mine), 0.0f);
-                            rec_chunk = ws.base + mine * kChunkFloat2;
-                            rec_pos = 0;
-                        } else {
-                            rec_lost = true;
+                    if (phase == kMarch1) {
+                        accum = fma_(weight, total_color, accum);
+                        if constexpr (kReplay) {
+                            note = true;
+                            note_s[0] = s[0];
+                            note_s[1] = s[1];
+                            note_s[2] = s[2];
                         }
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < 3; ++c) {
+                            if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                                tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
+                            } else {
+                                tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)go[c] *
+                                                  (double)d_rgb_pad);
+                            }
+                        }
+                        accum = fma_(-weight, total_color, accum);
+                        g_sigma = q_dt[q] * r.dscale * fma_(total_color, light, -accum);
+                        emit = true;
                     }
-                    shared_next += __popcll(m);
                 }
-                if (note) {
-                    if (!rec_lost) {
-                        float2* e = rec_chunk + rec_pos * 3;
-                        e[0] = make_float2(__int_as_float(q_leaf[q]), q_dt[q]);
-                        e[1] = make_float2(q_sigma[q], note_s[0]);
-                        e[2] = make_float2(note_s[1], note_s[2]);
-                        rec_pos += 1;
+                if constexpr (kReplay) {
+                    // lanes whose chunk is full take the next chunks of the wavefront's share, in lane order
+                    const bool need = note && !rec_lost && rec_pos == kChunkRecords;
+                    const unsigned long long m = __ballot(need);
+                    if (m) {
+                        const int64_t mine = shared_next + rank_in(m);
+                        if (need) {
+                            if (mine < shared_end) {
+                                rec_chunk[kHeadFloat2] = make_float2(__int_as_float((int32_t)mine), 0.0f);
+                                rec_chunk = ws.base + mine * kChunkFloat2;
+                                rec_pos = 0;
+                            } else {
+                                rec_lost = true;
+                            }
+                        }
+                        shared_next += __popcll(m);
                     }
-                    rec_count += 1;
+                    if (note) {
+                        if (!rec_lost) {
+                            float2* e = rec_chunk + rec_pos * 3;
+                            e[0] = make_float2(__int_as_float(q_leaf[q]), q_dt[q]);
+                            e[1] = make_float2(q_sigma[q], note_s[0]);
+                            e[2] = make_float2(note_s[1], note_s[2]);
+                            rec_pos += 1;
+                        }
+                        rec_count += 1;
+                    }
                 }
+                if constexpr (kMode != kForwardNoted) records.append(emit, q_leaf[q], tmp2, g_sigma);
             }
-            records.append(emit, q_leaf[q], tmp2, g_sigma);
+            if constexpr (kMode != kForwardNoted) records.flush();
         }
-        records.flush();
         // ---- end of a march
         if (active) {
             if (replaying) {
