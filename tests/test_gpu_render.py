@@ -444,3 +444,32 @@ def test_noted_forward_and_backward_from_notes(gpu, oracle_mod, fmt, fast, persi
         assert ok, err
     finally:
         C.set_debug_flags(0)
+
+
+def test_autograd_uses_notes_and_marches_again_after_a_write(gpu, oracle_mod):
+    """renderer(rays).backward(): the gradient from the forward pass's notes equals the oracle's; if
+    tree.data is written to between the two passes, the backward pass sees the tree as it then is
+    (svox/renderer.py:61-63 keeps no copy either)."""
+    tree = on_gpu(synth.shell_tree(depth=6, n_spheres=6, data_format="SH4", seed=31, sigma_range=(20.0, 200.0)), gpu)
+    rays = synth.sphere_rays(3000, seed=3)
+    rays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.dirs.clone().to(gpu))
+    r = svox.VolumeRenderer(tree, step_size=1e-3)
+    go = (torch.randn(3000, 3, generator=torch.Generator().manual_seed(1)) * 1e-2).to(gpu)
+    opt = r._get_options(True)
+
+    def oracle_grad():
+        ot = oracle_mod.Tree.from_n3tree(tree)      # copies the tensors to the host
+        return oracle_mod.volume_render_backward(ot, rays.origins.cpu(), rays.dirs.cpu(), rays.viewdirs.cpu(), opt,
+                                                 go.cpu())
+
+    out = r(rays, fast=True)
+    out.backward(go)
+    err, ok = grad_close(tree.data.grad.cpu().numpy(), oracle_grad())
+    assert ok, err
+    tree.data.grad = None
+    out = r(rays, fast=True)
+    with torch.no_grad():
+        tree.data[..., -1] *= 0.5          # the densities change after the forward pass
+    out.backward(go)
+    err, ok = grad_close(tree.data.grad.cpu().numpy(), oracle_grad())
+    assert ok, err
