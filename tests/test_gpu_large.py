@@ -225,3 +225,35 @@ def test_config5_depth10_sh25_ndc_against_the_oracle(gpu, oracle_mod):
     ref_vals, ref_ids = oracle_mod.query_vertical(host, pts)
     assert np.array_equal(ids.cpu().numpy(), ref_ids)
     assert np.array_equal(vals.detach().cpu().numpy(), ref_vals)
+
+
+def test_training_step_at_full_size_notes_against_marches(gpu):
+    """The benchmark's 1 Mi-ray batch on its 512^3 tree: the picture of the noted forward pass is the
+    plain one's, and the gradient replayed from its notes is the gradient of the two marches (the
+    persistent kernels, 512 rays per wavefront, dealt out over 2 048 wavefronts)."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 16 * 2 ** 30:
+        pytest.skip("needs 16 GB of free device memory")
+    tree = synth.shell_tree(depth=9, n_spheres=24, data_format="SH16", seed=0, device=gpu)
+    W = H = 800
+    poses = synth.orbit_poses(8, seed=1, radius=4.0)
+    g = torch.Generator().manual_seed(7)
+    B = 1 << 20
+    per_pose = [svox.VolumeRenderer.persp_rays(p.to(gpu), W, H, 1111.111) for p in poses]
+    pick = torch.randint(0, 8 * W * H, (B,), generator=g).to(gpu)
+    all_o = torch.cat([x.origins for x in per_pose])
+    all_d = torch.cat([x.dirs for x in per_pose])
+    rays = svox.Rays(all_o[pick].contiguous(), all_d[pick].contiguous(), all_d[pick].contiguous())
+    del all_o, all_d, per_pose
+    rs = rays_spec(rays, gpu)
+    opt = svox.VolumeRenderer(tree, step_size=5e-4)._get_options(True)
+    go = (torch.randn(B, 3, generator=g) * 1e-2).to(gpu)
+    plain = C.volume_render(tree._spec(), rs, opt)
+    out, notes = C.volume_render_noted(tree._spec(), rs, opt)
+    assert notes is not None and torch.equal(out, plain)
+    from_notes = C.volume_render_backward_noted(tree._spec(), rs, opt, go, notes)
+    del notes
+    marched = C.volume_render_backward(tree._spec(), rs, opt, go, workspace=False)
+    assert marched.abs().max().item() > 0
+    err, ok = grad_close(from_notes.cpu().numpy(), marched.cpu().numpy())
+    assert ok, err
