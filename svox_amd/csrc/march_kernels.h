@@ -871,7 +871,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
 // atomic instruction covers 64 consecutive scalars whatever K is.  The list is flushed when it is
 // full and at the end of the round.
 constexpr int kEmitCap = 60;   // 60 * (leaf 4 + g_sigma 4 + tmp2 12 + owner 1) = 1260 of 1280 bytes
-template <class P, int D>
+template <class P, int D, bool kByRecord = false>
 struct RecordList {
     static constexpr int K = P::kRecord;
     ShadeShared<D, true>& sh;
@@ -885,6 +885,10 @@ struct RecordList {
     __device__ __forceinline__ uint8_t* owners() const { return (uint8_t*)(sh.leaf + 5 * kEmitCap); }
 
     __device__ __forceinline__ void flush() {
+        if constexpr (kByRecord) {
+            flush_by_record();
+            return;
+        }
         if (n == 0) return;
         wave_lds_sync();
         const int total = n * K;
@@ -902,6 +906,48 @@ struct RecordList {
                 }
             }
             atomicAdd(grad_data + (int64_t)leaves()[rec] * K + e, val);
+        }
+        wave_lds_sync();
+        n = 0;
+    }
+
+    // The same additions with the lanes tied to elements instead of running over the flat list: lane l
+    // adds element l % K of record l / K of every group of 64 / K records (of every record, in two or
+    // more steps, if K > 64).  Which record and which element a lane serves never changes, so an
+    // addition costs about half the instructions of the flat form; the price is idle lanes where K
+    // does not divide 64.  (Measured: 12 % off replay_backward_kernel, whose time is mostly these
+    // additions; nothing for render_backward_kernel.)
+    __device__ __forceinline__ void flush_by_record() {
+        if (n == 0) return;
+        wave_lds_sync();
+        if constexpr (K <= kMarchThreads) {
+            constexpr int kPer = kMarchThreads / K;          // records per step
+            const int r = lane / K, e = lane - r * K;
+            const bool in_range = r < kPer;
+            const int c = e / D, i = e - c * D;
+            const bool colour = P::kFormat == SVOX_FORMAT_RGBA ? e < 3 : e < 3 * D;
+            for (int rec0 = 0; rec0 < n; rec0 += kPer) {
+                const int rec = rec0 + r;
+                if (in_range && rec < n) {
+                    float val;
+                    if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                        val = colour ? tmp2s()[rec * 3 + e] : g_sigmas()[rec];
+                    } else {
+                        val = colour ? sh.basis[owners()[rec] * D + i] * tmp2s()[rec * 3 + c] : g_sigmas()[rec];
+                    }
+                    atomicAdd(grad_data + (int64_t)leaves()[rec] * K + e, val);
+                }
+            }
+        } else {
+            for (int rec = 0; rec < n; ++rec) {
+                const int64_t at = (int64_t)leaves()[rec] * K;
+                const int owner = owners()[rec];
+                for (int e = lane; e < K; e += kMarchThreads) {
+                    const int c = e / D;
+                    const float val = e < 3 * D ? sh.basis[owner * D + (e - c * D)] * tmp2s()[rec * 3 + c] : g_sigmas()[rec];
+                    atomicAdd(grad_data + at + e, val);
+                }
+            }
         }
         wave_lds_sync();
         n = 0;
@@ -1346,7 +1392,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_backward_kernel(RayBatch
     wave_lds_sync();   // the basis rows are read by other lanes when the records are added
 
     float light = 1.0f, accum = 0.0f;
-    RecordList<P, D> records{sh, grad_data, lane};
+    RecordList<P, D, true> records{sh, grad_data, lane};
     struct Group {
         float2 note[kReplayGroup][3];
     };

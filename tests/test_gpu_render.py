@@ -410,7 +410,7 @@ def test_persistent_batch_kernels_on_a_small_batch(gpu, oracle_mod, fmt, order):
 
 
 @pytest.mark.parametrize("persistent", [False, True])
-@pytest.mark.parametrize("fmt,fast", [("SH9", True), ("SH16", False), ("RGBA", True)])
+@pytest.mark.parametrize("fmt,fast", [("SH9", True), ("SH16", False), ("SH25", True), ("RGBA", True)])
 def test_noted_forward_and_backward_from_notes(gpu, oracle_mod, fmt, fast, persistent, monkeypatch):
     """volume_render_noted gives volume_render's picture; volume_render_backward_noted gives the
     gradient from its notes alone: with room for every ray's notes, with room for some (the others are
