@@ -222,6 +222,18 @@ int svox_volume_render_backward_noted(const SvoxTreeSpec* tree, const SvoxRaysSp
                                       const SvoxRenderOptions* opt, const void* grad_output,
                                       void* grad_data_out, int32_t accumulate, void* workspace,
                                       int64_t workspace_bytes, void* stream);
+
+/* The same pair for images (svox_volume_render_images / svox_volume_render_images_backward): one
+ * ray per pixel, n_rays = n_images * H * W; the stamp holds cam->c2w in place of rays->origins. */
+int svox_volume_render_images_noted(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                                    int32_t n_images, int64_t pose_stride,
+                                    const SvoxRenderOptions* opt, void* out, void* workspace,
+                                    int64_t workspace_bytes, void* stream);
+int svox_volume_render_images_backward_noted(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
+                                             int32_t n_images, int64_t pose_stride,
+                                             const SvoxRenderOptions* opt, const void* grad_output,
+                                             void* grad_data_out, int32_t accumulate, void* workspace,
+                                             int64_t workspace_bytes, void* stream);
 int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray);
 
 /* The same for svox_volume_render_images_backward: one ray per pixel, n_rays = n_images * H * W. */

@@ -363,6 +363,47 @@ def volume_render_images_backward(tree, cam, opt, grad_output, workspace=True):
     return grad
 
 
+def volume_render_images_noted(tree, cam, opt):
+    """(images, notes): volume_render_images that also leaves the notes
+    volume_render_images_backward_noted works from (see volume_render_noted).  cam.c2w is
+    (n, 3, 4) / (n, 4, 4), or one pose (3, 4) / (4, 4), which gives (H, W, out_dim)."""
+    single = cam.c2w.dim() == 2
+    spec = _pack_tree(tree)
+    cspec = _pack_camera(cam, tree.data.dtype, batched=not single)
+    n, stride = (1, 12) if single else (int(cam.c2w.shape[0]), int(cam.c2w.shape[1]) * 4)
+    od = _render_out_dim(spec, opt)
+    shape = (cspec.height, cspec.width, od) if single else (n, cspec.height, cspec.width, od)
+    out = torch.empty(shape, dtype=tree.data.dtype, device=tree.data.device)
+    copt = opt._pack()
+    ws, ws_bytes = _backward_workspace(tree, n * cspec.height * cspec.width)
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_images_noted", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
+              ctypes.byref(copt), out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
+              _stream(tree.data.device))
+    return out, ws
+
+
+def volume_render_images_backward_noted(tree, cam, opt, grad_output, notes):
+    """The gradient of volume_render_images_noted's picture(s) from its notes (notes None: by marching)."""
+    single = cam.c2w.dim() == 2
+    if notes is None:
+        fn = volume_render_image_backward if single else volume_render_images_backward
+        return fn(tree, cam, opt, grad_output)
+    spec = _pack_tree(tree)
+    cspec = _pack_camera(cam, tree.data.dtype, batched=not single)
+    n, stride = (1, 12) if single else (int(cam.c2w.shape[0]), int(cam.c2w.shape[1]) * 4)
+    od = _render_out_dim(spec, opt)
+    shape = (cspec.height, cspec.width, od) if single else (n, cspec.height, cspec.width, od)
+    _check_grad(grad_output, shape, tree.data.dtype)
+    grad = torch.empty_like(tree.data)
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_images_backward_noted", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
+              ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0, notes.data_ptr(),
+              notes.numel() * notes.element_size(), _stream(tree.data.device))
+    return grad
+
+
 def _check_grad(grad_output, shape, dtype):
     _check_input(grad_output, "grad_output")
     _same_dtype(grad_output, dtype, "grad_output")

@@ -126,6 +126,12 @@ SIGNATURES = {
     "svox_volume_render_backward_noted": (
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int32, c_void_p, c_int64,
                        c_void_p]),
+    "svox_volume_render_images_noted": (
+        ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), c_int32, c_int64, P(RenderOptionsC), c_void_p, c_void_p, c_int64,
+                       c_void_p]),
+    "svox_volume_render_images_backward_noted": (
+        ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), c_int32, c_int64, P(RenderOptionsC), c_void_p, c_void_p, c_int32,
+                       c_void_p, c_int64, c_void_p]),
     "svox_volume_render_images_backward_ws": (
         ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), c_int32, c_int64, P(RenderOptionsC), c_void_p, c_void_p, c_int32,
                        c_void_p, c_int64, c_void_p]),

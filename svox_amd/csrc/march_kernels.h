@@ -125,6 +125,13 @@ struct BatchSource {
     // (groups of four keep the reads of the rays in whole 48-byte pieces; single rays cost 14 %).
     int64_t n_waves;
     __device__ __forceinline__ int64_t total() const { return n_waves > 0 ? n_waves * per_wave : rays.n_rays; }
+    // rays are numbered as they lie in the batch; with n_waves == 0 item i is ray i
+    static constexpr bool kItemsAreSlots = true;
+    __device__ __forceinline__ int64_t n_slots() const { return rays.n_rays; }
+    __device__ __forceinline__ void view_dir(int64_t slot, T* vdir) const {
+#pragma unroll
+        for (int k = 0; k < 3; ++k) vdir[k] = rays.vdirs[slot * 3 + k];
+    }
     __device__ __forceinline__ int64_t fetch_item(int64_t i, const SvoxRenderOptions&, const T* offset,
                                                   const T* scaling, T* origin, T* dir, T* vdir) const {
         if (n_waves > 0) {
@@ -170,6 +177,19 @@ struct ImageSource {
     int refill_at;          // idle lanes that trigger taking new rays
     int xcd_group;          // see chunk_of_block
     int run;                // > 0: the images advance together, `run` 16x16 blocks at a time
+    // pixels are numbered image by image, row by row; the items run through the tiles instead
+    static constexpr bool kItemsAreSlots = false;
+    __device__ __forceinline__ int64_t n_slots() const { return (int64_t)n_images * cam.height * cam.width; }
+    __device__ __forceinline__ void view_dir(int64_t slot, T* vdir) const {
+        const int64_t per_image = (int64_t)cam.height * cam.width;
+        const int64_t image = slot / per_image;
+        const int pixel = (int)(slot - image * per_image);
+        const int iy = pixel / cam.width, ix = pixel - iy * cam.width;
+        Camera<T> c = cam;
+        c.c2w = cam.c2w + image * pose_stride;
+        T origin[3];
+        cam2world_ray(ix, iy, c, vdir, origin);
+    }
     __device__ __forceinline__ int64_t total() const {
         const int64_t per_image = (int64_t)blocks16_of(cam.width) * blocks16_of(cam.height);
         const int64_t padded = run > 0 ? (per_image + run - 1) / run * run : per_image;
@@ -981,14 +1001,16 @@ static_assert(offsetof(ShadeSharedProbe, who) == sizeof(int32_t) * kQueue * kMar
               "the record list runs from ShadeShared::leaf into ShadeShared::who");
 
 // Workspace of the replaying backward: chunks of kChunkRecords records of 3 float2 (leaf and step
-// length, attenuation and first sigmoid, the other two sigmoids) followed by one float2 whose x
+// length, density and first sigmoid, the other two sigmoids) followed by one float2 whose x
 // holds the index of the ray's next chunk.  Ray number i starts in chunk i; further chunks come
-// from a part of the workspace that belongs to the wavefront (no atomics: the lanes that need a
-// chunk in the same step are ranked by ballot).
+// from the rest of the workspace, of which a wavefront takes a stock of 64 chunks at a time through
+// one atomic counter (a heavy image tile needs hundreds, most tiles none); the lanes that need a
+// chunk in the same step are ranked by ballot.
 struct ReplaySpace {
     float2* base;          // chunk c starts at base + c * kChunkFloat2
     int64_t first_shared;  // chunks [0, first_shared) are the rays' first chunks
-    int32_t per_block;     // chunks of the shared part that belong to one block
+    int64_t n_chunks;      // chunks [first_shared, n_chunks) are handed out in stocks of kChunkStock
+    unsigned long long* stocks_taken;   // counter of the stocks handed out (zero when the launch starts)
     // kForwardNoted writes `stamp` (what the notes belong to) to stamp_at; replay_backward_kernel uses
     // the notes only if it finds its own stamp there
     unsigned long long* stamp_at;
@@ -1014,6 +1036,7 @@ enum BackwardMode { kBackwardPlain = 0, kBackwardReplay = 1, kForwardNoted = 2 }
 constexpr int kChunkRecords = 15;
 constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
 constexpr int kHeadFloat2 = kChunkRecords * 3;          // float2 index of {link, count}, then {delta_scale, -}
+constexpr int kChunkStock = 64;   // further chunks a wavefront takes at a time (at most 64 lanes ask at once)
 
 // kReplay: during march 1 a lane notes, for every leaf with sigma > 0, what march 2 needs of it; if
 // the notes fit into the workspace, march 2 does not walk the tree again but replays them (a ray
@@ -1064,17 +1087,17 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     bool rec_lost = false;             // the workspace ran out: this ray marches twice
     float2* rec_first = ws.base;
     float2* rec_chunk = ws.base;
-    int64_t shared_next = ws.first_shared + (int64_t)blockIdx.x * ws.per_block;   // wavefront-uniform
-    const int64_t shared_end = shared_next + ws.per_block;
+    int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of further chunks (uniform)
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
     // takes ray `item` into this lane if it hits the tree
     auto start = [&](int64_t item) {
         float origin[3], dir[3], vdir[3];
-        // (with a bitmap the items are ray numbers: such a launch does not deal its rays out)
-        if (ws.only && !((ws.only[item >> 6] >> (item & 63)) & 1ull)) return;
+        // (with a bitmap a batch launch does not deal its rays out: its items are ray numbers)
+        if (Source::kItemsAreSlots && ws.only && !((ws.only[item >> 6] >> (item & 63)) & 1ull)) return;
         const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+        if (!Source::kItemsAreSlots && ws.only && slot >= 0 && !((ws.only[slot >> 6] >> (slot & 63)) & 1ull)) return;
         if (slot >= 0 && setup_ray(r, origin, dir, scaling)) {
             if constexpr (P::kFormat == SVOX_FORMAT_SH) {
                 float basis[D];
@@ -1118,7 +1141,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 
     while (true) {
         if constexpr (kRefill) {
-            if (ws.only) {
+            if (Source::kItemsAreSlots && ws.only) {
                 // skip the 64-ray words of the bitmap in which no ray is left to do, 64 words at a time
                 while (next < end) {
                     const int64_t word = next >> 6, last_word = (end - 1) >> 6;
@@ -1259,10 +1282,21 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                     }
                 }
                 if constexpr (kReplay) {
-                    // lanes whose chunk is full take the next chunks of the wavefront's share, in lane order
+                    // lanes whose chunk is full take the next chunks of the wavefront's stock, in lane order
                     const bool need = note && !rec_lost && rec_pos == kChunkRecords;
                     const unsigned long long m = __ballot(need);
                     if (m) {
+                        if (shared_next + __popcll(m) > shared_end) {
+                            // a new stock (what is left of the old one is given up): one atomic per 64 chunks
+                            unsigned long long t = 0;
+                            if (lane == 0) t = atomicAdd(ws.stocks_taken, 1ull);
+                            const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)t);
+                            const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(t >> 32));
+                            const int64_t stock = (int64_t)(((unsigned long long)hi << 32) | lo);
+                            shared_next = ws.first_shared + stock * kChunkStock;
+                            shared_end = shared_next + kChunkStock < ws.n_chunks ? shared_next + kChunkStock : ws.n_chunks;
+                            if (shared_next > shared_end) shared_next = shared_end;
+                        }
                         const int64_t mine = shared_next + rank_in(m);
                         if (need) {
                             if (mine < shared_end) {
@@ -1347,8 +1381,8 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 constexpr int kReplayGroup = 5;
 static_assert(kChunkRecords % kReplayGroup == 0, "a group of notes never straddles two chunks");
 
-template <class P>
-__global__ __launch_bounds__(kMarchThreads) void replay_backward_kernel(RayBatch<float> rays, SvoxRenderOptions opt,
+template <class P, class Source>
+__global__ __launch_bounds__(kMarchThreads) void replay_backward_kernel(Source src, SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
                                                                         float* __restrict__ grad_data,
                                                                         ReplaySpace ws) {
@@ -1362,7 +1396,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_backward_kernel(RayBatch
     int count = 0;
     int32_t first_link = 0;
     float dscale = 0.0f;
-    if (ray < rays.n_rays) {
+    if (ray < src.n_slots()) {
         const float2 head = first[kHeadFloat2], tail = first[kHeadFloat2 + 1];
         first_link = __float_as_int(head.x);
         count = stamped ? __float_as_int(head.y) : -1;
@@ -1379,7 +1413,8 @@ __global__ __launch_bounds__(kMarchThreads) void replay_backward_kernel(RayBatch
     float go[3] = {0.f, 0.f, 0.f};
     if (work) {
         if constexpr (P::kFormat == SVOX_FORMAT_SH) {
-            const float vdir[3] = {rays.vdirs[ray * 3], rays.vdirs[ray * 3 + 1], rays.vdirs[ray * 3 + 2]};
+            float vdir[3];
+            src.view_dir(ray, vdir);
             float basis[D];
             sh_basis<float>(P::kBasis, vdir, basis);
 #pragma unroll

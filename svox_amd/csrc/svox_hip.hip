@@ -334,19 +334,23 @@ NoteStamp stamp_of(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const Svo
 }
 
 // The workspace of the replaying kernels: chunks of notes, then one bit per ray (rays left undone by
-// replay_backward_kernel), then 256 bytes that hold the stamp of the notes.
+// replay_backward_kernel), then 256 bytes that hold the stamp of the notes and, from byte 128 on, the
+// counter of the chunk stocks (cleared before every launch that takes notes).
 constexpr int64_t kStampOffset = 0;
+constexpr int64_t kStockCounterOffset = 128;
 int64_t bitmap_bytes(int64_t n_slots) { return ((n_slots + 63) / 64 * 8 + 15) / 16 * 16; }
 bool carve_workspace(void* workspace, int64_t workspace_bytes, int64_t n_slots, unsigned blocks, ReplaySpace* ws) {
-    *ws = ReplaySpace{nullptr, 0, 0, nullptr, {0, 0, 0, 0}, nullptr, nullptr};
+    *ws = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0}, nullptr, nullptr};
     const int64_t chunks = workspace && n_slots > 0
                                ? (workspace_bytes - kTailBytes - bitmap_bytes(n_slots)) / kChunkBytes : 0;
     if (n_slots <= 0 || chunks < n_slots || chunks >= 0x7fffffffll || ((uintptr_t)workspace & 15u) != 0) return false;
     ws->base = (float2*)workspace;
+    (void)blocks;
     ws->first_shared = n_slots;
-    ws->per_block = (int32_t)((chunks - n_slots) / blocks);
+    ws->n_chunks = chunks;
     ws->undone = (unsigned long long*)((char*)workspace + chunks * kChunkBytes);
     ws->stamp_at = (unsigned long long*)((char*)ws->undone + bitmap_bytes(n_slots) + kStampOffset);
+    ws->stocks_taken = (unsigned long long*)((char*)ws->undone + bitmap_bytes(n_slots) + kStockCounterOffset);
     return true;
 }
 
@@ -366,7 +370,8 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
             const Source dealt = dealt_out(src, blocks);
             // every ray owns one chunk; what is left of the workspace is dealt out to the blocks
             ReplaySpace ws;
-            if (carve_workspace(workspace, workspace_bytes, n_slots, blocks, &ws)) {
+            if (carve_workspace(workspace, workspace_bytes, n_slots, blocks, &ws) &&
+                zero_fill(ws.stocks_taken, 16, stream) == SVOX_OK) {
                 if (stamp) memcpy(ws.stamp, stamp->word, sizeof(ws.stamp));
                 if (mode == kBackwardPlain) mode = kBackwardReplay;
             }
@@ -434,6 +439,59 @@ int se_grad_prepare(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, void
     rc = zero_fill(grad, data_bytes(tree), stream);
     if (rc) return rc;
     return zero_fill(hess, data_bytes(tree), stream);
+}
+
+// wavefronts that look after the rays of a batch that replay_backward_kernel leaves undone (normally none)
+constexpr int kUndoneWaves = 256;
+
+// Can notes be taken (kForwardNoted) and used (replay_backward_kernel)?  The octree kernels, a forward
+// pass whose threshold does not admit leaves the backward pass ignores, no weight accumulator, and a
+// workspace with a chunk for every ray.
+bool noted_ok(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, int64_t n_slots, void* workspace,
+                     int64_t workspace_bytes) {
+    if (tree->dtype != SVOX_F32 || fast_basis(tree, opt) < 0 || tree->weight_accum) return false;
+    if (!(opt->sigma_thresh >= 0.0f)) return false;
+    ReplaySpace ws;
+    return carve_workspace(workspace, workspace_bytes, n_slots, 1, &ws);
+}
+
+NoteStamp stamp_of_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
+                                const SvoxRenderOptions* opt) {
+    SvoxRaysSpec as_rays;
+    as_rays.origins = cam->c2w;
+    as_rays.n_rays = ((int64_t)n_images * cam->height * cam->width) ^ ((int64_t)cam->width << 40);
+    return stamp_of(tree, &as_rays, opt);
+}
+
+// The backward pass of `all` from the notes in the workspace: the rays with complete notes by
+// replay_backward_kernel, the others, which it marks in the bitmap, by two marches.
+template <class Source>
+int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest, const SvoxRenderOptions* opt,
+                               const void* grad_output, void* grad_data_out, void* workspace, int64_t workspace_bytes,
+                               int64_t n_slots, const NoteStamp& stamp, hipStream_t stream) {
+    const int D = fast_basis(tree, opt);
+    const unsigned words = blocks_for(n_slots, kMarchThreads);
+    ReplaySpace ws;
+    carve_workspace(workspace, workspace_bytes, n_slots, 1, &ws);
+    memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P, Source>), dim3(words), dim3(kMarchThreads), 0,
+                                               stream, all, *opt, (const float*)grad_output, (float*)grad_data_out, ws));
+    int rc = check_launch("volume_render_backward_noted");
+    if (rc) return rc;
+    ReplaySpace only = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0}, nullptr, ws.undone};
+    const unsigned blocks = blocks_for(total_items_of(rest), rest.per_wave);
+    if (rest.per_wave > kMarchThreads) {
+        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, true, kBackwardPlain>), dim3(blocks),
+                                                   dim3(kMarchThreads), 0, stream, make_tree<float>(tree), rest, *opt,
+                                                   (const float*)grad_output, (float*)grad_data_out, only,
+                                                   (float*)nullptr));
+    } else {
+        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, false, kBackwardPlain>), dim3(blocks),
+                                                   dim3(kMarchThreads), 0, stream, make_tree<float>(tree), rest, *opt,
+                                                   (const float*)grad_output, (float*)grad_data_out, only,
+                                                   (float*)nullptr));
+    }
+    return check_launch("volume_render_backward_noted");
 }
 
 }  // namespace
@@ -544,17 +602,6 @@ int svox_calc_corners(const SvoxTreeSpec* tree, const int64_t* indexer, int64_t 
 // Can a ray batch be rendered with notes (kForwardNoted / kBackwardNoted)?  The octree kernels, a forward
 // pass whose threshold does not admit leaves the backward pass ignores, no weight accumulator, and a
 // workspace with a chunk for every ray.
-// wavefronts that look after the rays replay_backward_kernel leaves undone (normally none)
-constexpr int kUndoneWaves = 256;
-
-static bool noted_ok(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt, void* workspace,
-              int64_t workspace_bytes) {
-    if (tree->dtype != SVOX_F32 || fast_basis(tree, opt) < 0 || tree->weight_accum) return false;
-    if (!(opt->sigma_thresh >= 0.0f)) return false;
-    ReplaySpace ws;
-    return carve_workspace(workspace, workspace_bytes, rays->n_rays, 1, &ws);
-}
-
 int svox_volume_render_noted(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
                              void* out, void* workspace, int64_t workspace_bytes, void* stream) {
     int od;
@@ -565,10 +612,8 @@ int svox_volume_render_noted(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
     if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
     if (rays->n_rays == 0) return SVOX_OK;
     if (!out) return fail(SVOX_ERR_NULL_POINTER, "out is NULL");
-    if (!noted_ok(tree, rays, opt, workspace, workspace_bytes)) {
-        // no notes: a stamp left by an earlier call must not survive
+    if (!noted_ok(tree, opt, rays->n_rays, workspace, workspace_bytes))
         return svox_volume_render(tree, rays, opt, out, stream);
-    }
     const NoteStamp stamp = stamp_of(tree, rays, opt);
     launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays, true), opt, od, nullptr, nullptr,
                                                workspace, workspace_bytes, rays->n_rays, (hipStream_t)stream,
@@ -585,7 +630,7 @@ int svox_volume_render_backward_noted(const SvoxTreeSpec* tree, const SvoxRaysSp
     rc = check_rays(rays);
     if (rc) return rc;
     if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
-    if (!noted_ok(tree, rays, opt, workspace, workspace_bytes))
+    if (!noted_ok(tree, opt, rays->n_rays, workspace, workspace_bytes))
         return svox_volume_render_backward_ws(tree, rays, opt, grad_output, grad_data_out, accumulate, workspace,
                                               workspace_bytes, stream);
     if (!grad_data_out) return fail(SVOX_ERR_NULL_POINTER, "grad_data_out is NULL");
@@ -595,35 +640,59 @@ int svox_volume_render_backward_noted(const SvoxTreeSpec* tree, const SvoxRaysSp
     }
     if (rays->n_rays == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
-    // the rays with complete notes from the notes; the others, marked in the bitmap, by two marches
-    const int D = fast_basis(tree, opt);
-    const unsigned words = blocks_for(rays->n_rays, kMarchThreads);
-    ReplaySpace ws;
-    carve_workspace(workspace, workspace_bytes, rays->n_rays, 1, &ws);
-    const NoteStamp stamp = stamp_of(tree, rays, opt);
-    memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
     const BatchSource<float> all = batch_source<float>(rays, true);
-    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P>), dim3(words), dim3(kMarchThreads), 0,
-                                               (hipStream_t)stream, all.rays, *opt, (const float*)grad_output,
-                                               (float*)grad_data_out, ws));
-    rc = check_launch("volume_render_backward_noted");
-    if (rc) return rc;
     BatchSource<float> rest = all;
-    rest.per_wave = (int)(((int64_t)words + kUndoneWaves - 1) / kUndoneWaves) * kMarchThreads;
-    ReplaySpace only = ReplaySpace{nullptr, 0, 0, nullptr, {0, 0, 0, 0}, nullptr, ws.undone};
-    const unsigned blocks = blocks_for(rays->n_rays, rest.per_wave);
-    if (rest.per_wave > kMarchThreads) {
-        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, BatchSource<float>, true, kBackwardPlain>),
-                                                   dim3(blocks), dim3(kMarchThreads), 0, (hipStream_t)stream,
-                                                   make_tree<float>(tree), rest, *opt, (const float*)grad_output,
-                                                   (float*)grad_data_out, only, (float*)nullptr));
-    } else {
-        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, BatchSource<float>, false, kBackwardPlain>),
-                                                   dim3(blocks), dim3(kMarchThreads), 0, (hipStream_t)stream,
-                                                   make_tree<float>(tree), rest, *opt, (const float*)grad_output,
-                                                   (float*)grad_data_out, only, (float*)nullptr));
+    const int64_t words = (rays->n_rays + kMarchThreads - 1) / kMarchThreads;
+    rest.per_wave = (int)((words + kUndoneWaves - 1) / kUndoneWaves) * kMarchThreads;
+    return backward_from_notes(tree, all, rest, opt, grad_output, grad_data_out, workspace, workspace_bytes,
+                               rays->n_rays, stamp_of(tree, rays, opt), (hipStream_t)stream);
+}
+
+int svox_volume_render_images_noted(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
+                                    int64_t pose_stride, const SvoxRenderOptions* opt, void* out, void* workspace,
+                                    int64_t workspace_bytes, void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    rc = check_camera(cam, n_images, pose_stride);
+    if (rc) return rc;
+    if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
+    if (cam->width == 0 || cam->height == 0 || n_images == 0) return SVOX_OK;
+    if (!out) return fail(SVOX_ERR_NULL_POINTER, "out is NULL");
+    const int64_t n_slots = (int64_t)n_images * cam->width * cam->height;
+    if (!noted_ok(tree, opt, n_slots, workspace, workspace_bytes))
+        return svox_volume_render_images(tree, cam, n_images, pose_stride, opt, out, stream);
+    const NoteStamp stamp = stamp_of_image(tree, cam, n_images, opt);
+    launch_backward<ImageSource<float>, float>(tree, image_source<float>(cam, n_images, pose_stride), opt, od, nullptr,
+                                               nullptr, workspace, workspace_bytes, n_slots, (hipStream_t)stream,
+                                               kForwardNoted, out, &stamp);
+    return check_launch("volume_render_images_noted");
+}
+
+int svox_volume_render_images_backward_noted(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
+                                             int64_t pose_stride, const SvoxRenderOptions* opt,
+                                             const void* grad_output, void* grad_data_out, int32_t accumulate,
+                                             void* workspace, int64_t workspace_bytes, void* stream) {
+    int od;
+    int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    rc = check_camera(cam, n_images, pose_stride);
+    if (rc) return rc;
+    if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
+    const int64_t n_slots = (int64_t)n_images * cam->width * cam->height;
+    if (!noted_ok(tree, opt, n_slots, workspace, workspace_bytes))
+        return svox_volume_render_images_backward_ws(tree, cam, n_images, pose_stride, opt, grad_output, grad_data_out,
+                                                     accumulate, workspace, workspace_bytes, stream);
+    if (!grad_data_out) return fail(SVOX_ERR_NULL_POINTER, "grad_data_out is NULL");
+    if (!accumulate) {
+        rc = zero_fill(grad_data_out, data_bytes(tree), (hipStream_t)stream);
+        if (rc) return rc;
     }
-    return check_launch("volume_render_backward_noted");
+    if (n_slots == 0) return SVOX_OK;
+    if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
+    const ImageSource<float> all = image_source<float>(cam, n_images, pose_stride);
+    return backward_from_notes(tree, all, all, opt, grad_output, grad_data_out, workspace, workspace_bytes, n_slots,
+                               stamp_of_image(tree, cam, n_images, opt), (hipStream_t)stream);
 }
 
 int svox_volume_render(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt, void* out,

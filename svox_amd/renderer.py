@@ -69,37 +69,35 @@ def _versions(tree, rays):
 
 
 class _VolumeRenderImageFunction(torch.autograd.Function):
-    """svox/renderer.py:74-89"""
+    """svox/renderer.py:74-89; one pose (3, 4) / (4, 4) or, beyond the reference, a stack of poses
+    rendered in one launch.  Notes are kept between the passes as in _VolumeRenderFunction."""
 
     @staticmethod
     def forward(ctx, data, tree, cam, opt):
-        out = _C.volume_render_image(tree, cam, opt)
         ctx.tree, ctx.cam, ctx.opt = tree, cam, opt
-        return out
+        ctx.notes = None
+        if ctx.needs_input_grad[0]:
+            out, ctx.notes = _C.volume_render_images_noted(tree, cam, opt)
+            ctx.versions = _image_versions(tree, cam)
+            return out
+        return _C.volume_render_image(tree, cam, opt) if cam.c2w.dim() == 2 else _C.volume_render_images(tree, cam, opt)
 
     @staticmethod
     def backward(ctx, grad_out):
         if not ctx.needs_input_grad[0]:
             return None, None, None, None
-        grad = _C.volume_render_image_backward(ctx.tree, ctx.cam, ctx.opt, grad_out.contiguous())
+        notes, ctx.notes = ctx.notes, None
+        if notes is not None and ctx.versions != _image_versions(ctx.tree, ctx.cam):
+            notes = None
+        grad = _C.volume_render_images_backward_noted(ctx.tree, ctx.cam, ctx.opt, grad_out.contiguous(), notes)
         return grad, None, None, None
 
 
-class _VolumeRenderImagesFunction(torch.autograd.Function):
-    """Several poses in one launch (no counterpart in the reference)."""
+_VolumeRenderImagesFunction = _VolumeRenderImageFunction
 
-    @staticmethod
-    def forward(ctx, data, tree, cam, opt):
-        out = _C.volume_render_images(tree, cam, opt)
-        ctx.tree, ctx.cam, ctx.opt = tree, cam, opt
-        return out
 
-    @staticmethod
-    def backward(ctx, grad_out):
-        if not ctx.needs_input_grad[0]:
-            return None, None, None, None
-        grad = _C.volume_render_images_backward(ctx.tree, ctx.cam, ctx.opt, grad_out.contiguous())
-        return grad, None, None, None
+def _image_versions(tree, cam):
+    return tuple(t._version for t in (tree.data, tree.child, cam.c2w))
 
 
 def convert_to_ndc(origins, directions, focal, w, h, near=1.0):

@@ -119,6 +119,12 @@ def test_image_render_and_backward(gpu, oracle_mod, ndc):
     grad = C.volume_render_image_backward(dev._spec(), cam, opt, go.to(gpu), workspace=False)
     err, ok = grad_close(grad.cpu().numpy(), ref_grad)
     assert ok, err
+    # and from the notes of a forward pass that keeps them
+    noted, notes = C.volume_render_images_noted(dev._spec(), cam, opt)
+    assert notes is not None and torch.equal(noted, out)
+    grad = C.volume_render_images_backward_noted(dev._spec(), cam, opt, go.to(gpu), notes)
+    err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+    assert ok, err
     # the batch kernels on the oracle's pixel rays give the same picture
     ro, rd, rv = oracle_mod.image_rays(oracle_mod.Tree.from_n3tree(tree), c2w, fx, fx, W, H, opt)
     assert np.isfinite(rd).all()
