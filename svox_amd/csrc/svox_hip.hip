@@ -339,13 +339,12 @@ NoteStamp stamp_of(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const Svo
 constexpr int64_t kStampOffset = 0;
 constexpr int64_t kStockCounterOffset = 128;
 int64_t bitmap_bytes(int64_t n_slots) { return ((n_slots + 63) / 64 * 8 + 15) / 16 * 16; }
-bool carve_workspace(void* workspace, int64_t workspace_bytes, int64_t n_slots, unsigned blocks, ReplaySpace* ws) {
+bool carve_workspace(void* workspace, int64_t workspace_bytes, int64_t n_slots, ReplaySpace* ws) {
     *ws = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0}, nullptr, nullptr};
     const int64_t chunks = workspace && n_slots > 0
                                ? (workspace_bytes - kTailBytes - bitmap_bytes(n_slots)) / kChunkBytes : 0;
     if (n_slots <= 0 || chunks < n_slots || chunks >= 0x7fffffffll || ((uintptr_t)workspace & 15u) != 0) return false;
     ws->base = (float2*)workspace;
-    (void)blocks;
     ws->first_shared = n_slots;
     ws->n_chunks = chunks;
     ws->undone = (unsigned long long*)((char*)workspace + chunks * kChunkBytes);
@@ -368,9 +367,9 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
             const Source dealt = dealt_out(src, blocks);
-            // every ray owns one chunk; what is left of the workspace is dealt out to the blocks
+            // every ray owns one chunk; the wavefronts draw on what is left of the workspace
             ReplaySpace ws;
-            if (carve_workspace(workspace, workspace_bytes, n_slots, blocks, &ws) &&
+            if (carve_workspace(workspace, workspace_bytes, n_slots, &ws) &&
                 zero_fill(ws.stocks_taken, 16, stream) == SVOX_OK) {
                 if (stamp) memcpy(ws.stamp, stamp->word, sizeof(ws.stamp));
                 if (mode == kBackwardPlain) mode = kBackwardReplay;
@@ -452,7 +451,7 @@ bool noted_ok(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, int64_t n_
     if (tree->dtype != SVOX_F32 || fast_basis(tree, opt) < 0 || tree->weight_accum) return false;
     if (!(opt->sigma_thresh >= 0.0f)) return false;
     ReplaySpace ws;
-    return carve_workspace(workspace, workspace_bytes, n_slots, 1, &ws);
+    return carve_workspace(workspace, workspace_bytes, n_slots, &ws);
 }
 
 NoteStamp stamp_of_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
@@ -472,7 +471,7 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
     const int D = fast_basis(tree, opt);
     const unsigned words = blocks_for(n_slots, kMarchThreads);
     ReplaySpace ws;
-    carve_workspace(workspace, workspace_bytes, n_slots, 1, &ws);
+    carve_workspace(workspace, workspace_bytes, n_slots, &ws);
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P, Source>), dim3(words), dim3(kMarchThreads), 0,
                                                stream, all, *opt, (const float*)grad_output, (float*)grad_data_out, ws));

@@ -32,6 +32,11 @@ def _make_camera_spec(c2w, width, height, fx, fy):
     return spec
 
 
+# Whether a forward pass that will be differentiated keeps notes for its backward pass (faster
+# training steps; the forward pass itself takes longer, as it follows every ray to its end).
+KEEP_NOTES = True
+
+
 class _VolumeRenderFunction(torch.autograd.Function):
     """svox/renderer.py:57-72.  The specs are kept on ctx as plain attributes, so the backward
     pass sees the tree as it is when backward runs.
@@ -45,7 +50,7 @@ class _VolumeRenderFunction(torch.autograd.Function):
     def forward(ctx, data, tree, rays, opt):
         ctx.tree, ctx.rays, ctx.opt = tree, rays, opt
         ctx.notes = None
-        if ctx.needs_input_grad[0]:
+        if KEEP_NOTES and ctx.needs_input_grad[0]:
             out, ctx.notes = _C.volume_render_noted(tree, rays, opt)
             ctx.versions = _versions(tree, rays)
             return out
@@ -76,7 +81,7 @@ class _VolumeRenderImageFunction(torch.autograd.Function):
     def forward(ctx, data, tree, cam, opt):
         ctx.tree, ctx.cam, ctx.opt = tree, cam, opt
         ctx.notes = None
-        if ctx.needs_input_grad[0]:
+        if KEEP_NOTES and ctx.needs_input_grad[0]:
             out, ctx.notes = _C.volume_render_images_noted(tree, cam, opt)
             ctx.versions = _image_versions(tree, cam)
             return out
