@@ -479,3 +479,49 @@ def test_autograd_uses_notes_and_marches_again_after_a_write(gpu, oracle_mod):
     out.backward(go)
     err, ok = grad_close(tree.data.grad.cpu().numpy(), oracle_grad())
     assert ok, err
+
+
+def test_noted_entry_points_argument_handling(gpu, oracle_mod):
+    """svox_volume_render_noted / _backward_noted through the C ABI: without a usable workspace they are
+    the plain operators; a negative size and missing buffers are errors."""
+    import ctypes
+    from svox_amd.csrc import _abi
+    tree = synth.shell_tree(depth=5, n_spheres=4, data_format="SH4", seed=2, sigma_range=(2.0, 20.0))
+    rays = synth.sphere_rays(700, seed=1)
+    opt = options(tree, step_size=1e-3, fast=True)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    ref = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    go = torch.randn(700, 3, generator=torch.Generator().manual_seed(5))
+    want = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    dev = on_gpu(tree, gpu)
+    lib = _abi.load_library()
+    spec = C._pack_tree(dev._spec())
+    rs_obj = rays_spec(rays, gpu)
+    rs = C._pack_rays(rs_obj, torch.float32)
+    copt = opt._pack()
+    go_d = go.to(gpu)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    enough = int(lib.svox_volume_render_backward_workspace_bytes(700, 30))
+    buf = torch.zeros(enough + 64, dtype=torch.uint8, device=gpu)
+    for ptr, nbytes in [(None, 0), (buf.data_ptr() + 4, enough), (buf.data_ptr(), 700 * 384), (buf.data_ptr(), enough)]:
+        out = torch.full((700, 3), 7.0, device=gpu)
+        rc = lib.svox_volume_render_noted(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), out.data_ptr(),
+                                          ptr, nbytes, stream)
+        assert rc == 0, lib.svox_last_error()
+        assert np.array_equal(out.cpu().numpy(), ref)
+        grad = torch.full_like(dev.data.data, 7.0)
+        rc = lib.svox_volume_render_backward_noted(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt),
+                                                   go_d.data_ptr(), grad.data_ptr(), 0, ptr, nbytes, stream)
+        assert rc == 0, lib.svox_last_error()
+        err, ok = grad_close(grad.cpu().numpy(), want)
+        assert ok, (nbytes, err)
+    out = torch.empty(700, 3, device=gpu)
+    rc = lib.svox_volume_render_noted(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), out.data_ptr(),
+                                      buf.data_ptr(), -1, stream)
+    assert rc < 0 and b"workspace" in lib.svox_last_error()
+    rc = lib.svox_volume_render_noted(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), None,
+                                      buf.data_ptr(), enough, stream)
+    assert rc < 0 and b"out" in lib.svox_last_error()
+    rc = lib.svox_volume_render_backward_noted(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt),
+                                               go_d.data_ptr(), None, 0, buf.data_ptr(), enough, stream)
+    assert rc < 0 and b"grad_data_out" in lib.svox_last_error()
