@@ -525,3 +525,36 @@ def test_noted_entry_points_argument_handling(gpu, oracle_mod):
     rc = lib.svox_volume_render_backward_noted(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt),
                                                go_d.data_ptr(), None, 0, buf.data_ptr(), enough, stream)
     assert rc < 0 and b"grad_data_out" in lib.svox_last_error()
+
+
+def test_training_step_in_a_hip_graph(gpu):
+    """The entry points allocate nothing and clear with a kernel, so a caller may capture them: a noted
+    forward + backward recorded once and replayed, with eager work in between, gives the eager result
+    every time (the tree's data changes between the replays)."""
+    tree = on_gpu(synth.shell_tree(depth=6, n_spheres=6, data_format="SH9", seed=37, sigma_range=(20.0, 200.0)), gpu)
+    rays = synth.sphere_rays(5000, seed=4)
+    rs = rays_spec(rays, gpu)
+    opt = options(tree, step_size=1e-3, fast=True)
+    go = (torch.randn(5000, 3, generator=torch.Generator().manual_seed(2)) * 1e-2).to(gpu)
+    spec = tree._spec()
+
+    def eager():
+        out, notes = C.volume_render_noted(spec, rs, opt)
+        return out, C.volume_render_backward_noted(spec, rs, opt, go, notes)
+
+    eager()                                  # loads the library and its kernels outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_out, g_notes = C.volume_render_noted(spec, rs, opt)
+        g_grad = C.volume_render_backward_noted(spec, rs, opt, go, g_notes)
+    for step in range(3):
+        with torch.no_grad():
+            tree.data[..., -1] *= 0.9        # eager work between the replays: the densities change
+        want_out, want_grad = eager()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_out, want_out), step
+        err, ok = grad_close(g_grad.cpu().numpy(), want_grad.cpu().numpy())
+        assert ok, (step, err)
