@@ -37,6 +37,13 @@ def _make_camera_spec(c2w, width, height, fx, fy):
 KEEP_NOTES = True
 
 
+def _wants_notes(data):
+    """True when a forward pass started now will be followed by a backward pass.  Asked before
+    Function.apply: inside Function.forward gradient mode is always off, and needs_input_grad is
+    also set inside torch.no_grad(), where no graph is recorded."""
+    return KEEP_NOTES and torch.is_grad_enabled() and data.requires_grad
+
+
 class _VolumeRenderFunction(torch.autograd.Function):
     """svox/renderer.py:57-72.  The specs are kept on ctx as plain attributes, so the backward
     pass sees the tree as it is when backward runs.
@@ -47,10 +54,10 @@ class _VolumeRenderFunction(torch.autograd.Function):
     the two passes (their version counters tell), the backward pass marches as the reference does."""
 
     @staticmethod
-    def forward(ctx, data, tree, rays, opt):
+    def forward(ctx, data, tree, rays, opt, keep_notes=False):
         ctx.tree, ctx.rays, ctx.opt = tree, rays, opt
         ctx.notes = None
-        if KEEP_NOTES and ctx.needs_input_grad[0]:
+        if keep_notes:
             out, ctx.notes = _C.volume_render_noted(tree, rays, opt)
             ctx.versions = _versions(tree, rays)
             return out
@@ -59,13 +66,13 @@ class _VolumeRenderFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         if not ctx.needs_input_grad[0]:
-            return None, None, None, None
+            return None, None, None, None, None
         notes, ctx.notes = ctx.notes, None
         if notes is not None and ctx.versions == _versions(ctx.tree, ctx.rays):
             grad = _C.volume_render_backward_noted(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous(), notes)
         else:
             grad = _C.volume_render_backward(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous())
-        return grad, None, None, None
+        return grad, None, None, None, None
 
 
 def _versions(tree, rays):
@@ -78,10 +85,10 @@ class _VolumeRenderImageFunction(torch.autograd.Function):
     rendered in one launch.  Notes are kept between the passes as in _VolumeRenderFunction."""
 
     @staticmethod
-    def forward(ctx, data, tree, cam, opt):
+    def forward(ctx, data, tree, cam, opt, keep_notes=False):
         ctx.tree, ctx.cam, ctx.opt = tree, cam, opt
         ctx.notes = None
-        if KEEP_NOTES and ctx.needs_input_grad[0]:
+        if keep_notes:
             out, ctx.notes = _C.volume_render_images_noted(tree, cam, opt)
             ctx.versions = _image_versions(tree, cam)
             return out
@@ -90,12 +97,12 @@ class _VolumeRenderImageFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         if not ctx.needs_input_grad[0]:
-            return None, None, None, None
+            return None, None, None, None, None
         notes, ctx.notes = ctx.notes, None
         if notes is not None and ctx.versions != _image_versions(ctx.tree, ctx.cam):
             notes = None
         grad = _C.volume_render_images_backward_noted(ctx.tree, ctx.cam, ctx.opt, grad_out.contiguous(), notes)
-        return grad, None, None, None
+        return grad, None, None, None, None
 
 
 _VolumeRenderImagesFunction = _VolumeRenderImageFunction
@@ -165,7 +172,8 @@ class VolumeRenderer(nn.Module):
         """Render a batch of rays -> (B, rgb_dim).  `fast` sets sigma_thresh = stop_thresh = 1e-2."""
         self._require_gpu(cuda, "VolumeRenderer.forward")
         return _VolumeRenderFunction.apply(self.tree.data, self.tree._spec(),
-                                           _rays_spec_from_rays(rays), self._get_options(fast))
+                                           _rays_spec_from_rays(rays), self._get_options(fast),
+                                           _wants_notes(self.tree.data))
 
     def render_persp(self, c2w, width=800, height=800, fx=1111.111, fy=None, cuda=True, fast=False):
         """Render a pinhole image -> (height, width, rgb_dim).  c2w is (3, 4) or (4, 4), OpenGL
@@ -179,7 +187,8 @@ class VolumeRenderer(nn.Module):
         cam = _make_camera_spec(c2w.to(dtype=self.tree.data.dtype, device=self.tree.data.device).contiguous(),
                                 width, height, fx, fy)
         fn = _VolumeRenderImagesFunction if c2w.dim() == 3 else _VolumeRenderImageFunction
-        return fn.apply(self.tree.data, self.tree._spec(), cam, self._get_options(fast))
+        return fn.apply(self.tree.data, self.tree._spec(), cam, self._get_options(fast),
+                        _wants_notes(self.tree.data))
 
     def se_grad(self, rays, colors):
         """Rendered colour plus gradient and Hessian diagonal (Gauss-Newton: squared Jacobian rows) of

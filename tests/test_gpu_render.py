@@ -485,6 +485,40 @@ def test_autograd_uses_notes_and_marches_again_after_a_write(gpu, oracle_mod):
     assert ok, err
 
 
+def test_no_notes_are_kept_where_no_gradient_is_recorded(gpu, monkeypatch):
+    """Inside torch.no_grad(), or for a tree whose data does not require a gradient, the renderer
+    calls the plain forward operators (which stop rays early); with a gradient on, the noted ones.
+    The images are the same either way."""
+    from svox_amd import renderer as rmod
+    tree = on_gpu(synth.shell_tree(depth=5, n_spheres=4, data_format="SH4", seed=5, sigma_range=(20.0, 200.0)), gpu)
+    rays = synth.sphere_rays(900, seed=2)
+    rays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.dirs.clone().to(gpu))
+    r = svox.VolumeRenderer(tree, step_size=1e-3)
+    c2w = synth.orbit_poses(1, seed=4, radius=2.5)[0].to(gpu)
+    calls = []
+    for name in ("volume_render", "volume_render_noted", "volume_render_image", "volume_render_images",
+                 "volume_render_images_noted"):
+        def counted(*a, _f=getattr(rmod._C, name), _n=name, **kw):
+            calls.append(_n)
+            return _f(*a, **kw)
+        monkeypatch.setattr(rmod._C, name, counted)
+    assert tree.data.requires_grad
+    with torch.no_grad():
+        plain = r(rays, fast=True)
+        plain_img = r.render_persp(c2w, width=96, height=64, fx=80.0, fast=True)
+    assert calls == ["volume_render", "volume_render_image"], calls
+    calls.clear()
+    noted = r(rays, fast=True)
+    noted_img = r.render_persp(c2w, width=96, height=64, fx=80.0, fast=True)
+    assert calls == ["volume_render_noted", "volume_render_images_noted"], calls
+    assert noted.grad_fn is not None and plain.grad_fn is None
+    assert torch.equal(plain, noted) and torch.equal(plain_img, noted_img)
+    calls.clear()
+    tree.data.requires_grad_(False)
+    r(rays, fast=True)
+    assert calls == ["volume_render"], calls
+
+
 def test_noted_entry_points_argument_handling(gpu, oracle_mod):
     """svox_volume_render_noted / _backward_noted through the C ABI: without a usable workspace they are
     the plain operators; a negative size and missing buffers are errors."""
