@@ -264,6 +264,22 @@ int svox_se_grad(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxR
 int svox_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
                        const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out, void* stream);
 
+/* svox_se_grad / svox_se_grad_image with a caller workspace (no reference counterpart: the reference
+ * marches every ray three times, rt_kernel.cu:518-710): one march notes the leaves with sigma > 0 of
+ * every ray in the workspace, the residual, gradient and Hessian terms are then formed from the notes.
+ * Same terms, same results as the plain entry points up to the order of the atomic additions; the
+ * rendered colour is bit-identical.  The workspace is the one of svox_volume_render_backward_ws
+ * (svox_volume_render_backward_workspace_bytes(n_rays or H * W, per_ray); 16-byte aligned); rays whose
+ * notes do not fit are marched as without a workspace.  Without a usable workspace, with fp64 data or
+ * options the octree kernels do not cover, the call is the plain one.  The notes left in the workspace
+ * are those svox_volume_render_noted would leave with both thresholds at zero. */
+int svox_se_grad_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
+                    const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+int svox_se_grad_image_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
+                          const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
 /* grid_weight_render(data, CameraSpec&, RenderOptions&, offset, scaling) -> {grid_weight, grid_hit};
  * svox.cpp:38-40, 120, rt_kernel.cu:1174-1203 (kernel :898-1003).
  * Marches the pixel rays of one camera through a dense density grid data (reso, reso, reso): per

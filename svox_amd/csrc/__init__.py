@@ -516,9 +516,11 @@ def _se_out_dim(spec, opt):
     return od
 
 
-def se_grad(tree, rays, color, opt):
+def se_grad(tree, rays, color, opt, workspace=True):
     """(result (B, C), grad, hessdiag) of 0.5 * |render - color|^2, grad and hessdiag like tree.data;
-    svox.cpp:115, rt_kernel.cu:1111-1139.  Argument order as in the reference: color before opt."""
+    svox.cpp:115, rt_kernel.cu:1111-1139.  Argument order as in the reference: color before opt.
+    With `workspace` (default) the rays are marched once and their notes used for the rest
+    (svox_se_grad_ws); without, the rays are marched twice."""
     spec = _pack_tree(tree)
     rspec = _pack_rays(rays, tree.data.dtype)
     od = _se_out_dim(spec, opt)
@@ -527,15 +529,17 @@ def se_grad(tree, rays, color, opt):
     grad = torch.empty_like(tree.data)
     hessdiag = torch.empty_like(tree.data)
     copt = opt._pack()
+    ws, ws_bytes = _backward_workspace(tree, rspec.n_rays) if workspace else (None, 0)
     with torch.cuda.device(tree.data.device):
-        _call("svox_se_grad", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt), color.data_ptr(),
-              result.data_ptr(), grad.data_ptr(), hessdiag.data_ptr(), _stream(tree.data.device))
+        _call("svox_se_grad_ws", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt), color.data_ptr(),
+              result.data_ptr(), grad.data_ptr(), hessdiag.data_ptr(), ws.data_ptr() if ws is not None else None,
+              ws_bytes, _stream(tree.data.device))
     return result, grad, hessdiag
 
 
-def se_grad_persp(tree, cam, opt, color):
+def se_grad_persp(tree, cam, opt, color, workspace=True):
     """Image version: color and result are (H, W, C); svox.cpp:116, rt_kernel.cu:1141-1173.
-    Argument order as in the reference: opt before color."""
+    Argument order as in the reference: opt before color.  `workspace` as in se_grad."""
     spec = _pack_tree(tree)
     cspec = _pack_camera(cam, tree.data.dtype)
     od = _se_out_dim(spec, opt)
@@ -544,9 +548,11 @@ def se_grad_persp(tree, cam, opt, color):
     grad = torch.empty_like(tree.data)
     hessdiag = torch.empty_like(tree.data)
     copt = opt._pack()
+    ws, ws_bytes = _backward_workspace(tree, cspec.height * cspec.width) if workspace else (None, 0)
     with torch.cuda.device(tree.data.device):
-        _call("svox_se_grad_image", ctypes.byref(spec), ctypes.byref(cspec), ctypes.byref(copt), color.data_ptr(),
-              result.data_ptr(), grad.data_ptr(), hessdiag.data_ptr(), _stream(tree.data.device))
+        _call("svox_se_grad_image_ws", ctypes.byref(spec), ctypes.byref(cspec), ctypes.byref(copt),
+              color.data_ptr(), result.data_ptr(), grad.data_ptr(), hessdiag.data_ptr(),
+              ws.data_ptr() if ws is not None else None, ws_bytes, _stream(tree.data.device))
     return result, grad, hessdiag
 
 

@@ -143,6 +143,12 @@ SIGNATURES = {
     "svox_se_grad_image": (
         ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p, c_void_p,
                        c_void_p]),
+    "svox_se_grad_ws": (
+        ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p, c_void_p,
+                       c_void_p, c_int64, c_void_p]),
+    "svox_se_grad_image_ws": (
+        ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p, c_void_p,
+                       c_void_p, c_int64, c_void_p]),
     "svox_grid_weight_render": (
         ctypes.c_int, [c_void_p, c_int32, c_int32, P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p,
                        c_void_p, c_void_p]),

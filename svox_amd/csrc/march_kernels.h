@@ -890,6 +890,44 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
 // and added together: the n * K scalars of the list flat, scalar f from lane f mod 64, so that every
 // atomic instruction covers 64 consecutive scalars whatever K is.  The list is flushed when it is
 // full and at the end of the round.
+// Adds the n records of a list, K elements each, with the lanes tied to elements: the list is cut
+// into 64 / K slices of consecutive records and lane l serves element l % K of slice l / K (of every
+// record, in two or more steps, if K > 64).  Which element a lane serves never changes, so an
+// addition costs about half the instructions of running over the flat list; the price is idle lanes
+// where K does not divide 64.  Consecutive records of the same leaf (neighbouring rays of an image)
+// are summed in registers and added once.  term(rec, e, t) gives the NV values of element e of
+// record rec, emit(leaf, e, sum) adds them.
+template <int K, int NV, class Term, class Emit>
+__device__ __forceinline__ void add_records_by_leaf(int n, int lane, const int32_t* leaves, Term&& term,
+                                                    Emit&& emit) {
+    constexpr int kPer = K <= kMarchThreads ? kMarchThreads / K : 1;
+    const int r = K <= kMarchThreads ? lane / K : 0;
+    if (r >= kPer) return;
+    const int per = (n + kPer - 1) / kPer;
+    const int lo = r * per;
+    const int hi = lo + per < n ? lo + per : n;
+    for (int e = K <= kMarchThreads ? lane - r * K : lane; e < K; e += kMarchThreads) {
+        int32_t cur = -1;
+        float acc[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
+        for (int rec = lo; rec < hi; ++rec) {
+            const int32_t leaf = leaves[rec];
+            if (leaf != cur) {
+                if (cur >= 0) emit(cur, e, acc);
+                cur = leaf;
+#pragma unroll
+                for (int v = 0; v < NV; ++v) acc[v] = 0.0f;
+            }
+            float t[NV];
+            term(rec, e, t);
+#pragma unroll
+            for (int v = 0; v < NV; ++v) acc[v] += t[v];
+        }
+        if (cur >= 0) emit(cur, e, acc);
+    }
+}
+
 constexpr int kEmitCap = 60;   // 60 * (leaf 4 + g_sigma 4 + tmp2 12 + owner 1) = 1260 of 1280 bytes
 template <class P, int D, bool kByRecord = false>
 struct RecordList {
@@ -931,44 +969,23 @@ struct RecordList {
         n = 0;
     }
 
-    // The same additions with the lanes tied to elements instead of running over the flat list: lane l
-    // adds element l % K of record l / K of every group of 64 / K records (of every record, in two or
-    // more steps, if K > 64).  Which record and which element a lane serves never changes, so an
-    // addition costs about half the instructions of the flat form; the price is idle lanes where K
-    // does not divide 64.  (Measured: 12 % off replay_backward_kernel, whose time is mostly these
-    // additions; nothing for render_backward_kernel.)
+    // The same additions by add_records_by_leaf.  (Measured: 12 % off replay_backward_kernel, whose
+    // time is mostly these additions; nothing for render_backward_kernel.)
     __device__ __forceinline__ void flush_by_record() {
         if (n == 0) return;
         wave_lds_sync();
-        if constexpr (K <= kMarchThreads) {
-            constexpr int kPer = kMarchThreads / K;          // records per step
-            const int r = lane / K, e = lane - r * K;
-            const bool in_range = r < kPer;
-            const int c = e / D, i = e - c * D;
-            const bool colour = P::kFormat == SVOX_FORMAT_RGBA ? e < 3 : e < 3 * D;
-            for (int rec0 = 0; rec0 < n; rec0 += kPer) {
-                const int rec = rec0 + r;
-                if (in_range && rec < n) {
-                    float val;
-                    if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                        val = colour ? tmp2s()[rec * 3 + e] : g_sigmas()[rec];
-                    } else {
-                        val = colour ? sh.basis[owners()[rec] * D + i] * tmp2s()[rec * 3 + c] : g_sigmas()[rec];
-                    }
-                    atomicAdd(grad_data + (int64_t)leaves()[rec] * K + e, val);
+        add_records_by_leaf<K, 1>(
+            n, lane, leaves(),
+            [&](int rec, int e, float* t) {
+                const int c = P::kFormat == SVOX_FORMAT_RGBA ? e : e / D;
+                if (c < 3) {
+                    const float v = tmp2s()[rec * 3 + c];
+                    t[0] = P::kFormat == SVOX_FORMAT_RGBA ? v : sh.basis[owners()[rec] * D + (e - c * D)] * v;
+                } else {
+                    t[0] = g_sigmas()[rec];
                 }
-            }
-        } else {
-            for (int rec = 0; rec < n; ++rec) {
-                const int64_t at = (int64_t)leaves()[rec] * K;
-                const int owner = owners()[rec];
-                for (int e = lane; e < K; e += kMarchThreads) {
-                    const int c = e / D;
-                    const float val = e < 3 * D ? sh.basis[owner * D + (e - c * D)] * tmp2s()[rec * 3 + c] : g_sigmas()[rec];
-                    atomicAdd(grad_data + at + e, val);
-                }
-            }
-        }
+            },
+            [&](int32_t leaf, int e, const float* sum) { atomicAdd(grad_data + (int64_t)leaf * K + e, sum[0]); });
         wave_lds_sync();
         n = 0;
     }
@@ -1022,6 +1039,25 @@ struct ReplaySpace {
     const unsigned long long* only;
 };
 
+// The first ray at or after `next` (a wavefront-uniform ray number below `end`) whose 64-ray word of
+// the bitmap `only` is not zero, found 64 words at a time; a value >= end if there is none.
+__device__ __forceinline__ int64_t skip_clear_words(const unsigned long long* __restrict__ only, int64_t next,
+                                                    int64_t end, int lane) {
+    while (next < end) {
+        const int64_t word = next >> 6, last_word = (end - 1) >> 6;
+        const bool some = word + lane <= last_word && only[word + lane] != 0ull;
+        const unsigned long long nz = __ballot(some);
+        if (nz == 0ull) {
+            next = (word + kMarchThreads) << 6;
+            continue;
+        }
+        const int64_t first = (word + __builtin_ctzll(nz)) << 6;
+        if (first > next) next = first;
+        break;
+    }
+    return next;
+}
+
 // What a launch of render_backward_kernel does:
 //   kBackwardPlain   both marches walk the tree;
 //   kBackwardReplay  march 1 leaves notes in the workspace, march 2 replays them;
@@ -1032,7 +1068,7 @@ enum BackwardMode { kBackwardPlain = 0, kBackwardReplay = 1, kForwardNoted = 2 }
 
 // Head of a ray's notes, kept in the spare floats of its first chunk (after the 15 records): the
 // link to the next chunk, the number of notes (-1: they did not fit; 0 also for a ray that misses
-// the tree) and the ray's delta_scale (rt_kernel.cu:228).
+// the tree), the ray's delta_scale (rt_kernel.cu:228) and 1.0f if the ray misses the tree, else 0.0f.
 constexpr int kChunkRecords = 15;
 constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
 constexpr int kHeadFloat2 = kChunkRecords * 3;          // float2 index of {link, count}, then {delta_scale, -}
@@ -1133,6 +1169,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             out[slot * 3 + 1] = bg;
             out[slot * 3 + 2] = bg;
             ws.base[slot * kChunkFloat2 + kHeadFloat2] = make_float2(0.0f, __int_as_float(0));   // no notes
+            ws.base[slot * kChunkFloat2 + kHeadFloat2 + 1] = make_float2(0.0f, 1.0f);            // missed
         }
     };
     if constexpr (!kRefill) {
@@ -1141,21 +1178,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 
     while (true) {
         if constexpr (kRefill) {
-            if (Source::kItemsAreSlots && ws.only) {
-                // skip the 64-ray words of the bitmap in which no ray is left to do, 64 words at a time
-                while (next < end) {
-                    const int64_t word = next >> 6, last_word = (end - 1) >> 6;
-                    const bool some = word + lane <= last_word && ws.only[word + lane] != 0ull;
-                    const unsigned long long nz = __ballot(some);
-                    if (nz == 0ull) {
-                        next = (word + kMarchThreads) << 6;
-                        continue;
-                    }
-                    const int64_t first = (word + __builtin_ctzll(nz)) << 6;
-                    if (first > next) next = first;
-                    break;
-                }
-            }
+            if (Source::kItemsAreSlots && ws.only) next = skip_clear_words(ws.only, next, end, lane);
             const RoundState state = refill_lanes(active, next, end, src.refill_at, start);
             if (state == kRoundRefilled) continue;
             if (state == kRoundDone) break;
@@ -1668,7 +1691,8 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
                                                                 const float* __restrict__ color_ref,
                                                                 float* __restrict__ color_out,
                                                                 float* __restrict__ grad_data,
-                                                                float* __restrict__ hess_data) {
+                                                                float* __restrict__ hess_data,
+                                                                const unsigned long long* __restrict__ only) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
@@ -1696,10 +1720,14 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
     cur.reset(path + lane, kMarchThreads);
 
     // takes ray `item` into this lane: a miss is answered at once, a hit becomes the lane's ray
+    // (with a bitmap `only` the launch does the rays whose bit is set and no others; a batch launch
+    // then does not deal its rays out: its items are ray numbers)
     auto start = [&](int64_t item) {
         float origin[3], dir[3], vdir[3];
+        if (Source::kItemsAreSlots && only && !((only[item >> 6] >> (item & 63)) & 1ull)) return;
         slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
         if (slot < 0) return;
+        if (!Source::kItemsAreSlots && only && !((only[slot >> 6] >> (slot & 63)) & 1ull)) return;
         if (setup_ray(r, origin, dir, scaling)) {
             if constexpr (P::kFormat == SVOX_FORMAT_SH) {
                 float basis[D];
@@ -1730,6 +1758,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
 
     while (true) {
         if constexpr (kRefill) {
+            if (Source::kItemsAreSlots && only) next = skip_clear_words(only, next, end, lane);
             const RoundState state = refill_lanes(active, next, end, src.refill_at, start);
             if (state == kRoundRefilled) continue;
             if (state == kRoundDone) break;
@@ -1851,6 +1880,219 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
             }
         }
     }
+}
+
+// se_grad from the notes render_backward_kernel<kForwardNoted> left (taken with both thresholds at
+// zero): one lane per ray, no tree walk.  The first pass over a ray's notes forms the residual and the
+// rendered colour as march 1 of se_grad_kernel does, the second pass the gradient and Hessian records
+// of its march 2, term by term the same values; the wavefront adds the records of its rays together,
+// each lane serving one element of one record (RecordList::flush_by_record's scheme, with two output
+// arrays).  Rays that miss the tree keep the background colour the noting launch wrote; a ray whose
+// notes are incomplete, or every ray if the workspace carries another stamp, is marked in the bitmap
+// for a launch of se_grad_kernel.
+constexpr int kSeRecordCap = 48;
+
+template <class P, class Source>
+__global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source src, SvoxRenderOptions opt,
+                                                                       const float* __restrict__ color_ref,
+                                                                       float* __restrict__ color_out,
+                                                                       float* __restrict__ grad_data,
+                                                                       float* __restrict__ hess_data,
+                                                                       ReplaySpace ws) {
+    constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
+    constexpr int K = P::kRecord;
+    constexpr bool kRgba = P::kFormat == SVOX_FORMAT_RGBA;
+    __shared__ float basis_rows[kMarchThreads * D];
+    __shared__ float resid_rows[kMarchThreads * 3];
+    __shared__ int32_t l_leaf[kSeRecordCap];
+    __shared__ float l_gs[kSeRecordCap], l_hs[kSeRecordCap], l_gci[kSeRecordCap * 3];
+    __shared__ uint8_t l_owner[kSeRecordCap];
+    const int lane = threadIdx.x;
+    const int64_t ray = blockIdx.x * (int64_t)kMarchThreads + lane;
+    const bool stamped = ws.stamp_at[0] == ws.stamp[0] && ws.stamp_at[1] == ws.stamp[1] &&
+                         ws.stamp_at[2] == ws.stamp[2] && ws.stamp_at[3] == ws.stamp[3];
+    const float2* first = ws.base + ray * kChunkFloat2;
+    int count = 0;
+    int32_t first_link = 0;
+    float dscale = 0.0f;
+    bool missed = true;
+    if (ray < src.n_slots()) {
+        const float2 head = first[kHeadFloat2], tail = first[kHeadFloat2 + 1];
+        first_link = __float_as_int(head.x);
+        count = stamped ? __float_as_int(head.y) : -1;
+        dscale = tail.x;
+        missed = tail.y != 0.0f;
+    }
+    const unsigned long long undone = __ballot(count < 0);
+    if (lane == 0) ws.undone[blockIdx.x] = undone;
+    const bool hit = count >= 0 && !missed;   // the rays this launch answers
+    const bool work = hit && count > 0;
+    if (!__any(hit)) return;
+
+    const float bg = opt.background_brightness;
+    const float pad = opt.rgb_padding;
+    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
+    float ref[3] = {0.f, 0.f, 0.f};
+    if (hit) {
+        ref[0] = color_ref[ray * 3];
+        ref[1] = color_ref[ray * 3 + 1];
+        ref[2] = color_ref[ray * 3 + 2];
+    }
+    if (work) {
+        if constexpr (!kRgba) {
+            float vdir[3];
+            src.view_dir(ray, vdir);
+            float basis[D];
+            sh_basis<float>(P::kBasis, vdir, basis);
+#pragma unroll
+            for (int i = 0; i < D; ++i) basis_rows[lane * D + i] = basis[i];
+        }
+    }
+
+    int n = 0;   // records in the list (wavefront-uniform)
+    auto flush = [&]() {
+        if (n == 0) return;
+        wave_lds_sync();
+        add_records_by_leaf<K, 2>(
+            n, lane, l_leaf,
+            // element e of a record: colour coefficient (c, i) or, last, the density
+            [&](int rec, int e, float* t) {
+                const int c = kRgba ? e : e / D;
+                if (c < 3) {
+                    const int owner = l_owner[rec];
+                    const float v = l_gci[rec * 3 + c];
+                    const float gw = kRgba ? v : basis_rows[owner * D + (e - c * D)] * v;
+                    t[0] = gw * resid_rows[owner * 3 + c];
+                    t[1] = gw * gw;
+                } else {
+                    t[0] = l_gs[rec];
+                    t[1] = l_hs[rec];
+                }
+            },
+            [&](int32_t leaf, int e, const float* sum) {
+                const int64_t at = (int64_t)leaf * K + e;
+                atomicAdd(grad_data + at, sum[0]);
+                atomicAdd(hess_data + at, sum[1]);
+            });
+        wave_lds_sync();
+        n = 0;
+    };
+    // the record of every lane with `emit` set joins the list (in lane order)
+    auto append = [&](bool emit, int32_t leaf, const float* gci, float g_sigma, float h_sigma) {
+        unsigned long long todo = __ballot(emit);
+        while (todo) {
+            if (n == kSeRecordCap) flush();
+            const bool pending = (todo >> lane) & 1ull;
+            const int at = n + rank_in(todo);
+            const bool take = pending && at < kSeRecordCap;
+            if (take) {
+                l_leaf[at] = leaf;
+                l_owner[at] = (uint8_t)lane;
+                l_gs[at] = g_sigma;
+                l_hs[at] = h_sigma;
+                l_gci[at * 3] = gci[0];
+                l_gci[at * 3 + 1] = gci[1];
+                l_gci[at * 3 + 2] = gci[2];
+            }
+            const unsigned long long taken = __ballot(take);
+            n += __popcll(taken);
+            todo &= ~taken;
+        }
+    };
+
+    float resid[3] = {0.f, 0.f, 0.f};    // pass 0: colour so far; afterwards the residual
+    float caccum[3] = {0.f, 0.f, 0.f};   // rendered colour not yet passed (second spelling)
+    float light = 1.0f, light1 = 1.0f;
+    struct Group {
+        float2 note[kReplayGroup][3];
+    };
+#pragma unroll 1
+    for (int pass = 0; pass < 2; ++pass) {
+        const float2* chunk = first;
+        int32_t link = first_link;
+        int pos = 0;
+        auto fetch = [&](Group& g, int base) {
+            if (work && base < count) {
+                if (pos == kChunkRecords) {
+                    chunk = ws.base + (int64_t)link * kChunkFloat2;
+                    link = __float_as_int(chunk[kHeadFloat2].x);
+                    pos = 0;
+                }
+#pragma unroll
+                for (int k = 0; k < kReplayGroup; ++k) {
+#pragma unroll
+                    for (int j = 0; j < 3; ++j) g.note[k][j] = chunk[(pos + k) * 3 + j];
+                }
+                pos += kReplayGroup;
+            }
+        };
+        auto work_on = [&](const Group& g, int base) {
+#pragma unroll
+            for (int k = 0; k < kReplayGroup; ++k) {
+                const bool have = work && base + k < count;
+                const int32_t leaf = __float_as_int(g.note[k][0].x);
+                const float dt = g.note[k][0].y, sigma = g.note[k][1].x;
+                const float s[3] = {g.note[k][1].y, g.note[k][2].x, g.note[k][2].y};
+                float gci[3] = {0.f, 0.f, 0.f};
+                float g_sigma = 0.0f, h_sigma = 0.0f;
+                if (have) {
+                    const float att = expf_fixed(-dt * sigma * dscale);
+                    const float weight = light * (1.0f - att);
+                    float col[3];
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) col[c] = fma_(s[c], d_rgb_pad, -pad);
+                    light *= att;
+                    if (pass == 0) {
+                        const float att1 = expf_fixed(-dt * dscale * sigma);
+                        const float weight1 = light1 * (1.0f - att1);
+                        light1 *= att1;
+#pragma unroll
+                        for (int c = 0; c < 3; ++c) {
+                            resid[c] = fma_(weight1, col[c], resid[c]);
+                            caccum[c] = fma_(weight, col[c], caccum[c]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < 3; ++c) {
+                            if constexpr (kRgba) {
+                                gci[c] = weight * s[c] * (1.0f - s[c]) * d_rgb_pad;
+                            } else {
+                                gci[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)d_rgb_pad);
+                            }
+                            caccum[c] = fma_(-weight, col[c], caccum[c]);
+                            const float gs = dt * dscale * fma_(col[c], light, -caccum[c]);
+                            g_sigma += gs * resid[c];
+                            h_sigma += gs * gs;
+                        }
+                    }
+                }
+                if (pass == 1) append(have, leaf, gci, g_sigma, h_sigma);
+            }
+        };
+        Group a, b;
+        fetch(a, 0);
+        for (int base = 0; __any(work && base < count); base += 2 * kReplayGroup) {
+            fetch(b, base + kReplayGroup);
+            work_on(a, base);
+            fetch(a, base + 2 * kReplayGroup);
+            work_on(b, base + kReplayGroup);
+        }
+        if (pass == 0) {
+            // the end of march 1 (rt_kernel.cu:560-563, the background of :635-637, and :711-713)
+            if (hit) {
+#pragma unroll
+                for (int c = 0; c < 3; ++c) {
+                    resid[c] += fma_(light1, bg, -ref[c]);
+                    caccum[c] = fma_(light, bg, caccum[c]);
+                    color_out[ray * 3 + c] = resid[c] + ref[c];
+                    resid_rows[lane * 3 + c] = resid[c];
+                }
+            }
+            light = 1.0f;
+            wave_lds_sync();   // basis and residual rows are read by other lanes when the records are added
+        }
+    }
+    flush();
 }
 
 // ------------------------------------------------------------------------------------------------

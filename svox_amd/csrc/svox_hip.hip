@@ -400,25 +400,27 @@ int64_t data_bytes(const SvoxTreeSpec* t) {
     return t->capacity * t->N * t->N * t->N * t->data_dim * esz;
 }
 
+// `only`: a bitmap of the rays to do (octree kernels only; the batch rays are then not dealt out)
 template <class Source, typename T>
 void launch_se_grad(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, int out_dim,
-                    const void* color_ref, void* color_out, void* grad, void* hess, hipStream_t stream) {
+                    const void* color_ref, void* color_out, void* grad, void* hess, hipStream_t stream,
+                    const unsigned long long* only = nullptr) {
     const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
-            const Source dealt = dealt_out(src, blocks);
+            const Source dealt = only ? src : dealt_out(src, blocks);
             if (src.per_wave > kMarchThreads) {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source, true>), dim3(blocks),
                                                            dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
                                                            dealt, *opt, (const float*)color_ref, (float*)color_out,
-                                                           (float*)grad, (float*)hess));
+                                                           (float*)grad, (float*)hess, only));
             } else {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source, false>), dim3(blocks),
                                                            dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
                                                            src, *opt, (const float*)color_ref, (float*)color_out,
-                                                           (float*)grad, (float*)hess));
+                                                           (float*)grad, (float*)hess, only));
             }
             return;
         }
@@ -491,6 +493,39 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
                                                    (float*)nullptr));
     }
     return check_launch("volume_render_backward_noted");
+}
+
+// se_grad of the rays of `all` with their notes kept in the workspace between its two halves: one
+// march that takes the notes (thresholds play no part in se_grad, rt_kernel.cu:479-715), then
+// replay_se_grad_kernel; rays it marks in the bitmap are done by se_grad_kernel (`rest`: the launch
+// shape for those).  The caller has checked noted_ok() with the same options.
+template <class Source>
+int se_grad_from_notes(const SvoxTreeSpec* tree, const Source& all, const Source& rest, const SvoxRenderOptions* opt,
+                       const void* color_ref, void* color_out, void* grad, void* hess, void* workspace,
+                       int64_t workspace_bytes, int64_t n_slots, const NoteStamp& stamp, hipStream_t stream) {
+    const int D = fast_basis(tree, opt);
+    launch_backward<Source, float>(tree, all, opt, 3, nullptr, nullptr, workspace, workspace_bytes, n_slots, stream,
+                                   kForwardNoted, color_out, &stamp);
+    int rc = check_launch("se_grad");
+    if (rc) return rc;
+    ReplaySpace ws;
+    carve_workspace(workspace, workspace_bytes, n_slots, &ws);
+    memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_se_grad_kernel<P, Source>), dim3(blocks_for(n_slots, kMarchThreads)),
+                                               dim3(kMarchThreads), 0, stream, all, *opt, (const float*)color_ref,
+                                               (float*)color_out, (float*)grad, (float*)hess, ws));
+    rc = check_launch("se_grad");
+    if (rc) return rc;
+    launch_se_grad<Source, float>(tree, rest, opt, 3, color_ref, color_out, grad, hess, stream, ws.undone);
+    return check_launch("se_grad");
+}
+
+// the options under which se_grad's notes are taken: every leaf with sigma > 0, no early stop
+SvoxRenderOptions without_thresholds(const SvoxRenderOptions* opt) {
+    SvoxRenderOptions o = *opt;
+    o.sigma_thresh = 0.0f;
+    o.stop_thresh = 0.0f;
+    return o;
 }
 
 }  // namespace
@@ -855,6 +890,50 @@ int svox_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, cons
                                                     hessdiag_out, (hipStream_t)stream);
     }
     return check_launch("se_grad_persp");
+}
+
+int svox_se_grad_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
+                    const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out, void* workspace,
+                    int64_t workspace_bytes, void* stream) {
+    if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
+    int od;
+    int rc = check_rays(rays);
+    if (rc) return rc;
+    rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    const SvoxRenderOptions plain = without_thresholds(opt);
+    if (od != 3 || rays->n_rays == 0 || !color_ref || !color_out ||
+        !noted_ok(tree, &plain, rays->n_rays, workspace, workspace_bytes))
+        return svox_se_grad(tree, rays, opt, color_ref, color_out, grad_out, hessdiag_out, stream);
+    rc = se_grad_prepare(tree, opt, grad_out, hessdiag_out, &od, (hipStream_t)stream);
+    if (rc) return rc;
+    const BatchSource<float> all = batch_source<float>(rays, true);
+    BatchSource<float> rest = all;
+    const int64_t words = (rays->n_rays + kMarchThreads - 1) / kMarchThreads;
+    rest.per_wave = (int)((words + kUndoneWaves - 1) / kUndoneWaves) * kMarchThreads;
+    return se_grad_from_notes(tree, all, rest, &plain, color_ref, color_out, grad_out, hessdiag_out, workspace,
+                              workspace_bytes, rays->n_rays, stamp_of(tree, rays, &plain), (hipStream_t)stream);
+}
+
+int svox_se_grad_image_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
+                          const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out,
+                          void* workspace, int64_t workspace_bytes, void* stream) {
+    if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
+    int od;
+    int rc = check_camera(cam, 1, 12);
+    if (rc) return rc;
+    rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    const SvoxRenderOptions plain = without_thresholds(opt);
+    const int64_t n_slots = (int64_t)cam->width * cam->height;
+    if (od != 3 || n_slots == 0 || !color_ref || !color_out ||
+        !noted_ok(tree, &plain, n_slots, workspace, workspace_bytes))
+        return svox_se_grad_image(tree, cam, opt, color_ref, color_out, grad_out, hessdiag_out, stream);
+    rc = se_grad_prepare(tree, opt, grad_out, hessdiag_out, &od, (hipStream_t)stream);
+    if (rc) return rc;
+    const ImageSource<float> all = image_source<float>(cam, 1, 12);
+    return se_grad_from_notes(tree, all, all, &plain, color_ref, color_out, grad_out, hessdiag_out, workspace,
+                              workspace_bytes, n_slots, stamp_of_image(tree, cam, 1, &plain), (hipStream_t)stream);
 }
 
 int svox_grid_weight_render(const void* data, int32_t reso, int32_t dtype, const SvoxCameraSpec* cam,

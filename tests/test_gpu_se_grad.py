@@ -13,13 +13,19 @@ from util import cam_spec, grad_close, on_gpu, options, rays_spec
 pytestmark = pytest.mark.gpu
 
 
-def check(gpu, oracle_mod, tree, rays, ref, opt, exact=True, generic=0):
+# how a call reaches the kernels: debug flags and whether the rays' notes are kept in a workspace
+PATHS = {"generic": (1, False), "marches": (0, False), "notes": (0, True),
+         "marches_large_batch_kernels": (2, False), "notes_large_batch_kernels": (2, True)}
+
+
+def check(gpu, oracle_mod, tree, rays, ref, opt, exact=True, path="notes"):
     ot = oracle_mod.Tree.from_n3tree(tree)
     want = oracle_mod.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, opt, n_threads=4)
     dev = on_gpu(tree, gpu)
-    C.set_debug_flags(generic)
+    flags, workspace = PATHS[path]
+    C.set_debug_flags(flags)
     try:
-        got = C.se_grad(dev._spec(), rays_spec(rays, gpu), ref.to(gpu), opt)
+        got = C.se_grad(dev._spec(), rays_spec(rays, gpu), ref.to(gpu), opt, workspace=workspace)
     finally:
         C.set_debug_flags(0)
     got = [x.cpu().numpy() for x in got]
@@ -34,9 +40,9 @@ def check(gpu, oracle_mod, tree, rays, ref, opt, exact=True, generic=0):
     return got, want
 
 
-@pytest.mark.parametrize("generic", [0, 1])
+@pytest.mark.parametrize("path", list(PATHS))
 @pytest.mark.parametrize("fmt", ["RGBA", "SH1", "SH4", "SH9", "SH16", "SH25"])
-def test_se_grad_sparse_tree(gpu, oracle_mod, fmt, generic):
+def test_se_grad_sparse_tree(gpu, oracle_mod, fmt, path):
     tree = synth.shell_tree(depth=6, n_spheres=6, data_format=fmt, seed=21, sigma_range=(20.0, 200.0))
     rays = synth.sphere_rays(3000, seed=5)
     o = rays.origins.clone()
@@ -45,7 +51,7 @@ def test_se_grad_sparse_tree(gpu, oracle_mod, fmt, generic):
     rays = svox.Rays(o.contiguous(), rays.dirs, rays.viewdirs)
     ref = torch.rand(3000, 3, generator=torch.Generator().manual_seed(7))
     opt = options(tree, step_size=5e-4, background_brightness=0.8)
-    got, want = check(gpu, oracle_mod, tree, rays, ref, opt, generic=generic)
+    got, want = check(gpu, oracle_mod, tree, rays, ref, opt, path=path)
     assert np.all(got[0][:50] == np.float32(0.8))
     assert np.abs(want[2]).max() > 0
 
@@ -84,8 +90,50 @@ def test_se_grad_generic_options_and_double(gpu, oracle_mod):
     check(gpu, oracle_mod, t, r64, ref.double(), options(t, step_size=2e-3))
 
 
+@pytest.mark.parametrize("fmt", ["RGBA", "SH9", "SH25"])
+def test_se_grad_rays_whose_notes_do_not_fit(gpu, oracle_mod, fmt):
+    """Through the C ABI with the smallest workspace (one chunk of 15 notes per ray and nothing to
+    spare) on a dense tree: rays with more leaves than that are marked and marched, the others are
+    done from their notes; together they give the oracle's result."""
+    import ctypes
+    from svox_amd.csrc import _abi
+    tree = synth.dense_tree(3, fmt, seed=4, sigma="lognormal", coeff_std=0.5)
+    n = 1500
+    rays = synth.sphere_rays(n, seed=11)
+    ref = torch.rand(n, 3, generator=torch.Generator().manual_seed(3))
+    opt = options(tree, step_size=1e-3)
+    want = oracle_mod.se_grad(oracle_mod.Tree.from_n3tree(tree), rays.origins, rays.dirs, rays.viewdirs, ref, opt,
+                              n_threads=4)
+    dev = on_gpu(tree, gpu)
+    lib = _abi.load_library()
+    spec = C._pack_tree(dev._spec())
+    dev_rays = rays_spec(rays, gpu)            # owns the device tensors the packed struct points to
+    rs = C._pack_rays(dev_rays, torch.float32)
+    copt = opt._pack()
+    nbytes = int(lib.svox_volume_render_backward_workspace_bytes(n, 15))
+    ws = torch.zeros(nbytes // 8, dtype=torch.float64, device=gpu)
+    colour = torch.empty(n, 3, device=gpu)
+    grad = torch.empty_like(dev.data)
+    hess = torch.empty_like(dev.data)
+    ref_dev = ref.to(gpu)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.svox_se_grad_ws(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), ref_dev.data_ptr(),
+                             colour.data_ptr(), grad.data_ptr(), hess.data_ptr(), ws.data_ptr(), nbytes, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(colour.cpu().numpy(), want[0])
+    for name, g, w in (("grad", grad, want[1]), ("hessdiag", hess, want[2])):
+        err, ok = grad_close(g.cpu().numpy(), w)
+        assert ok, (name, err)
+    # the bitmap of the rays left to the marching kernel sits behind the n chunks of 384 bytes
+    words = ws.view(torch.int64)[n * 384 // 8: n * 384 // 8 + (n + 63) // 64].cpu().numpy().view(np.uint64)
+    undone = sum(bin(int(w)).count("1") for w in words)
+    assert 0 < undone < n, undone
+
+
+@pytest.mark.parametrize("workspace", [False, True])
 @pytest.mark.parametrize("ndc", [False, True])
-def test_se_grad_persp(gpu, oracle_mod, ndc):
+def test_se_grad_persp(gpu, oracle_mod, ndc, workspace):
     tree = synth.shell_tree(depth=6, n_spheres=5, data_format="SH9", seed=33,
                             geometry="noise" if ndc else "spheres")
     W, H, fx = 75, 53, 60.0
@@ -102,7 +150,11 @@ def test_se_grad_persp(gpu, oracle_mod, ndc):
     want = oracle_mod.se_grad_image(oracle_mod.Tree.from_n3tree(tree), c2w, fx, fx, W, H, ref, opt, n_threads=4)
     dev = on_gpu(tree, gpu)
     r = svox.VolumeRenderer(dev, step_size=1e-3, **kw)
-    got = r.se_grad_persp(c2w.to(gpu), ref.to(gpu), width=W, height=H, fx=fx)
+    cam = cam_spec(c2w.to(gpu), W, H, fx)
+    got = C.se_grad_persp(dev._spec(), cam, r._get_options(False), ref.to(gpu), workspace=workspace)
+    if workspace:
+        again = r.se_grad_persp(c2w.to(gpu), ref.to(gpu), width=W, height=H, fx=fx)   # the renderer's default
+        assert torch.equal(again[0], got[0])
     assert got[0].shape == (H, W, 3)
     assert np.array_equal(got[0].cpu().numpy(), want[0])
     for g, w in zip(got[1:], want[1:]):
