@@ -633,9 +633,8 @@ int svox_calc_corners(const SvoxTreeSpec* tree, const int64_t* indexer, int64_t 
     return check_launch("calc_corners");
 }
 
-// Can a ray batch be rendered with notes (kForwardNoted / kBackwardNoted)?  The octree kernels, a forward
-// pass whose threshold does not admit leaves the backward pass ignores, no weight accumulator, and a
-// workspace with a chunk for every ray.
+// The forward pass of a training step: the picture of svox_volume_render, and in the workspace the notes
+// svox_volume_render_backward_noted works from (where noted_ok() allows; else the plain forward pass).
 int svox_volume_render_noted(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
                              void* out, void* workspace, int64_t workspace_bytes, void* stream) {
     int od;
