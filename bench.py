@@ -257,6 +257,28 @@ def main():
             "positive_per_ray": round(train_stats["samples_bwd_pos"] / B, 2),
         }
         tree.data.grad = None
+        # the squared-error step on the same rays: colour, gradient and Hessian diagonal in one call
+        target = torch.rand(B, 3, generator=g).to(dev)
+
+        def se_step(workspace):
+            C.se_grad(spec, rspec, target, opt, workspace=workspace)
+
+        se_ms = {}
+        for workspace in (True, False):
+            for _ in range(args.warmup):
+                se_step(workspace)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                se_step(workspace)
+            torch.cuda.synchronize()
+            se_ms[workspace] = (time.perf_counter() - t0) * 1e3 / args.steps
+        fwd_bwd["se_grad"] = {
+            "ms": round(se_ms[True], 3), "mrays_s": round(B / (se_ms[True] * 1e-3) / 1e6, 1),
+            "ms_marching_twice": round(se_ms[False], 3),
+            "includes": "zero-fill of gradient and Hessian diagonal (2 x data); one march that takes notes, "
+                        "then residual, gradient and Hessian from the notes"}
+        del target
         log(f"[bench] fwd+bwd {fwd_bwd}")
 
     # ---------------------------------------------------------------- point queries (dense 128^3 SH9 tree)
