@@ -177,3 +177,46 @@ def test_se_grad_argument_checks(gpu):
     colour, grad, hess = r.se_grad(svox.Rays(dev_rays.origins[:0], dev_rays.dirs[:0], dev_rays.viewdirs[:0]),
                                    torch.zeros(0, 3, device=gpu))
     assert colour.shape == (0, 3) and not grad.any().item() and not hess.any().item()
+
+
+def test_se_grad_ws_argument_handling(gpu):
+    """svox_se_grad_ws / svox_se_grad_image_ws through the C ABI: a negative workspace size is an error;
+    without a workspace, or with one too small to hold a chunk per ray, the call is the plain one."""
+    import ctypes
+    from svox_amd.csrc import _abi
+    tree = synth.shell_tree(depth=5, n_spheres=4, data_format="SH4", seed=2, sigma_range=(2.0, 20.0)).to(gpu)
+    n = 700
+    rays = synth.sphere_rays(n, seed=1)
+    dev_rays = rays_spec(rays, gpu)
+    opt = options(tree, step_size=1e-3)
+    ref = torch.rand(n, 3, generator=torch.Generator().manual_seed(3)).to(gpu)
+    want = C.se_grad(tree._spec(), dev_rays, ref, opt, workspace=False)
+    lib = _abi.load_library()
+    spec = C._pack_tree(tree._spec())
+    rs = C._pack_rays(dev_rays, torch.float32)
+    copt = opt._pack()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    colour = torch.empty(n, 3, device=gpu)
+    grad = torch.empty_like(tree.data)
+    hess = torch.empty_like(tree.data)
+    small = torch.empty(n * 384 // 8, dtype=torch.float64, device=gpu)     # no room for bitmap and bookkeeping
+
+    def call(ws, nbytes):
+        return lib.svox_se_grad_ws(ctypes.byref(spec), ctypes.byref(rs), ctypes.byref(copt), ref.data_ptr(),
+                                   colour.data_ptr(), grad.data_ptr(), hess.data_ptr(), ws, nbytes, stream)
+
+    assert call(None, -1) < 0 and b"negative" in lib.svox_last_error()
+    for ws, nbytes in ((None, 0), (small.data_ptr(), small.numel() * 8)):
+        colour.fill_(-1.0)
+        assert call(ws, nbytes) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(colour, want[0])
+        for g, w in ((grad, want[1]), (hess, want[2])):
+            err, ok = grad_close(g.cpu().numpy(), w.cpu().numpy())
+            assert ok, err
+    cam = C._pack_camera(cam_spec(synth.orbit_poses(1, seed=4, radius=2.5)[0].to(gpu), 40, 30, 35.0), torch.float32)
+    img_ref = torch.rand(30, 40, 3, device=gpu)
+    img = torch.empty(30, 40, 3, device=gpu)
+    rc = lib.svox_se_grad_image_ws(ctypes.byref(spec), ctypes.byref(cam), ctypes.byref(copt), img_ref.data_ptr(),
+                                   img.data_ptr(), grad.data_ptr(), hess.data_ptr(), None, -8, stream)
+    assert rc < 0 and b"negative" in lib.svox_last_error()
