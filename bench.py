@@ -131,14 +131,30 @@ def main():
     fwd_mrays = n_rays_step / (fwd_ms * 1e-3) / 1e6
     per_call_ms = timed(forward_step_per_call)
 
-    # launch duration of the dominant kernel with events on the launching stream
+    # Launch duration of the dominant kernel with events on the launching stream.  A launch of this
+    # size marks the empty leaves first (C._marks_for_this_call: a small kernel of its own, inside
+    # `value`'s timed region); the render launch is timed here alone, with such marks already made.
+    marked_spec = tree._spec()
+    marks = C._marks_for_this_call(marked_spec, opt, n_rays_step)
+    marked_spec.child_marks = marks
+    cam_all = _make_camera_spec(pose_stack, W, H, fx, fx)
     events = []
     for _ in range(max(3, args.steps)):
-        forward_step(events)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        C.volume_render_images(marked_spec, cam_all, opt)
+        b.record()
+        events.append((a, b))
     torch.cuda.synchronize()
     durs = np.array([a.elapsed_time(b) for (a, b) in events])  # ms
-    launch_bytes = np.array([float(sum(fwd_bytes))])
+    if marks is not None:
+        # the density of a leaf marked empty is not read: 4 bytes are counted for it only where the leaf is shaded
+        launch_bytes = np.array([float(sum(W * H * 12 + st["samples"] * 4 + st["samples_shaded"] * 4 * K
+                                           for st in pose_stats))])
+    else:
+        launch_bytes = np.array([float(sum(fwd_bytes))])
     achieved = launch_bytes.mean() / (durs.mean() * 1e-3) / 1e9
+    del marked_spec, marks
 
     # copy ceiling of this device (read + write of 1 GiB)
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev)
@@ -170,6 +186,8 @@ def main():
         "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": traffic,
         "algorithmic_bytes_per_launch": int(launch_bytes.mean()),
         "avg_launch_ms": round(float(durs.mean()), 4),
+        "empty_leaves_marked_per_call": bool(C.AUTO_MARK_RAYS_PER_CELL is not None
+                                             and n_rays_step >= C.AUTO_MARK_RAYS_PER_CELL * tree.child.numel()),
         "copy_ceiling_gbs": round(copy_gbs, 1),
         "samples_per_ray": round(sum(s["samples"] for s in pose_stats) / n_rays_step, 2),
         "shaded_per_ray": round(sum(s["samples_shaded"] for s in pose_stats) / n_rays_step, 2),
@@ -178,6 +196,39 @@ def main():
                 "ms_per_step": round(per_call_ms, 4),
                 "note": "same step as one render_persp call (one launch) per pose, the reference's calling pattern"}
     log(f"[bench] forward {fwd_ms:.2f} ms/step, {fwd_mrays:.1f} Mrays/s (one call per pose: {per_call}), roofline {roofline}")
+
+    # ---------------------------------------------------------------- the same step with the empty leaves marked
+    # (opt-in, for a tree that is rendered as it is many times: tree.mark_empty_leaves() once, then
+    # the renderer passes through empty leaves without reading their density; pictures are identical)
+    auto_mark = C.AUTO_MARK_RAYS_PER_CELL
+    C.AUTO_MARK_RAYS_PER_CELL = None          # no marks at all: the launch reads the density of every leaf it visits
+    plain_imgs = forward_step()
+    plain_ms = timed(forward_step)
+    C.AUTO_MARK_RAYS_PER_CELL = auto_mark
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    tree.mark_empty_leaves()
+    torch.cuda.synchronize()
+    a.record()
+    tree.mark_empty_leaves()
+    b.record()
+    torch.cuda.synchronize()
+    mark_ms = a.elapsed_time(b)
+    marked_ms = timed(forward_step)
+    marked_equal = bool(torch.equal(forward_step(), plain_imgs))
+    del plain_imgs
+    tree.clear_leaf_marks()
+    # the density of a leaf marked empty is not read: count 4 bytes for it only where the leaf is shaded
+    marked_bytes = sum(W * H * 12 + st["samples"] * 4 + st["samples_shaded"] * 4 * K for st in pose_stats)
+    static_tree = {
+        "value": round(n_rays_step / (marked_ms * 1e-3) / 1e6, 3), "unit": "Mrays/s", "ms_per_step": round(marked_ms, 4),
+        "mark_empty_leaves_ms": round(mark_ms, 4), "pictures_identical": marked_equal,
+        "ms_per_step_without_marks": round(plain_ms, 4),
+        "algorithmic_gbs": round(marked_bytes / (marked_ms * 1e-3) / 1e9, 2),
+        "frac_of_peak": round(marked_bytes / (marked_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 5),
+        "note": "not the headline: N3Tree.mark_empty_leaves() is an explicit call outside the reference's interface, "
+                "made once per version of the tree and not inside the timed region; `value` at the top is the "
+                "stateless path, which makes the marks inside every call of this size"}
+    log(f"[bench] forward with marked empty leaves {static_tree}")
 
     # ---------------------------------------------------------------- forward + backward + SGD
     fwd_bwd = None
@@ -447,6 +498,7 @@ def main():
                    "data_gib": round(data_bytes / 2**30, 3)},
         "roofline": roofline,
         "fwd_per_call": per_call,
+        "fwd_static_tree": static_tree,
         "fwd_bwd": fwd_bwd,
         "query": query,
         "large": large,

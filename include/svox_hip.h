@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define SVOX_ABI_VERSION 1
+#define SVOX_ABI_VERSION 2
 
 typedef enum SvoxStatus {
     SVOX_OK = 0,
@@ -68,6 +68,7 @@ typedef struct SvoxTreeSpec {
     int32_t extra_cols;
     int32_t weight_accum_max;    /* nonzero: max-reduce into weight_accum, zero: sum */
     int32_t dtype;               /* SvoxDType of data/extra_data/offset/scaling/weight_accum */
+    const int32_t* child_marks;  /* optional (NULL: none): what svox_mark_empty_leaves wrote for this tree */
 } SvoxTreeSpec;
 
 /* RaysSpec, svox/csrc/include/data_spec.hpp:51-63 */
@@ -279,6 +280,19 @@ int svox_se_grad_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const Sv
 int svox_se_grad_image_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
                           const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out,
                           void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Marks the empty leaves of a tree for the renderers (no reference counterpart; for trees that are
+ * rendered many times between changes, e.g. when serving views of a finished model).
+ * marks_out (capacity, N, N, N) int32 receives a copy of tree->child in which every leaf cell whose
+ * density is not > 0 holds SVOX_EMPTY_LEAF instead of 0.  Passed as SvoxTreeSpec.child_marks, it lets
+ * the fp32 octree render kernels pass through such leaves without reading their density (a 128-byte
+ * line for 4 bytes, four fifths of the leaves a ray of a sparse scene visits).  Results are bit-identical:
+ * no kernel lets a leaf with sigma <= 0 contribute (the marks are ignored for a negative sigma_thresh,
+ * for fp64 trees, N != 2 and density_softplus).  The marks describe data and child as they were when
+ * the call ran: after any write to the densities or to the structure they must be made again or left
+ * out -- the library cannot tell.  Point queries and svox_calc_corners never use them. */
+#define SVOX_EMPTY_LEAF (-2)
+int svox_mark_empty_leaves(const SvoxTreeSpec* tree, int32_t* marks_out, void* stream);
 
 /* grid_weight_render(data, CameraSpec&, RenderOptions&, offset, scaling) -> {grid_weight, grid_hit};
  * svox.cpp:38-40, 120, rt_kernel.cu:1174-1203 (kernel :898-1003).

@@ -40,6 +40,7 @@ class TreeSpec:
         self.scaling = None
         self._weight_accum = None
         self._weight_accum_max = False
+        self.child_marks = None   # optional: what mark_empty_leaves returned for this tree (no reference counterpart)
 
 
 class CameraSpec:
@@ -167,6 +168,14 @@ def _pack_tree(tree, dtype=None, need_data=True):
     else:
         spec.weight_accum = None
     spec.weight_accum_max = int(bool(tree._weight_accum_max))
+    marks = getattr(tree, "child_marks", None)
+    if marks is not None:
+        _check_input(marks, "child_marks")
+        if marks.dtype != torch.int32 or marks.shape != tree.child.shape:
+            raise RuntimeError("child_marks must be an int32 tensor shaped like child")
+        spec.child_marks = marks.data_ptr()
+    else:
+        spec.child_marks = None
     spec.capacity = int(tree.child.shape[0])
     spec.N = int(tree.child.shape[1])
     spec.data_dim = int(tree.data.shape[4])
@@ -331,6 +340,24 @@ def volume_render_image(tree, cam, opt):
     return out
 
 
+# A launch of volume_render_images with at least this many rays per cell of the tree marks the empty
+# leaves first, for this call only (mark_empty_leaves costs about 24 ps per cell, passing through an
+# empty leaf unread saves about 40 ps per ray on a sparse scene).  None: never.
+AUTO_MARK_RAYS_PER_CELL = 0.7
+
+
+def _marks_for_this_call(tree, opt, n_rays):
+    """Marks of the empty leaves made for one large launch, or None where they would not pay or
+    would not be used (the fp32 octree kernels read them, and only for sigma_thresh >= 0)."""
+    if AUTO_MARK_RAYS_PER_CELL is None or getattr(tree, "child_marks", None) is not None:
+        return None
+    if tree.data.dtype != torch.float32 or tree.child.shape[1] != 2 or opt.density_softplus:
+        return None
+    if not opt.sigma_thresh >= 0 or n_rays < AUTO_MARK_RAYS_PER_CELL * tree.child.numel():
+        return None
+    return mark_empty_leaves(tree)
+
+
 def volume_render_images(tree, cam, opt):
     """(n, H, W, out_dim): n images in one launch; cam.c2w is (n, 3, 4) or (n, 4, 4).
     No counterpart in the reference, whose extension renders one image per call."""
@@ -340,6 +367,9 @@ def volume_render_images(tree, cam, opt):
     od = _render_out_dim(spec, opt)
     out = torch.empty((n, cspec.height, cspec.width, od), dtype=tree.data.dtype, device=tree.data.device)
     copt = opt._pack()
+    marks = _marks_for_this_call(tree, opt, n * cspec.height * cspec.width)
+    if marks is not None:
+        spec.child_marks = marks.data_ptr()
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_images", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
               ctypes.byref(copt), out.data_ptr(), _stream(tree.data.device))
@@ -554,6 +584,19 @@ def se_grad_persp(tree, cam, opt, color, workspace=True):
               color.data_ptr(), result.data_ptr(), grad.data_ptr(), hessdiag.data_ptr(),
               ws.data_ptr() if ws is not None else None, ws_bytes, _stream(tree.data.device))
     return result, grad, hessdiag
+
+
+def mark_empty_leaves(tree):
+    """An int32 tensor shaped like tree.child: child with SVOX_EMPTY_LEAF (-2) in every leaf cell whose
+    density is not > 0 (no reference counterpart).  Set as TreeSpec.child_marks it lets the render
+    operators pass through empty leaves without reading their density; results are bit-identical.
+    It describes the tree as it is now: make it again, or leave it out, after a write to the
+    densities or the structure."""
+    spec = _pack_tree(tree)
+    marks = torch.empty_like(tree.child)
+    with torch.cuda.device(tree.data.device):
+        _call("svox_mark_empty_leaves", ctypes.byref(spec), marks.data_ptr(), _stream(tree.data.device))
+    return marks
 
 
 def grid_weight_render(data, cam, opt, offset, scaling):

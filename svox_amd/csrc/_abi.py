@@ -21,6 +21,9 @@ c_int64 = ctypes.c_int64
 c_float = ctypes.c_float
 
 
+ABI_VERSION = 2   # SVOX_ABI_VERSION of include/svox_hip.h: the struct layouts below
+
+
 class TreeSpecC(ctypes.Structure):
     _fields_ = [
         ("data", c_void_p),
@@ -37,6 +40,7 @@ class TreeSpecC(ctypes.Structure):
         ("extra_cols", c_int32),
         ("weight_accum_max", c_int32),
         ("dtype", c_int32),
+        ("child_marks", c_void_p),
     ]
 
 
@@ -149,6 +153,7 @@ SIGNATURES = {
     "svox_se_grad_image_ws": (
         ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p, c_void_p,
                        c_void_p, c_int64, c_void_p]),
+    "svox_mark_empty_leaves": (ctypes.c_int, [P(TreeSpecC), c_void_p, c_void_p]),
     "svox_grid_weight_render": (
         ctypes.c_int, [c_void_p, c_int32, c_int32, P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p,
                        c_void_p, c_void_p]),
@@ -177,9 +182,14 @@ def load_library(path=None):
             "(run `python -m svox_amd.csrc.build`); there is no CPU fallback")
     lib = ctypes.CDLL(lib_path)
     for name, (restype, argtypes) in SIGNATURES.items():
-        fn = getattr(lib, name)
+        fn = getattr(lib, name, None)
+        if fn is None:
+            raise RuntimeError(f"{lib_path} does not export {name}: it was built from other sources, build it again")
         fn.restype = restype
         fn.argtypes = argtypes
+    if path is None and lib.svox_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{lib_path} has ABI version {lib.svox_abi_version()}, this package expects "
+                           f"{ABI_VERSION}: build it again")
     if path is None:
         _lib = lib
     return lib

@@ -208,6 +208,18 @@ __global__ __launch_bounds__(kQueryThreads) void corners_kernel(const int32_t* _
     out[q * 3 + 2] = res[2];
 }
 
+// The child table with the empty leaves marked: a leaf cell (child == 0) whose density is not > 0
+// receives SVOX_EMPTY_LEAF, every other cell its child entry.  One thread per cell.
+template <typename T>
+__global__ __launch_bounds__(256) void mark_empty_leaves_kernel(const T* __restrict__ data,
+                                                                const int32_t* __restrict__ child, int64_t cells,
+                                                                int K, int32_t* __restrict__ marks) {
+    const int64_t i = blockIdx.x * 256ll + threadIdx.x;
+    if (i >= cells) return;
+    const int32_t c = child[i];
+    marks[i] = c != 0 ? c : (data[i * K + (K - 1)] > T(0) ? 0 : SVOX_EMPTY_LEAF);
+}
+
 // Zero-fill used in place of a memset so that a caller may capture the call in a graph.
 __global__ __launch_bounds__(256) void zero_kernel(uint4* __restrict__ p16, int64_t n16,
                                                    uint32_t* __restrict__ tail, int n_tail) {

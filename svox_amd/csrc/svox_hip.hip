@@ -67,6 +67,7 @@ TreeDev<T> make_tree(const SvoxTreeSpec* t) {
     d.K = t->data_dim;
     d.extra_cols = t->extra_cols;
     d.weight_accum_max = t->weight_accum_max;
+    d.marked = 0;
     return d;
 }
 
@@ -176,6 +177,17 @@ int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
     if (D != 1 && D != 4 && D != 9 && D != 16 && D != 25) return -1;
     if (tree->data_dim != 3 * D + 1 || opt->min_comp != 0 || opt->max_comp != D - 1) return -1;
     return D;
+}
+
+// The tree as the octree march kernels see it: with the caller's marks of the empty leaves in place
+// of the child table where they apply (no leaf with sigma <= 0 may contribute: sigma_thresh >= 0).
+TreeDev<float> march_tree(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
+    TreeDev<float> d = make_tree<float>(tree);
+    if (tree->child_marks && opt->sigma_thresh >= 0.0f) {
+        d.child = tree->child_marks;
+        d.marked = 1;
+    }
+    return d;
 }
 
 // Items (rays) a persistent wavefront owns.  With few rays every wavefront gets one 64-item chunk so
@@ -296,7 +308,7 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
             const Source dealt = dealt_out(src, blocks);
 #define SVOX_LAUNCH_FORWARD(ACCUM, REFILL)                                                                     \
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, ACCUM, REFILL>), dim3(blocks), \
-                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), dealt,   \
+                                               dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt,    \
                                                *opt, (float*)out))
             const bool refill = src.per_wave > kMarchThreads;
             if (tree->weight_accum) {
@@ -376,7 +388,7 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
             }
 #define SVOX_LAUNCH_BACKWARD(REFILL, MODE)                                                                      \
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, REFILL, MODE>), dim3(blocks),  \
-                                               dim3(kMarchThreads), 0, stream, make_tree<float>(tree), dealt,    \
+                                               dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt,     \
                                                *opt, (const float*)grad_out, (float*)grad_data, ws, (float*)out))
             const bool refill = src.per_wave > kMarchThreads;
             if (mode == kBackwardReplay) {
@@ -413,12 +425,12 @@ void launch_se_grad(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
             const Source dealt = only ? src : dealt_out(src, blocks);
             if (src.per_wave > kMarchThreads) {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source, true>), dim3(blocks),
-                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                           dim3(kMarchThreads), 0, stream, march_tree(tree, opt),
                                                            dealt, *opt, (const float*)color_ref, (float*)color_out,
                                                            (float*)grad, (float*)hess, only));
             } else {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((se_grad_kernel<P, Source, false>), dim3(blocks),
-                                                           dim3(kMarchThreads), 0, stream, make_tree<float>(tree),
+                                                           dim3(kMarchThreads), 0, stream, march_tree(tree, opt),
                                                            src, *opt, (const float*)color_ref, (float*)color_out,
                                                            (float*)grad, (float*)hess, only));
             }
@@ -483,12 +495,12 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
     const unsigned blocks = blocks_for(total_items_of(rest), rest.per_wave);
     if (rest.per_wave > kMarchThreads) {
         SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, true, kBackwardPlain>), dim3(blocks),
-                                                   dim3(kMarchThreads), 0, stream, make_tree<float>(tree), rest, *opt,
+                                                   dim3(kMarchThreads), 0, stream, march_tree(tree, opt), rest, *opt,
                                                    (const float*)grad_output, (float*)grad_data_out, only,
                                                    (float*)nullptr));
     } else {
         SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, false, kBackwardPlain>), dim3(blocks),
-                                                   dim3(kMarchThreads), 0, stream, make_tree<float>(tree), rest, *opt,
+                                                   dim3(kMarchThreads), 0, stream, march_tree(tree, opt), rest, *opt,
                                                    (const float*)grad_output, (float*)grad_data_out, only,
                                                    (float*)nullptr));
     }
@@ -933,6 +945,22 @@ int svox_se_grad_image_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, c
     const ImageSource<float> all = image_source<float>(cam, 1, 12);
     return se_grad_from_notes(tree, all, all, &plain, color_ref, color_out, grad_out, hessdiag_out, workspace,
                               workspace_bytes, n_slots, stamp_of_image(tree, cam, 1, &plain), (hipStream_t)stream);
+}
+
+int svox_mark_empty_leaves(const SvoxTreeSpec* tree, int32_t* marks_out, void* stream) {
+    int rc = check_tree(tree, true);
+    if (rc) return rc;
+    if (!marks_out) return fail(SVOX_ERR_NULL_POINTER, "marks_out is NULL");
+    const int64_t cells = tree->capacity * tree->N * tree->N * tree->N;
+    if (cells == 0) return SVOX_OK;
+    const unsigned blocks = blocks_for(cells, 256);
+    if (tree->dtype == SVOX_F32)
+        hipLaunchKernelGGL((mark_empty_leaves_kernel<float>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                           (const float*)tree->data, tree->child, cells, tree->data_dim, marks_out);
+    else
+        hipLaunchKernelGGL((mark_empty_leaves_kernel<double>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                           (const double*)tree->data, tree->child, cells, tree->data_dim, marks_out);
+    return check_launch("mark_empty_leaves");
 }
 
 int svox_grid_weight_render(const void* data, int32_t reso, int32_t dtype, const SvoxCameraSpec* cam,

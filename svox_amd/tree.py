@@ -119,6 +119,7 @@ class N3Tree(nn.Module):
         if not cuda or not self.data.is_cuda:
             _no_fallback("N3Tree.set")
         _C.assign_vertical(self._spec(), indices.contiguous(), values.contiguous())
+        self._leaf_marks = None   # densities may have changed under the marks
 
     def forward(self, indices, cuda=True, want_node_ids=False, world=True):
         """Leaf values at the points `indices` (Q, 3); differentiable w.r.t. `data`.
@@ -624,7 +625,34 @@ class N3Tree(nn.Module):
         spec.scaling = self.invradius if world else None
         spec._weight_accum = getattr(self, "_weight_accum", None)
         spec._weight_accum_max = getattr(self, "_weight_accum_op", None) == "max"
+        if getattr(self, "_leaf_marks", None) is not None:
+            if self._leaf_marks_key == self._marks_key():
+                spec.child_marks = self._leaf_marks
+            else:
+                self._leaf_marks = None      # the tree has changed since: the marks are void
         return spec
+
+    # ------------------------------------------------------------------ marks of the empty leaves
+    def mark_empty_leaves(self):
+        """For a tree that will be rendered many times as it is (beyond the reference): note which
+        leaves have no density, so that the renderers pass through them without reading it.  Renders
+        are bit-identical and faster on sparse scenes.
+
+        The marks describe the tree as it is now.  They are dropped by every method of the tree and
+        its views that writes values or changes the structure, and by in-place torch operations on
+        `tree.data` / `tree.child` (their version counters tell).  A write that bypasses both --
+        `tree.data.data -= ...` as in svox's own toy example -- does not: call `clear_leaf_marks()`
+        (or this method again) after such a write."""
+        self._leaf_marks = None
+        self._leaf_marks = _C.mark_empty_leaves(self._spec())
+        self._leaf_marks_key = self._marks_key()
+        return self
+
+    def clear_leaf_marks(self):
+        self._leaf_marks = None
+
+    def _marks_key(self):
+        return (self._ver, self.data._version, self.child._version, self.data.data_ptr(), self.child.data_ptr())
 
     def _maybe_auto_data_dim(self):
         fmt_dim = self.data_format.data_dim if self.data_format is not None else None
