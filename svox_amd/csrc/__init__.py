@@ -321,6 +321,7 @@ def volume_render(tree, rays, opt):
     od = _render_out_dim(spec, opt)
     out = torch.empty((rspec.n_rays, od), dtype=rays.origins.dtype, device=rays.origins.device)
     copt = opt._pack()
+    marks = _attach_marks(spec, tree, opt, rspec.n_rays)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),
               out.data_ptr(), _stream(tree.data.device))
@@ -340,8 +341,8 @@ def volume_render_image(tree, cam, opt):
     return out
 
 
-# A launch of volume_render_images with at least this many rays per cell of the tree marks the empty
-# leaves first, for this call only (mark_empty_leaves costs about 24 ps per cell, passing through an
+# A render call (forward, noted forward or marching backward) with at least this many rays per cell of
+# the tree marks the empty leaves first, for this call only (mark_empty_leaves costs about 24 ps per cell, passing through an
 # empty leaf unread saves about 40 ps per ray on a sparse scene).  None: never.
 AUTO_MARK_RAYS_PER_CELL = 0.7
 
@@ -358,6 +359,15 @@ def _marks_for_this_call(tree, opt, n_rays):
     return mark_empty_leaves(tree)
 
 
+def _attach_marks(spec, tree, opt, n_rays):
+    """Points the packed `spec` to marks made for this call, where they pay; returns the tensor,
+    which the caller keeps until its launch is queued."""
+    marks = _marks_for_this_call(tree, opt, n_rays)
+    if marks is not None:
+        spec.child_marks = marks.data_ptr()
+    return marks
+
+
 def volume_render_images(tree, cam, opt):
     """(n, H, W, out_dim): n images in one launch; cam.c2w is (n, 3, 4) or (n, 4, 4).
     No counterpart in the reference, whose extension renders one image per call."""
@@ -367,9 +377,7 @@ def volume_render_images(tree, cam, opt):
     od = _render_out_dim(spec, opt)
     out = torch.empty((n, cspec.height, cspec.width, od), dtype=tree.data.dtype, device=tree.data.device)
     copt = opt._pack()
-    marks = _marks_for_this_call(tree, opt, n * cspec.height * cspec.width)
-    if marks is not None:
-        spec.child_marks = marks.data_ptr()
+    marks = _attach_marks(spec, tree, opt, n * cspec.height * cspec.width)  # noqa: F841 (kept alive for the launch)
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_images", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
               ctypes.byref(copt), out.data_ptr(), _stream(tree.data.device))
@@ -386,6 +394,7 @@ def volume_render_images_backward(tree, cam, opt, grad_output, workspace=True):
     grad = torch.empty_like(tree.data)
     copt = opt._pack()
     ws, ws_bytes = _backward_workspace(tree, n * cspec.height * cspec.width) if workspace else (None, 0)
+    marks = _attach_marks(spec, tree, opt, n * cspec.height * cspec.width)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_images_backward_ws", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
               ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
@@ -406,6 +415,7 @@ def volume_render_images_noted(tree, cam, opt):
     out = torch.empty(shape, dtype=tree.data.dtype, device=tree.data.device)
     copt = opt._pack()
     ws, ws_bytes = _backward_workspace(tree, n * cspec.height * cspec.width)
+    marks = _attach_marks(spec, tree, opt, n * cspec.height * cspec.width)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_images_noted", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
               ctypes.byref(copt), out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
@@ -474,6 +484,7 @@ def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
     grad = torch.empty_like(tree.data)
     copt = opt._pack()
     ws, ws_bytes = _backward_workspace(tree, rspec.n_rays) if workspace else (None, 0)
+    marks = _attach_marks(spec, tree, opt, rspec.n_rays)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_backward_ws", ctypes.byref(spec), ctypes.byref(rspec),
               ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
@@ -492,6 +503,7 @@ def volume_render_noted(tree, rays, opt):
     out = torch.empty((rspec.n_rays, od), dtype=rays.origins.dtype, device=rays.origins.device)
     copt = opt._pack()
     ws, ws_bytes = _backward_workspace(tree, rspec.n_rays)
+    marks = _attach_marks(spec, tree, opt, rspec.n_rays)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_noted", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),
               out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, _stream(tree.data.device))
