@@ -407,6 +407,12 @@ def main():
 
         with torch.no_grad():
             l_ms = ev_time(lambda: C.volume_render_images(lspec, lcam, lopt))
+            # (a launch of 3 M rays does not pay for marking 48 M cells; with marks kept on the tree:)
+            lmarked = ltree._spec()
+            lmarked.child_marks = C.mark_empty_leaves(lspec)
+            l_marked_ms = ev_time(lambda: C.volume_render_images(lmarked, lcam, lopt))
+            l_mark_ms = ev_time(lambda: C.mark_empty_leaves(lspec), n=2)
+            del lmarked
             Ql = 1 << 24
             # uniform over the whole tree: world coordinates of this tree span [-1, 1]^3
             lpts = (torch.rand(Ql, 3, generator=torch.Generator().manual_seed(4)) * 2 - 1).to(dev)
@@ -424,7 +430,8 @@ def main():
                         "samples_per_ray": round(sum(st["samples"] for st in lstats) / (4 * LW * LH), 2),
                         "shaded_per_ray": round(sum(st["samples_shaded"] for st in lstats) / (4 * LW * LH), 2),
                         "algorithmic_gbs": round(l_bytes / l_ms / 1e6, 1),
-                        "frac_of_peak": round(l_bytes / l_ms / 1e6 / PEAK_HBM_GBS, 4)},
+                        "frac_of_peak": round(l_bytes / l_ms / 1e6 / PEAK_HBM_GBS, 4),
+                        "ms_with_kept_marks": round(l_marked_ms, 4), "mark_empty_leaves_ms": round(l_mark_ms, 4)},
             "query_vertical": {"mpoints_s": round(Ql / lq_ms / 1e3, 1), "ms": round(lq_ms, 4),
                                "algorithmic_gbs": round(lq_bytes / lq_ms / 1e6, 1),
                                "frac_of_peak": round(lq_bytes / lq_ms / 1e6 / PEAK_HBM_GBS, 4)},
