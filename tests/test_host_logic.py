@@ -261,3 +261,41 @@ def test_gen_grid_centres():
     grid = gen_grid(4)
     assert grid.shape == (4, 4, 4, 3)
     assert torch.allclose(grid[1, 2, 3], torch.tensor([0.375, 0.625, 0.875]))
+
+
+def test_tree_keeps_marks_only_while_it_is_unchanged():
+    """The bookkeeping around N3Tree.mark_empty_leaves() (the marks themselves come from a kernel):
+    _spec() hands the marks on while nothing has changed and drops them after a write through a view,
+    an in-place torch operation, a change of structure or a move; one large call makes its own."""
+    tree = svox.N3Tree(data_format="SH4", init_refine=2)
+
+    def pretend_marked():
+        tree._leaf_marks = torch.zeros_like(tree.child)
+        tree._leaf_marks_key = tree._marks_key()
+
+    assert tree._spec().child_marks is None
+    pretend_marked()
+    assert tree._spec().child_marks is tree._leaf_marks
+    assert tree._spec(world=False).child_marks is tree._leaf_marks
+    tree[0, -1:] = 5.0                      # a view writes through data.data: no version counter moves
+    assert tree._spec().child_marks is None
+    pretend_marked()
+    with torch.no_grad():
+        tree.data.add_(1.0)
+    assert tree._spec().child_marks is None and tree._leaf_marks is None
+    pretend_marked()
+    tree.refine(sel=(torch.tensor([0]), torch.tensor([0]), torch.tensor([0]), torch.tensor([0])))
+    assert tree._spec().child_marks is None
+    pretend_marked()
+    tree.clear_leaf_marks()
+    assert tree._spec().child_marks is None
+    pretend_marked()
+    tree.double()                           # new storage for data
+    assert tree._spec().child_marks is None
+    # the size from which a call marks the leaves for itself
+    spec = tree.float()._spec()
+    opt = svox.VolumeRenderer(tree)._get_options(True)
+    assert C.AUTO_MARK_RAYS_PER_CELL * tree.child.numel() > 10
+    assert C._marks_for_this_call(spec, opt, 10) is None
+    spec.child_marks = torch.zeros_like(tree.child)
+    assert C._marks_for_this_call(spec, opt, 10 ** 9) is None       # the caller brought marks
