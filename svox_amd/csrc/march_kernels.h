@@ -306,7 +306,7 @@ __device__ __forceinline__ void walk_turn_flat(const TreeDev<float>& tr, RayStat
 #pragma unroll
     for (int j = 0; j < 3; ++j) pc[j] = clamp01(fma_(r.t, r.d[j], r.o[j]));
     int32_t leaf = cur.seek_flat<kSeekBudget>(go, tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]),
-                                              cell_coord(pc[1]), cell_coord(pc[2]), tr.marked != 0);
+                                              cell_coord(pc[1]), cell_coord(pc[2]));
     // 2^levels and 2^-levels: dividing by the power of two is the multiplication by its reciprocal
     const float cube = __uint_as_float((uint32_t)(127 + cur.levels) << 23);
     float inv_cube = __uint_as_float((uint32_t)(127 - cur.levels) << 23);
@@ -321,8 +321,7 @@ __device__ __forceinline__ void walk_turn_flat(const TreeDev<float>& tr, RayStat
             int levels_f;
 #pragma unroll
             for (int j = 0; j < 3; ++j) local[j] = pc[j];
-            leaf = (int32_t)descend_generic<float>(tr.child, tr.capacity, 2, local, &cube_f, &levels_f,
-                                                   tr.marked != 0);
+            leaf = (int32_t)descend_generic<float>(tr.child, tr.capacity, 2, local, &cube_f, &levels_f, true);
             inv_cube = 1.0f / cube_f;
             broken = broken || leaf < 0;
         }

@@ -67,7 +67,6 @@ TreeDev<T> make_tree(const SvoxTreeSpec* t) {
     d.K = t->data_dim;
     d.extra_cols = t->extra_cols;
     d.weight_accum_max = t->weight_accum_max;
-    d.marked = 0;
     return d;
 }
 
@@ -183,10 +182,7 @@ int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
 // of the child table where they apply (no leaf with sigma <= 0 may contribute: sigma_thresh >= 0).
 TreeDev<float> march_tree(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
     TreeDev<float> d = make_tree<float>(tree);
-    if (tree->child_marks && opt->sigma_thresh >= 0.0f) {
-        d.child = tree->child_marks;
-        d.marked = 1;
-    }
+    if (tree->child_marks && opt->sigma_thresh >= 0.0f) d.child = tree->child_marks;
     return d;
 }
 

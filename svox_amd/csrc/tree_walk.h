@@ -39,12 +39,12 @@ struct TreeDev {
     int32_t K;
     int32_t extra_cols;
     int32_t weight_accum_max;
-    // nonzero: `child` is the copy svox_mark_empty_leaves made -- a negative entry is a leaf whose
-    // density is not > 0 (only the octree march kernels are given such a copy)
-    int32_t marked;
 };
 
-// set in the leaf id a marked walk returns for an empty leaf (octree leaf ids stay below 2^30)
+// The octree march kernels may be given, in place of the child table, the copy svox_mark_empty_leaves
+// made of it, in which a negative entry is a leaf whose density is not > 0.  Their walk reads every
+// negative entry so (the child table of a well-formed tree has none on a cell that can be reached)
+// and sets this bit in the leaf id it returns for such a leaf (octree leaf ids stay below 2^30).
 constexpr int32_t kEmptyLeafBit = 1 << 30;
 
 template <typename T>
@@ -225,7 +225,7 @@ struct OctreeCursor {
     // condition.  `go`: this lane searches; a lane that does not keeps its state and returns kIdle.
     template <int kBudget>
     __device__ __forceinline__ int32_t seek_flat(bool go, const int32_t* __restrict__ child, int32_t last_node,
-                                                 uint32_t nx, uint32_t ny, uint32_t nz, bool marked) {
+                                                 uint32_t nx, uint32_t ny, uint32_t nz) {
         const bool pending = pend_level > 0;
         const bool have = levels > 0;
         const uint32_t diff = (ix ^ nx) | (iy ^ ny) | (iz ^ nz);
@@ -249,14 +249,14 @@ struct OctreeCursor {
                 cell = (node << 3) | cell_at(nx, ny, nz, level);
                 skip = *(const int32_t*)((const char*)child + ((uint32_t)cell << 2));
             }
-            want = want && skip != 0 && !(marked && skip < 0) && level != kCoordBits;
+            want = want && skip > 0 && level != kCoordBits;
             node = want ? (int32_t)min((uint32_t)(node + skip), (uint32_t)last_node) : node;
             level = want ? level + 1 : level;
         }
         // want: the budget ran out; skip == 0: found; else more levels than the coordinates hold
-        const bool empty = marked && skip < 0;   // a leaf marked empty
-        const bool found = search && (skip == 0 || empty);
-        const bool open = search && !(skip == 0 || empty);
+        const bool empty = skip < 0;   // a leaf marked empty
+        const bool found = search && skip <= 0;
+        const bool open = search && skip > 0;
         pend_level = go ? (want ? level : 0) : pend_level;
         pend_node = want ? node : pend_node;
         levels = found ? level : (open ? 0 : levels);
