@@ -202,6 +202,22 @@ int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec*
                                    void* grad_data_out, int32_t accumulate, void* workspace,
                                    int64_t workspace_bytes, void* stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): svox_volume_render_backward_ws
+ * whose workspace is a fixed array inside the library (SVOX_STATIC_WORKSPACE_BYTES of device memory per
+ * GPU the library runs on, held until the process ends) instead of a caller's buffer.  The call
+ * allocates and frees nothing.  At most SVOX_STATIC_RAYS_MAX rays per call: more is SVOX_ERR_BAD_SHAPE
+ * (split the batch and pass accumulate = 1 from the second part on).  The array holds 30 noted leaves
+ * per ray at the maximum ray count and more per ray for smaller batches; rays whose notes do not fit
+ * are marched twice, as by svox_volume_render_backward.  Same gradient as svox_volume_render_backward_ws.
+ * All calls on one GPU share that GPU's array: two such calls that overlap in time on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered and safe. */
+#define SVOX_STATIC_RAYS_MAX 65536
+#define SVOX_STATIC_WORKSPACE_BYTES (65536LL * 768 + 8192 + 256)
+int svox_volume_render_backward_static(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                                       const SvoxRenderOptions* opt, const void* grad_output,
+                                       void* grad_data_out, int32_t accumulate, void* stream);
+
 /* No counterpart in the reference: the pair a training step calls instead of svox_volume_render and
  * svox_volume_render_backward when it runs both on the same rays (what an autograd function keeps
  * between its forward and its backward).  svox_volume_render_noted gives the output of

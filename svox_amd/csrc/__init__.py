@@ -492,6 +492,26 @@ def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
     return grad
 
 
+def volume_render_backward_static(tree, rays, opt, grad_output, grad_data_out, accumulate=False):
+    """volume_render_backward into the caller's `grad_data_out` (shaped like tree.data) with the
+    library's own fixed workspace: nothing is allocated on the way, by torch or by the library, so the
+    call can be recorded into a HIP graph.  At most _abi.STATIC_RAYS_MAX rays per call.  Calls that
+    overlap in time on one GPU race on the shared workspace.  No counterpart in the reference."""
+    spec = _pack_tree(tree)
+    rspec = _pack_rays(rays, tree.data.dtype)
+    od = _render_out_dim(spec, opt)
+    _check_grad(grad_output, (rspec.n_rays, od), tree.data.dtype)
+    _check_input(grad_data_out, "grad_data_out")
+    _same_dtype(grad_data_out, tree.data.dtype, "grad_data_out")
+    if tuple(grad_data_out.shape) != tuple(tree.data.shape):
+        raise RuntimeError("grad_data_out must have the shape of tree.data")
+    copt = opt._pack()
+    with torch.cuda.device(tree.data.device):
+        _call("svox_volume_render_backward_static", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),
+              grad_output.data_ptr(), grad_data_out.data_ptr(), int(bool(accumulate)), _stream(tree.data.device))
+    return grad_data_out
+
+
 def volume_render_noted(tree, rays, opt):
     """(out, notes): volume_render, which in the same march leaves in `notes` (a workspace tensor, or
     None where the library cannot take notes) what volume_render_backward_noted needs of the rays.

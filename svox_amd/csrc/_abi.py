@@ -14,6 +14,7 @@ SVOX_F32, SVOX_F64 = 0, 1
 FORMAT_RGBA, FORMAT_SH, FORMAT_SG, FORMAT_ASG = 0, 1, 2, 3
 MAX_BASIS_DIM = 25
 MAX_OUT_DIM = 16
+STATIC_RAYS_MAX = 65536   # SVOX_STATIC_RAYS_MAX
 
 c_void_p = ctypes.c_void_p
 c_int32 = ctypes.c_int32
@@ -124,6 +125,8 @@ SIGNATURES = {
     "svox_volume_render_backward_ws": (
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int32, c_void_p, c_int64,
                        c_void_p]),
+    "svox_volume_render_backward_static": (
+        ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int32, c_void_p]),
     "svox_volume_render_backward_workspace_bytes": (c_int64, [c_int64, c_int32]),
     "svox_volume_render_noted": (
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int64, c_void_p]),

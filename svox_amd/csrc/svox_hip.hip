@@ -13,6 +13,14 @@
 #include "march_kernels.h"
 #include "query_kernels.h"
 
+#include <mutex>
+
+// Workspace of svox_volume_render_backward_static: one array per GPU, inside the library's code object.
+// In host code the name `scratch` is only a handle for hipGetSymbolAddress (static_workspace below); it
+// is never passed to a kernel or a runtime call as an address.
+static_assert(SVOX_STATIC_WORKSPACE_BYTES % 256 == 0, "whole 256-byte units");
+static __device__ __align__(256) unsigned char scratch[SVOX_STATIC_WORKSPACE_BYTES];
+
 namespace {
 
 using namespace svox;
@@ -401,6 +409,30 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
     hipLaunchKernelGGL((render_backward_generic_kernel<T, Source>), dim3(blocks_for(items, kMarchThreads)),
                        dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (const T*)grad_out,
                        (T*)grad_data);
+}
+
+// The device address of `scratch` on the current device, looked up once per device (every GPU holds
+// its own copy of the array at its own address).
+constexpr int kStaticDevicesMax = 64;
+int static_workspace(void** out) {
+    static std::mutex guard;
+    static void* address[kStaticDevicesMax] = {nullptr};
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess || device < 0 || device >= kStaticDevicesMax)
+        return fail(SVOX_ERR_NO_DEVICE, "svox.volume_render_backward_static: no usable current device (%s)",
+                    err != hipSuccess ? hipGetErrorString(err) : "device index out of range");
+    std::lock_guard<std::mutex> lock(guard);
+    if (!address[device]) {
+        void* ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !ptr)
+            return fail(SVOX_ERR_LAUNCH, "svox.volume_render_backward_static: hipGetSymbolAddress failed (%s)",
+                        hipGetErrorString(err));
+        address[device] = ptr;
+    }
+    *out = address[device];
+    return SVOX_OK;
 }
 
 int64_t data_bytes(const SvoxTreeSpec* t) {
@@ -814,6 +846,27 @@ int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec*
         launch_backward<BatchSource<double>, double>(tree, batch_source<double>(rays, true), opt, od, grad_output,
                                                      grad_data_out, nullptr, 0, 0, (hipStream_t)stream);
     return check_launch("volume_render_backward");
+}
+
+// svox_volume_render_backward_ws on the library's own array: no allocation anywhere on the way (the
+// stock counter in the array's tail is cleared by the fill kernel of launch_backward before every
+// launch; everything else in the array is written before it is read within the launch).
+int svox_volume_render_backward_static(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
+                                       const SvoxRenderOptions* opt, const void* grad_output, void* grad_data_out,
+                                       int32_t accumulate, void* stream) {
+    int rc = check_rays(rays);
+    if (rc) return rc;
+    if (rays->n_rays > SVOX_STATIC_RAYS_MAX)
+        return fail(SVOX_ERR_BAD_SHAPE,
+                    "svox.volume_render_backward_static: %lld rays exceed the %d rays the library's fixed "
+                    "workspace serves per call; split the batch (accumulate = 1 from the second part on) or "
+                    "call svox_volume_render_backward_ws with a workspace of your own",
+                    (long long)rays->n_rays, (int)SVOX_STATIC_RAYS_MAX);
+    void* ws = nullptr;
+    rc = static_workspace(&ws);
+    if (rc) return rc;
+    return svox_volume_render_backward_ws(tree, rays, opt, grad_output, grad_data_out, accumulate, ws,
+                                          (int64_t)SVOX_STATIC_WORKSPACE_BYTES, stream);
 }
 
 int svox_volume_render_images_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, int32_t n_images,
