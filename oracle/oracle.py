@@ -51,10 +51,14 @@ def lib():
             "oracle_calc_corners": (ctypes.c_int, [T, c_void_p, c_int64, c_void_p]),
             "oracle_volume_render": (ctypes.c_int, [T, R, O, c_void_p, S, c_int32]),
             "oracle_volume_render_image": (ctypes.c_int, [T, C, O, c_void_p, S, c_int32]),
-            "oracle_volume_render_backward": (ctypes.c_int, [T, R, O, c_void_p, c_void_p, c_int32, S, c_int32]),
-            "oracle_volume_render_image_backward": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_int32, S, c_int32]),
-            "oracle_se_grad": (ctypes.c_int, [T, R, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int32]),
-            "oracle_se_grad_image": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int32]),
+            "oracle_volume_render_backward": (ctypes.c_int, [T, R, O, c_void_p, c_void_p, c_int32, S, c_int32, c_int32,
+                                                             c_void_p]),
+            "oracle_volume_render_image_backward": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_int32, S, c_int32,
+                                                                   c_int32, c_void_p]),
+            "oracle_se_grad": (ctypes.c_int, [T, R, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p,
+                                              c_void_p]),
+            "oracle_se_grad_image": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+                                                    c_void_p, c_void_p]),
             "oracle_grid_weight_render": (ctypes.c_int, [c_void_p, c_int32, c_int32, C, O, c_void_p, c_void_p, c_void_p,
                                                          c_void_p]),
             "oracle_image_rays": (ctypes.c_int, [T, C, O, c_void_p, c_void_p, c_void_p]),
@@ -234,35 +238,51 @@ def volume_render_image(tree, c2w, fx, fy, width, height, opt, want_stats=False,
     return (out, st.as_dict()) if want_stats else out
 
 
-def volume_render_backward(tree, origins, dirs, vdirs, opt, grad_output, want_stats=False, n_threads=1):
+def volume_render_backward(tree, origins, dirs, vdirs, opt, grad_output, want_stats=False, n_threads=1,
+                           exact_sum=True, want_slack=False):
+    """d(data) of the reference's backward kernel.  exact_sum (the default of every gradient function
+    here): the terms (formed in the tree's scalar type, as the reference forms them) are added in
+    float64 and rounded once -- the sum every floating-point order of the reference's atomics
+    approximates, independent of ray order and thread count.  exact_sum=False adds them in the
+    tree's scalar type in ray order (thread-dependent with n_threads > 1).
+    want_slack (with exact_sum): also returns, shaped like the gradient, how far a sum of an element's
+    n terms in the tree's scalar type may stray from the exact sum in any order:
+    sqrt(n) * unit roundoff * sum |term| (what "up to the order of the atomics" amounts to)."""
     keep, r = _rays(tree, origins, dirs, vdirs)
     o = _opt(opt)
     go = _np(grad_output, tree.dtype)
     grad = np.empty_like(tree.data)
+    slack = np.zeros_like(tree.data) if want_slack and exact_sum else None
     st = _abi.MarchStatsC()
     s = tree.spec()
     _check(lib().oracle_volume_render_backward(ctypes.byref(s), ctypes.byref(r), ctypes.byref(o), _ptr(go),
-                                               _ptr(grad), 0, ctypes.byref(st), n_threads),
+                                               _ptr(grad), 0, ctypes.byref(st), n_threads, int(exact_sum),
+                                               _ptr(slack) if slack is not None else None),
            "volume_render_backward")
-    return (grad, st.as_dict()) if want_stats else grad
+    res = (grad, slack) if want_slack else grad
+    return (res, st.as_dict()) if want_stats else res
 
 
 def volume_render_image_backward(tree, c2w, fx, fy, width, height, opt, grad_output, want_stats=False,
-                                 n_threads=1):
+                                 n_threads=1, exact_sum=True, want_slack=False):
     keep, c = _cam(tree, c2w, fx, fy, width, height)
     o = _opt(opt)
     go = _np(grad_output, tree.dtype)
     grad = np.empty_like(tree.data)
+    slack = np.zeros_like(tree.data) if want_slack and exact_sum else None
     st = _abi.MarchStatsC()
     s = tree.spec()
     _check(lib().oracle_volume_render_image_backward(ctypes.byref(s), ctypes.byref(c), ctypes.byref(o),
-                                                     _ptr(go), _ptr(grad), 0, ctypes.byref(st), n_threads),
+                                                     _ptr(go), _ptr(grad), 0, ctypes.byref(st), n_threads,
+                                                     int(exact_sum), _ptr(slack) if slack is not None else None),
            "volume_render_image_backward")
-    return (grad, st.as_dict()) if want_stats else grad
+    res = (grad, slack) if want_slack else grad
+    return (res, st.as_dict()) if want_stats else res
 
 
-def se_grad(tree, origins, dirs, vdirs, colors, opt, n_threads=1):
-    """(colour (B, C), grad, hessdiag) of 0.5 * |render - colors|^2; grad and hessdiag shaped like tree.data."""
+def se_grad(tree, origins, dirs, vdirs, colors, opt, n_threads=1, exact_sum=True, want_slack=False):
+    """(colour (B, C), grad, hessdiag) of 0.5 * |render - colors|^2; grad and hessdiag shaped like tree.data.
+    want_slack: two more arrays, the order slack of grad and of hessdiag (see volume_render_backward)."""
     keep, r = _rays(tree, origins, dirs, vdirs)
     o = _opt(opt)
     od = lib().oracle_out_data_dim(o.format, o.basis_dim, tree.data.shape[4])
@@ -270,13 +290,15 @@ def se_grad(tree, origins, dirs, vdirs, colors, opt, n_threads=1):
     assert ref.shape == (r.n_rays, od)
     out = np.empty((r.n_rays, od), dtype=tree.dtype)
     grad, hess = np.empty_like(tree.data), np.empty_like(tree.data)
+    slack = (np.zeros_like(tree.data), np.zeros_like(tree.data)) if want_slack and exact_sum else (None, None)
     s = tree.spec()
     _check(lib().oracle_se_grad(ctypes.byref(s), ctypes.byref(r), ctypes.byref(o), _ptr(ref), _ptr(out), _ptr(grad),
-                                _ptr(hess), n_threads), "se_grad")
-    return out, grad, hess
+                                _ptr(hess), n_threads, int(exact_sum), *[_ptr(x) if x is not None else None for x in slack]),
+           "se_grad")
+    return (out, grad, hess) + (slack if want_slack else ())
 
 
-def se_grad_image(tree, c2w, fx, fy, width, height, colors, opt, n_threads=1):
+def se_grad_image(tree, c2w, fx, fy, width, height, colors, opt, n_threads=1, exact_sum=True, want_slack=False):
     keep, c = _cam(tree, c2w, fx, fy, width, height)
     o = _opt(opt)
     od = lib().oracle_out_data_dim(o.format, o.basis_dim, tree.data.shape[4])
@@ -284,10 +306,12 @@ def se_grad_image(tree, c2w, fx, fy, width, height, colors, opt, n_threads=1):
     assert ref.shape == (height, width, od)
     out = np.empty((height, width, od), dtype=tree.dtype)
     grad, hess = np.empty_like(tree.data), np.empty_like(tree.data)
+    slack = (np.zeros_like(tree.data), np.zeros_like(tree.data)) if want_slack and exact_sum else (None, None)
     s = tree.spec()
     _check(lib().oracle_se_grad_image(ctypes.byref(s), ctypes.byref(c), ctypes.byref(o), _ptr(ref), _ptr(out),
-                                      _ptr(grad), _ptr(hess), n_threads), "se_grad_image")
-    return out, grad, hess
+                                      _ptr(grad), _ptr(hess), n_threads, int(exact_sum),
+                                      *[_ptr(x) if x is not None else None for x in slack]), "se_grad_image")
+    return (out, grad, hess) + (slack if want_slack else ())
 
 
 def grid_weight_render(data, c2w, fx, fy, width, height, opt, offset, scaling):

@@ -17,10 +17,23 @@
 // restated here as oracle_expf (Cody-Waite reduction + degree-5 polynomial, <= 1 ulp, flushed to 0
 // below e^-87) so that the value is a fixed function of its argument on every machine.
 //
+// Sums of gradient terms.  The reference adds every term to d(data) with an fp32 atomicAdd, in an
+// order no two runs share; any fp32 order is within the comparison tolerance only while few terms
+// meet in one element.  The backward and se_grad entry points therefore take `exact_sum`: every
+// term is still formed in the tree's scalar type exactly as the reference forms it, but the terms of
+// one element are added in double (SumBuffer) and rounded once at the end.  That result does not
+// depend on the order of the rays or on the thread count beyond the last bit of the double sum, and
+// it is what any fp32 summation order is an approximation of: the checker for many rays per leaf.
+// With it the adder can report, per element, how far a sum of the same terms in the scalar type may
+// stray from the exact one whatever the order (`slack`): sqrt(n) * u * sum |term| for n terms and
+// unit roundoff u -- every one of the n - 1 additions rounds a partial sum no larger than sum |term|,
+// and the roundings add up like a random walk.  The reference's own atomics are subject to it.
+//
 // Parity pins (which test fixes which function) are listed in tests/ and in oracle/README.md.
 
 #include <cmath>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <vector>
@@ -770,11 +783,78 @@ int render_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCa
     return SVOX_OK;
 }
 
+// Destination of the reference's atomicAdds.  Plain: dst[off] += v in the scalar type, in the order the
+// calls arrive (an OpenMP atomic when several threads add).  Exact: the terms are added in double
+// into a zero-initialised side buffer (untouched pages are never committed) and finish() adds the
+// rounded sums to dst.
+template <typename T>
+struct SumBuffer {
+    T* dst;
+    T* slack;                  // optional output of the exact mode: sqrt(n) * u * sum |term| per element
+    double* wide = nullptr;
+    double* wide_abs = nullptr;
+    uint32_t* terms = nullptr;
+    int64_t n;
+    bool par;
+    SumBuffer(T* dst_, int64_t n_, bool exact, bool par_, T* slack_ = nullptr)
+        : dst(dst_), slack(exact ? slack_ : nullptr), n(n_), par(par_) {
+        if (exact) wide = (double*)std::calloc((size_t)n_, sizeof(double));
+        if (slack) {
+            wide_abs = (double*)std::calloc((size_t)n_, sizeof(double));
+            terms = (uint32_t*)std::calloc((size_t)n_, sizeof(uint32_t));
+        }
+    }
+    SumBuffer(const SumBuffer&) = delete;
+    ~SumBuffer() {
+        std::free(wide);
+        std::free(wide_abs);
+        std::free(terms);
+    }
+    bool failed(bool exact) const { return (exact && !wide) || (slack && (!wide_abs || !terms)); }
+    inline void add(int64_t off, T v) const {
+        if (slack) {
+            const double a = std::fabs((double)v);
+            if (par) {
+#pragma omp atomic
+                wide_abs[off] += a;
+#pragma omp atomic
+                terms[off] += 1u;
+            } else {
+                wide_abs[off] += a;
+                terms[off] += 1u;
+            }
+        }
+        if (wide) {
+            if (par) {
+#pragma omp atomic
+                wide[off] += (double)v;
+            } else {
+                wide[off] += (double)v;
+            }
+        } else if (par) {
+#pragma omp atomic
+            dst[off] += v;
+        } else {
+            dst[off] += v;
+        }
+    }
+    void finish() const {
+        if (!wide) return;
+#pragma omp parallel for schedule(static) if (par)
+        for (int64_t i = 0; i < n; ++i)
+            if (wide[i] != 0.0) dst[i] = (T)((double)dst[i] + wide[i]);
+        if (!slack) return;
+        const double u = 0.5 * (double)std::numeric_limits<T>::epsilon();
+#pragma omp parallel for schedule(static) if (par)
+        for (int64_t i = 0; i < n; ++i) slack[i] = (T)(std::sqrt((double)terms[i]) * u * wide_abs[i]);
+    }
+};
+
 template <typename T>
 int render_backward_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
                          const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
                          const void* grad_out_v, void* grad_data_v, int accumulate,
-                         SvoxMarchStats* stats, int n_threads) {
+                         SvoxMarchStats* stats, int n_threads, int exact_sum, void* slack_v) {
     const TreeView<T> tr = make_view<T>(tree);
     const int od = oracle_out_data_dim(opt->format, opt->basis_dim, tree->data_dim);
     const int64_t n = rays ? rays->n_rays : (int64_t)cam->width * cam->height;
@@ -784,6 +864,8 @@ int render_backward_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
     if (!accumulate) std::memset(grad, 0, sizeof(T) * (size_t)total_elems);
     Counters total;
     const bool par = n_threads > 1;
+    const SumBuffer<T> sum(grad, total_elems, exact_sum != 0, par, (T*)slack_v);
+    if (sum.failed(exact_sum != 0)) return SVOX_ERR_BAD_SHAPE;
 #pragma omp parallel num_threads(n_threads > 0 ? n_threads : 1)
     {
         Counters local;
@@ -794,19 +876,9 @@ int render_backward_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
                 batch_ray(tr, *rays, r, origin, dir, vdir);
             else
                 pixel_ray(tr, *cam, *opt, r, origin, dir, vdir);
-            if (par) {
-                trace_ray_backward(
-                    tr, *opt, origin, dir, vdir, od, grad_out + r * od,
-                    [grad](int64_t off, T v) {
-#pragma omp atomic
-                        grad[off] += v;
-                    },
-                    stats ? &local : nullptr);
-            } else {
-                trace_ray_backward(
-                    tr, *opt, origin, dir, vdir, od, grad_out + r * od,
-                    [grad](int64_t off, T v) { grad[off] += v; }, stats ? &local : nullptr);
-            }
+            trace_ray_backward(
+                tr, *opt, origin, dir, vdir, od, grad_out + r * od,
+                [&sum](int64_t off, T v) { sum.add(off, v); }, stats ? &local : nullptr);
         }
 #pragma omp critical
         {
@@ -814,6 +886,7 @@ int render_backward_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
             total.bwd_pos += local.bwd_pos;
         }
     }
+    sum.finish();
     if (stats) merge(stats, total);
     return SVOX_OK;
 }
@@ -879,7 +952,8 @@ int grid_weight_impl(const void* data_v, int reso, const SvoxCameraSpec* cam,
 template <typename T>
 int se_grad_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCameraSpec* cam,
                  const SvoxRenderOptions* opt, const void* color_ref_v, void* color_out_v,
-                 void* grad_v, void* hess_v, int n_threads) {
+                 void* grad_v, void* hess_v, int n_threads, int exact_sum, void* grad_slack_v,
+                 void* hess_slack_v) {
     const TreeView<T> tr = make_view<T>(tree);
     const int od = oracle_out_data_dim(opt->format, opt->basis_dim, tree->data_dim);
     if (od > 4) return SVOX_ERR_BAD_SHAPE;  // "Tree's output dim cannot be > 4 for se_grad"
@@ -893,6 +967,9 @@ int se_grad_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxC
     std::memset(hess, 0, sizeof(T) * (size_t)total_elems);
     std::memset(out, 0, sizeof(T) * (size_t)(n * od));
     const bool par = n_threads > 1;
+    const SumBuffer<T> grad_sum(grad, total_elems, exact_sum != 0, par, (T*)grad_slack_v),
+        hess_sum(hess, total_elems, exact_sum != 0, par, (T*)hess_slack_v);
+    if (grad_sum.failed(exact_sum != 0) || hess_sum.failed(exact_sum != 0)) return SVOX_ERR_BAD_SHAPE;
 #pragma omp parallel for schedule(dynamic, 256) num_threads(n_threads > 0 ? n_threads : 1)
     for (int64_t r = 0; r < n; ++r) {
         T origin[3], dir[3], vdir[3];
@@ -900,19 +977,12 @@ int se_grad_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxC
             batch_ray(tr, *rays, r, origin, dir, vdir);
         else
             pixel_ray(tr, *cam, *opt, r, origin, dir, vdir);
-        auto add_to = [par](T* dst) {
-            return [dst, par](int64_t off, T v) {
-                if (par) {
-#pragma omp atomic
-                    dst[off] += v;
-                } else {
-                    dst[off] += v;
-                }
-            };
-        };
-        trace_ray_se_grad(tr, *opt, origin, dir, vdir, od, ref + r * od, out + r * od, add_to(grad),
-                          add_to(hess));
+        trace_ray_se_grad(tr, *opt, origin, dir, vdir, od, ref + r * od, out + r * od,
+                          [&grad_sum](int64_t off, T v) { grad_sum.add(off, v); },
+                          [&hess_sum](int64_t off, T v) { hess_sum.add(off, v); });
     }
+    grad_sum.finish();
+    hess_sum.finish();
     return SVOX_OK;
 }
 
@@ -1093,55 +1163,61 @@ int oracle_volume_render_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* c
 int oracle_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
                                   const SvoxRenderOptions* opt, const void* grad_output,
                                   void* grad_data_out, int32_t accumulate, SvoxMarchStats* stats,
-                                  int32_t n_threads) {
+                                  int32_t n_threads, int32_t exact_sum, void* slack_out) {
     const int rc = check_render_args(tree, opt);
     if (rc) return rc;
     if (!rays || !grad_output || !grad_data_out) return SVOX_ERR_NULL_POINTER;
     return tree->dtype == SVOX_F32
                ? render_backward_impl<float>(tree, rays, nullptr, opt, grad_output, grad_data_out,
-                                             accumulate, stats, n_threads)
+                                             accumulate, stats, n_threads, exact_sum, slack_out)
                : render_backward_impl<double>(tree, rays, nullptr, opt, grad_output, grad_data_out,
-                                              accumulate, stats, n_threads);
+                                              accumulate, stats, n_threads, exact_sum, slack_out);
 }
 
 // volume_render_image_backward, rt_kernel.cu:1085-1109
 int oracle_volume_render_image_backward(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
                                         const SvoxRenderOptions* opt, const void* grad_output,
                                         void* grad_data_out, int32_t accumulate,
-                                        SvoxMarchStats* stats, int32_t n_threads) {
+                                        SvoxMarchStats* stats, int32_t n_threads, int32_t exact_sum,
+                                        void* slack_out) {
     const int rc = check_render_args(tree, opt);
     if (rc) return rc;
     if (!cam || !cam->c2w || !grad_output || !grad_data_out) return SVOX_ERR_NULL_POINTER;
     return tree->dtype == SVOX_F32
                ? render_backward_impl<float>(tree, nullptr, cam, opt, grad_output, grad_data_out,
-                                             accumulate, stats, n_threads)
+                                             accumulate, stats, n_threads, exact_sum, slack_out)
                : render_backward_impl<double>(tree, nullptr, cam, opt, grad_output, grad_data_out,
-                                              accumulate, stats, n_threads);
+                                              accumulate, stats, n_threads, exact_sum, slack_out);
 }
 
 // se_grad, rt_kernel.cu:1111-1139: color_ref and color_out are (B, C); grad and hessdiag have the
 // shape of tree.data and are zero-filled here.
 int oracle_se_grad(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt,
                    const void* color_ref, void* color_out, void* grad_out, void* hessdiag_out,
-                   int32_t n_threads) {
+                   int32_t n_threads, int32_t exact_sum, void* grad_slack_out, void* hess_slack_out) {
     const int rc = check_render_args(tree, opt);
     if (rc) return rc;
     if (!rays || !color_ref || !color_out || !grad_out || !hessdiag_out) return SVOX_ERR_NULL_POINTER;
     return tree->dtype == SVOX_F32
-               ? se_grad_impl<float>(tree, rays, nullptr, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads)
-               : se_grad_impl<double>(tree, rays, nullptr, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads);
+               ? se_grad_impl<float>(tree, rays, nullptr, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads, exact_sum,
+                                     grad_slack_out, hess_slack_out)
+               : se_grad_impl<double>(tree, rays, nullptr, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads, exact_sum,
+                                     grad_slack_out, hess_slack_out);
 }
 
 // se_grad_persp, rt_kernel.cu:1141-1173: color_ref and color_out are (H, W, C)
 int oracle_se_grad_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
                          const SvoxRenderOptions* opt, const void* color_ref, void* color_out,
-                         void* grad_out, void* hessdiag_out, int32_t n_threads) {
+                         void* grad_out, void* hessdiag_out, int32_t n_threads, int32_t exact_sum,
+                         void* grad_slack_out, void* hess_slack_out) {
     const int rc = check_render_args(tree, opt);
     if (rc) return rc;
     if (!cam || !cam->c2w || !color_ref || !color_out || !grad_out || !hessdiag_out) return SVOX_ERR_NULL_POINTER;
     return tree->dtype == SVOX_F32
-               ? se_grad_impl<float>(tree, nullptr, cam, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads)
-               : se_grad_impl<double>(tree, nullptr, cam, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads);
+               ? se_grad_impl<float>(tree, nullptr, cam, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads, exact_sum,
+                                     grad_slack_out, hess_slack_out)
+               : se_grad_impl<double>(tree, nullptr, cam, opt, color_ref, color_out, grad_out, hessdiag_out, n_threads, exact_sum,
+                                     grad_slack_out, hess_slack_out);
 }
 
 // grid_weight_render, rt_kernel.cu:1174-1203.  data, grid_weight_out and grid_hit_out are

@@ -881,25 +881,88 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
 // A lane runs its ray twice.  March 1 accumulates <render, grad_out> and writes nothing.  March 2
 // replays the ray and produces, per visited leaf with sigma > 0, the reference's gradient record:
 // basis[i] * tmp2[c] for the colour coefficients and the density term.  The records are not
-// scattered lane by lane: for every queue slot the wavefront walks over the lanes that produced a
-// record, and for each such leaf all lanes add one element each of the K-long record with a single
-// coalesced atomic instruction (element e from lane e).  Lanes whose rays sit in the same leaf are
-// summed first, so that leaf receives one atomic per element instead of one per ray.  The per-term
-// products are the reference's; only the order in which they are added up differs.
+// scattered lane by lane: the records of a round are listed in LDS (RecordList) and added by the
+// whole wavefront, and where several rays of the wavefront sit in the same leaf their records are
+// summed first (group_by_leaf), so that the leaf receives one atomic per element instead of one per
+// ray.  The per-term products are the reference's; only the order in which they are added up differs.
 // Both marches test sigma > 0 and never stop early (rt_kernel.cu:377, 441).
+//
 // Gradient records of a round.  A record is the K-long vector (basis[i] * tmp2[c] for the colour
 // coefficients, g_sigma last) of a lane, to be added at a leaf.  The records of the queue slots are
 // collected in LDS -- in the shade list's storage, which is dead once the colours are evaluated --
-// and added together: the n * K scalars of the list flat, scalar f from lane f mod 64, so that every
-// atomic instruction covers 64 consecutive scalars whatever K is.  The list is flushed when it is
-// full and at the end of the round.
-// Adds the n records of a list, K elements each, with the lanes tied to elements: the list is cut
-// into 64 / K slices of consecutive records and lane l serves element l % K of slice l / K (of every
-// record, in two or more steps, if K > 64).  Which element a lane serves never changes, so an
-// addition costs about half the instructions of running over the flat list; the price is idle lanes
-// where K does not divide 64.  Consecutive records of the same leaf (neighbouring rays of an image)
-// are summed in registers and added once.  term(rec, e, t) gives the NV values of element e of
-// record rec, emit(leaf, e, sum) adds them.
+// and added together.  The list is flushed when it is full and at the end of the round.  Two forms:
+//   flat        the n * K scalars of the list, scalar f from lane f mod 64, so that every atomic
+//               instruction covers 64 consecutive scalars whatever K is;
+//   by record   the lanes tied to elements (add_records_by_leaf): the list is cut into 64 / K slices
+//               of consecutive records and lane l serves element l % K of slice l / K (of every
+//               record, in two or more steps, if K > 64).  Which element a lane serves never changes,
+//               so an addition costs about half the instructions of running over the flat list; the
+//               price is idle lanes where K does not divide 64.  Consecutive records of the same leaf
+//               are summed in registers and added once.  term(rec, e, t) gives the NV values of
+//               element e of record rec, emit(leaf, e, sum) adds them.
+// Before either, group_by_leaf looks for leaves that several records of the list share; if enough do,
+// the list is put in an order that brings the records of a leaf together and added by record.
+
+// Scratch of group_by_leaf, in LDS that is dead while records are added.
+struct GroupScratch {
+    uint8_t table[256];              // hash of a leaf -> some record of the list with that hash
+    uint8_t order[kMarchThreads];    // position in the grouped order -> record
+    int32_t leaf[kMarchThreads];     // position in the grouped order -> its leaf
+};
+// The list is regrouped if at least one record in kMergeMinShare repeats the leaf of another one.
+// Where rays do not share leaves (a shuffled training batch) looking for repeats is pure cost, so a
+// wavefront that found too few looks again only kMergeRecheck flushes later; one that found enough
+// looks at every flush (the look is small beside the regrouping it decides on).
+constexpr int kMergeMinShare = 2;
+constexpr int kMergeRecheck = 8;
+struct MergeState {
+    int skip = 0;   // flushes left before the next look (wavefront-uniform)
+};
+
+// n <= 64 records; record r's leaf is leaves[r] (visible to every lane).  Estimates how many records
+// repeat the leaf of another record: every record writes its number at its leaf's hash, reads the
+// number that stayed there and compares leaves (a record that reads its own number repeats nothing it
+// can see; two leaves with one hash hide each other's repeats, which only makes the estimate low).
+// If they are too few, returns false.  Otherwise fills gs.order / gs.leaf with the records grouped by
+// leaf (groups in the order of their first record, records of a group in list order) and returns true.
+__device__ __forceinline__ bool group_by_leaf(GroupScratch& gs, MergeState& state, const int32_t* leaves, int n,
+                                              int lane) {
+    if (state.skip > 0) {
+        state.skip -= 1;
+        return false;
+    }
+    const bool mine = lane < n;
+    const int32_t leaf = mine ? leaves[lane] : -1;
+    const unsigned h = ((uint32_t)leaf * 2654435761u) >> 24;
+    if (mine) gs.table[h] = (uint8_t)lane;
+    wave_lds_sync();
+    bool repeat = false;
+    if (mine) {
+        const int j = gs.table[h];
+        repeat = j != lane && leaves[j] == leaf;
+    }
+    if (__popcll(__ballot(repeat)) * kMergeMinShare < n) {
+        state.skip = kMergeRecheck;
+        return false;
+    }
+    unsigned long long todo = __ballot(mine);
+    int base = 0, pos = 0;
+    while (todo) {
+        const int lead = __builtin_ctzll(todo);
+        const int32_t l = __builtin_amdgcn_readlane(leaf, lead);
+        const unsigned long long same = __ballot(mine && leaf == l);
+        if ((same >> lane) & 1ull) pos = base + rank_in(same);
+        base += __popcll(same);
+        todo &= ~same;
+    }
+    if (mine) {
+        gs.order[pos] = (uint8_t)lane;
+        gs.leaf[pos] = leaf;
+    }
+    wave_lds_sync();
+    return true;
+}
+
 template <int K, int NV, class Term, class Emit>
 __device__ __forceinline__ void add_records_by_leaf(int n, int lane, const int32_t* leaves, Term&& term,
                                                     Emit&& emit) {
@@ -938,12 +1001,38 @@ struct RecordList {
     ShadeShared<D, true>& sh;
     float* grad_data;
     int lane;
+    MergeState& merge;
     int n = 0;   // wavefront-uniform
 
     __device__ __forceinline__ int32_t* leaves() const { return sh.leaf; }
     __device__ __forceinline__ float* g_sigmas() const { return (float*)(sh.leaf + kEmitCap); }
     __device__ __forceinline__ float* tmp2s() const { return (float*)(sh.leaf + 2 * kEmitCap); }
     __device__ __forceinline__ uint8_t* owners() const { return (uint8_t*)(sh.leaf + 5 * kEmitCap); }
+
+    // element e of record rec: basis[i] * tmp2[c] for a colour coefficient, g_sigma for the density
+    __device__ __forceinline__ float element(int rec, int e) const {
+        const int c = P::kFormat == SVOX_FORMAT_RGBA ? e : e / D;
+        if (c < 3) {
+            const float v = tmp2s()[rec * 3 + c];
+            return P::kFormat == SVOX_FORMAT_RGBA ? v : sh.basis[owners()[rec] * D + (e - c * D)] * v;
+        }
+        return g_sigmas()[rec];
+    }
+
+    // The colours of the round are in registers by the time records are added: their LDS is free.
+    __device__ __forceinline__ GroupScratch& scratch() const { return *(GroupScratch*)sh.colour; }
+
+    // Adds the list with the records of every leaf summed first, if enough records share a leaf.
+    __device__ __forceinline__ bool flush_grouped() {
+        GroupScratch& gs = scratch();
+        if (!group_by_leaf(gs, merge, leaves(), n, lane)) return false;
+        add_records_by_leaf<K, 1>(
+            n, lane, gs.leaf, [&](int at, int e, float* t) { t[0] = element(gs.order[at], e); },
+            [&](int32_t leaf, int e, const float* sum) { atomicAdd(grad_data + (int64_t)leaf * K + e, sum[0]); });
+        wave_lds_sync();
+        n = 0;
+        return true;
+    }
 
     __device__ __forceinline__ void flush() {
         if constexpr (kByRecord) {
@@ -952,6 +1041,7 @@ struct RecordList {
         }
         if (n == 0) return;
         wave_lds_sync();
+        if (flush_grouped()) return;
         const int total = n * K;
         for (int f = lane; f < total; f += kMarchThreads) {
             const int rec = f / K, e = f - rec * K;
@@ -977,17 +1067,9 @@ struct RecordList {
     __device__ __forceinline__ void flush_by_record() {
         if (n == 0) return;
         wave_lds_sync();
+        if (flush_grouped()) return;
         add_records_by_leaf<K, 1>(
-            n, lane, leaves(),
-            [&](int rec, int e, float* t) {
-                const int c = P::kFormat == SVOX_FORMAT_RGBA ? e : e / D;
-                if (c < 3) {
-                    const float v = tmp2s()[rec * 3 + c];
-                    t[0] = P::kFormat == SVOX_FORMAT_RGBA ? v : sh.basis[owners()[rec] * D + (e - c * D)] * v;
-                } else {
-                    t[0] = g_sigmas()[rec];
-                }
-            },
+            n, lane, leaves(), [&](int rec, int e, float* t) { t[0] = element(rec, e); },
             [&](int32_t leaf, int e, const float* sum) { atomicAdd(grad_data + (int64_t)leaf * K + e, sum[0]); });
         wave_lds_sync();
         n = 0;
@@ -1016,6 +1098,8 @@ struct RecordList {
     }
 };
 static_assert(5 * kEmitCap * 4 + kEmitCap <= kQueue * kMarchThreads * 5, "record list exceeds the shade list");
+static_assert(kEmitCap <= kMarchThreads, "group_by_leaf holds one record per lane");
+static_assert(sizeof(GroupScratch) <= sizeof(float) * kQueue * kMarchThreads * 3, "GroupScratch lives in ShadeShared::colour");
 using ShadeSharedProbe = ShadeShared<1, true>;
 static_assert(offsetof(ShadeSharedProbe, who) == sizeof(int32_t) * kQueue * kMarchThreads,
               "the record list runs from ShadeShared::leaf into ShadeShared::who");
@@ -1127,6 +1211,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     float2* rec_first = ws.base;
     float2* rec_chunk = ws.base;
     int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of further chunks (uniform)
+    MergeState merge;
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
@@ -1246,7 +1331,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             if (n_entries > 0) shade_entries<P, true>(tr.data, sh, n_entries, lane);
             wave_lds_sync();
             // ---- composite slot by slot; the gradient records of the round are added together
-            RecordList<P, D> records{sh, grad_data, lane};
+            RecordList<P, D> records{sh, grad_data, lane, merge};
             // what does not depend on the transmittance is evaluated for the four slots side by side
             float q_att[kQueue], q_total[kQueue], q_s[kQueue][3];
 #pragma unroll
@@ -1408,7 +1493,7 @@ constexpr int kReplayGroup = 5;
 static_assert(kChunkRecords % kReplayGroup == 0, "a group of notes never straddles two chunks");
 
 template <class P, class Source>
-__global__ __launch_bounds__(kMarchThreads) void replay_backward_kernel(Source src, SvoxRenderOptions opt,
+__global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3))) void replay_backward_kernel(Source src, SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
                                                                         float* __restrict__ grad_data,
                                                                         ReplaySpace ws) {
@@ -1453,7 +1538,8 @@ __global__ __launch_bounds__(kMarchThreads) void replay_backward_kernel(Source s
     wave_lds_sync();   // the basis rows are read by other lanes when the records are added
 
     float light = 1.0f, accum = 0.0f;
-    RecordList<P, D, true> records{sh, grad_data, lane};
+    MergeState merge{2};   // (a wavefront of 64 unrelated rays flushes about twice: it never looks)
+    RecordList<P, D, true> records{sh, grad_data, lane, merge};
     struct Group {
         float2 note[kReplayGroup][3];
     };
@@ -1894,6 +1980,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
 // notes are incomplete, or every ray if the workspace carries another stamp, is marked in the bitmap
 // for a launch of se_grad_kernel.
 constexpr int kSeRecordCap = 48;
+static_assert(kSeRecordCap <= kMarchThreads, "group_by_leaf holds one record per lane");
 
 template <class P, class Source>
 __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source src, SvoxRenderOptions opt,
@@ -1910,6 +1997,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
     __shared__ int32_t l_leaf[kSeRecordCap];
     __shared__ float l_gs[kSeRecordCap], l_hs[kSeRecordCap], l_gci[kSeRecordCap * 3];
     __shared__ uint8_t l_owner[kSeRecordCap];
+    __shared__ GroupScratch group;
     const int lane = threadIdx.x;
     const int64_t ray = blockIdx.x * (int64_t)kMarchThreads + lane;
     const bool stamped = ws.stamp_at[0] == ws.stamp[0] && ws.stamp_at[1] == ws.stamp[1] &&
@@ -1953,13 +2041,17 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
     }
 
     int n = 0;   // records in the list (wavefront-uniform)
+    MergeState merge{2};
     auto flush = [&]() {
         if (n == 0) return;
         wave_lds_sync();
+        // where enough records share a leaf, the records of a leaf are brought together first
+        const bool grouped = group_by_leaf(group, merge, l_leaf, n, lane);
         add_records_by_leaf<K, 2>(
-            n, lane, l_leaf,
+            n, lane, grouped ? group.leaf : l_leaf,
             // element e of a record: colour coefficient (c, i) or, last, the density
-            [&](int rec, int e, float* t) {
+            [&](int at, int e, float* t) {
+                const int rec = grouped ? group.order[at] : at;
                 const int c = kRgba ? e : e / D;
                 if (c < 3) {
                     const int owner = l_owner[rec];

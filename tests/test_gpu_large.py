@@ -215,8 +215,8 @@ def test_config5_depth10_sh25_ndc_against_the_oracle(gpu, oracle_mod):
     for s in range(0, grad.shape[0], 1 << 19):        # in slices, to bound the temporaries
         a, b = grad[s:s + (1 << 19)], ref_grad[s:s + (1 << 19)]
         worst = max(worst, float(((a - b).abs() / b.abs().clamp_min(floor)).max()))
-    # an OpenMP oracle adds in a thread-dependent order too; both sides are within 1e-4 of the exact sum
-    assert worst <= 2e-4, worst
+    # the oracle's gradient is the exact sum of the fp32 terms (float64 adder), whatever its thread count
+    assert worst <= 1e-4, worst
     del grad, ref_grad
 
     # point queries: values and leaf ids of a million points

@@ -428,6 +428,97 @@ def test_backward_ignores_thresholds_and_misses():
     assert not g_miss.any()
 
 
+def test_exact_sum_mode_is_the_float64_sum_of_the_per_ray_terms():
+    """exact_sum: every ray's terms as the reference forms them (fp32), added in float64, rounded once.
+    Pinned without the oracle's own adder: each ray alone gives at most one term per element, so the
+    per-ray gradients ARE the terms; numpy adds them in float64.  Also: the result does not depend on
+    the order of the rays or the thread count, and the plain fp32 order stays close to it."""
+    tree = synth.dense_tree(2, "SH4", seed=13, sigma="lognormal", coeff_std=0.7)
+    n = 240
+    rays = synth.sphere_rays(n, seed=12)
+    go = torch.randn(n, 3, generator=torch.Generator().manual_seed(5))
+    ref_colour = torch.rand(n, 3, generator=torch.Generator().manual_seed(6))
+    ot = oracle.Tree.from_n3tree(tree)
+    opt = options(tree, step_size=1e-3)
+    o, d, v = rays.origins, rays.dirs, rays.viewdirs
+
+    exact = oracle.volume_render_backward(ot, o, d, v, opt, go, exact_sum=True)
+    _, se_exact, hess_exact = oracle.se_grad(ot, o, d, v, ref_colour, opt, exact_sum=True)
+    wide = np.zeros(tree.data.shape, dtype=np.float64)
+    wide_se = np.zeros_like(wide)
+    wide_hess = np.zeros_like(wide)
+    for r in range(n):
+        sl = slice(r, r + 1)
+        one = oracle.volume_render_backward(ot, o[sl], d[sl], v[sl], opt, go[sl], exact_sum=False)
+        # one ray: exact and plain modes agree to the bit (nothing to reorder)
+        if r < 5:
+            assert np.array_equal(one, oracle.volume_render_backward(ot, o[sl], d[sl], v[sl], opt, go[sl], exact_sum=True))
+        wide += one
+        _, g1, h1 = oracle.se_grad(ot, o[sl], d[sl], v[sl], ref_colour[sl], opt, exact_sum=False)
+        wide_se += g1
+        wide_hess += h1
+    assert np.array_equal(exact, wide.astype(np.float32))
+    # (se_grad adds one term per channel to a density entry, rt_kernel.cu:687-702: a single ray already
+    # sums three of them in fp32 there, so only the colour entries are term-by-term)
+    assert np.array_equal(se_exact[..., :-1], wide_se.astype(np.float32)[..., :-1])
+    assert np.array_equal(hess_exact[..., :-1], wide_hess.astype(np.float32)[..., :-1])
+    assert np.abs(se_exact[..., -1] - wide_se[..., -1]).max() <= 1e-6 * np.abs(wide_se[..., -1]).max()
+    assert np.abs(hess_exact[..., -1] - wide_hess[..., -1]).max() <= 1e-6 * np.abs(wide_hess[..., -1]).max()
+
+    perm = torch.randperm(n, generator=torch.Generator().manual_seed(9))
+    shuffled = oracle.volume_render_backward(ot, o[perm].contiguous(), d[perm].contiguous(), v[perm].contiguous(), opt,
+                                             go[perm].contiguous(), exact_sum=True, n_threads=4)
+    assert np.array_equal(shuffled, exact)
+    shuffled_se = oracle.se_grad(ot, o[perm].contiguous(), d[perm].contiguous(), v[perm].contiguous(),
+                                 ref_colour[perm].contiguous(), opt, exact_sum=True, n_threads=4)
+    assert np.array_equal(shuffled_se[1], se_exact) and np.array_equal(shuffled_se[2], hess_exact)
+
+    plain = oracle.volume_render_backward(ot, o, d, v, opt, go, exact_sum=False)
+    assert not np.array_equal(plain, exact)          # fp32 adds in ray order do round differently ...
+    assert np.abs(plain - exact).max() <= 1e-5 * np.abs(exact).max()    # ... but only in the last bits
+    # the image entry points share the adder
+    c2w = synth.orbit_poses(1, seed=2, radius=2.5)[0]
+    gi = torch.randn(24, 32, 3, generator=torch.Generator().manual_seed(7))
+    a = oracle.volume_render_image_backward(ot, c2w, 30.0, 30.0, 32, 24, opt, gi, exact_sum=True)
+    b = oracle.volume_render_image_backward(ot, c2w, 30.0, 30.0, 32, 24, opt, gi, exact_sum=True, n_threads=3)
+    assert np.array_equal(a, b)
+    plain = oracle.volume_render_image_backward(ot, c2w, 30.0, 30.0, 32, 24, opt, gi, exact_sum=False)
+    assert np.abs(a - plain).max() <= 1e-5 * np.abs(a).max()
+
+
+def test_order_slack_is_what_fp32_sums_in_shuffled_orders_stray_by():
+    """The slack the exact-sum mode reports (sqrt(n) * 2^-24 * sum |term| per element) against what it
+    models: the same fp32 terms added sequentially in fp32, in several ray orders, on a scene where
+    4000 rays pass through a few dozen leaves.  The sums stay within 1.5 slack of the exact sum and
+    reach a good part of it, so GPU tests that allow twice the slack allow the reference's own
+    nondeterminism and little more."""
+    from util import grad_close
+    tree, point = synth.deep_tree(14, data_format="RGBA", seed=14)
+    g = torch.Generator().manual_seed(14)
+    n = 4000
+    origins = point[None] + 2.0 * synth.unit_vectors(n, g)
+    scale = 2.0 ** -torch.randint(1, 30, (n, 1), generator=g).float()
+    dirs = point[None] + (torch.rand(n, 3, generator=g) * 2 - 1) * scale - origins
+    dirs = (dirs / dirs.norm(dim=1, keepdim=True)).contiguous()
+    origins = origins.contiguous()
+    go = torch.randn(n, 3, generator=torch.Generator().manual_seed(1))
+    ot = oracle.Tree.from_n3tree(tree)
+    opt = options(tree, step_size=1e-4)
+    exact, slack = oracle.volume_render_backward(ot, origins, dirs, dirs, opt, go, want_slack=True, n_threads=4)
+    nz = slack > 0
+    assert nz.sum() > 1000
+    worst, relative = [], []
+    for seed in range(4):
+        perm = torch.randperm(n, generator=torch.Generator().manual_seed(seed))
+        plain = oracle.volume_render_backward(ot, origins[perm].contiguous(), dirs[perm].contiguous(),
+                                              dirs[perm].contiguous(), opt, go[perm].contiguous(), exact_sum=False)
+        worst.append(float((np.abs(plain.astype(np.float64) - exact)[nz] / slack[nz]).max()))
+        relative.append(grad_close(plain, exact)[0])
+        assert grad_close(plain, exact, slack=slack)[1]
+    assert 0.3 < max(worst) < 1.5, worst
+    assert max(relative) > 5e-5, relative    # the orders alone use up most of (or more than) a 1e-4 bar here
+
+
 # ------------------------------------------------------------------------------------------
 # camera rays and NDC
 # ------------------------------------------------------------------------------------------

@@ -46,14 +46,27 @@ def rel_err(a, b):
     return float(np.abs(a - b).max() / (denom if denom > 0 else 1.0))
 
 
-def grad_close(got, ref, rel=1e-4):
-    """Element-wise gradient comparison that tolerates atomic summation order: every element must be
-    within rel of the reference relative to the reference's own magnitude or to a floor tied to the
-    largest gradient (sums of many terms of mixed sign cancel)."""
+ORDER_SLACK_FACTOR = 2.0
+
+
+def grad_close(got, ref, rel=1e-4, slack=None):
+    """Element-wise gradient comparison against the oracle's exact sum: every element must be within
+    `rel` of the reference, relative to the reference's own magnitude or, for elements below it, to a
+    floor of 1e-3 of the largest gradient.
+
+    slack (the oracle's want_slack output): what fp32 additions of an element's terms in an arbitrary
+    order can differ from the exact sum by, sqrt(n) * 2^-24 * sum |term|.  Sequential fp32 sums of the
+    same terms in shuffled orders -- what the reference's own atomics produce -- reach 0.5 to 1.05 of
+    it on the many-rays-per-leaf cases of these tests, which is 2e-5 to 1.6e-4 in the relative measure
+    above; ORDER_SLACK_FACTOR times the slack is taken off the difference before it is measured.  One
+    term missing from a leaf that 4000 rays share is still 30 times that allowance."""
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     floor = np.abs(ref).max() * 1e-3
-    err = np.abs(got - ref) / np.maximum(np.abs(ref), floor if floor > 0 else 1.0)
+    diff = np.abs(got - ref)
+    if slack is not None:
+        diff = np.maximum(diff - ORDER_SLACK_FACTOR * np.asarray(slack, dtype=np.float64), 0.0)
+    err = diff / np.maximum(np.abs(ref), floor if floor > 0 else 1.0)
     if os.environ.get("SVOX_TEST_VERBOSE"):
         print(f"[grad_close] worst relative error {float(err.max()):.3e} (limit {rel:.0e})", flush=True)
     return float(err.max()), err.max() <= rel
