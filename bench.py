@@ -373,7 +373,44 @@ def main():
             "calc_corners": {"mleaves_s": round(leaves.shape[0] / c_ms / 1e3, 1), "ms": round(c_ms, 4),
                              "algorithmic_gbs": round(c_bytes / c_ms / 1e6, 1)},
         }
-        del qtree, pts, go, leaves
+        # render_persp of the same dense tree: one 800x800 pose from the radius-4 orbit, thresholds 0
+        # (every ray that hits shades some 57 leaves; the tree and its child table sit in the 256 MB
+        # Infinity Cache, so bytes fetched from HBM are far below the algorithmic ones here)
+        qrend = svox.VolumeRenderer(qtree)
+        qopt = qrend._get_options(False)
+        qcam = _make_camera_spec(poses[0].contiguous(), W, H, fx, fx)
+        qstats = C.volume_render_stats(qspec, qcam, qopt)
+        with torch.no_grad():
+            qr_ms = ev_time(lambda: qrend.render_persp(poses[0], width=W, height=H, fx=fx))
+            qimg = qrend.render_persp(poses[0], width=W, height=H, fx=fx)
+        qgo = (torch.randn(H, W, 3, generator=torch.Generator().manual_seed(5)) * 1e-2).to(dev)
+
+        def dense_train():
+            qtree.data.grad = None
+            qrend.render_persp(poses[0], width=W, height=H, fx=fx).backward(qgo)
+
+        qrb_ms = ev_time(dense_train, n=3)
+        qtree.data.grad = None
+        qr_bytes = forward_bytes(qstats, W * H, Kq, 12)
+        query["render_persp"] = {
+            "workload": f"one {W}x{H} pose of the dense tree, radius-4 orbit, focal {fx:.0f}, thresholds 0",
+            "ms": round(qr_ms, 4), "mrays_s": round(W * H / qr_ms / 1e3, 1),
+            "rays_hit": qstats["rays_hit"], "mrays_hit_s": round(qstats["rays_hit"] / qr_ms / 1e3, 1),
+            "msamples_s": round(qstats["samples"] / qr_ms / 1e3, 1),
+            "samples_per_hit_ray": round(qstats["samples"] / max(qstats["rays_hit"], 1), 1),
+            "shaded_per_hit_ray": round(qstats["samples_shaded"] / max(qstats["rays_hit"], 1), 1),
+            "algorithmic_gbs": round(qr_bytes / qr_ms / 1e6, 1),
+            "frac_of_peak": round(qr_bytes / qr_ms / 1e6 / PEAK_HBM_GBS, 4),
+            "forward_backward_ms": round(qrb_ms, 4),
+        }
+        if not args.no_cpu:
+            from oracle import oracle as _oracle
+            qot = _oracle.Tree.from_n3tree(qtree.cpu())
+            qref = _oracle.volume_render_image(qot, poses[0].cpu(), fx, fx, W, H, qopt,
+                                               n_threads=min(os.cpu_count() or 1, 16))
+            query["render_persp"]["max_abs_err_vs_oracle"] = float(np.abs(qimg.cpu().numpy() - qref).max())
+            del qot, qref
+        del qtree, pts, go, leaves, qimg, qgo
         log(f"[bench] query {query}")
 
     # ---------------------------------------------------------------- depth-10 SH25 tree, NDC camera

@@ -257,3 +257,59 @@ def test_training_step_at_full_size_notes_against_marches(gpu):
     assert marched.abs().max().item() > 0
     err, ok = grad_close(from_notes.cpu().numpy(), marched.cpu().numpy())
     assert ok, err
+
+
+def test_config2_dense128_sh9_query_and_render_against_the_oracle(gpu, oracle_mod):
+    """The dense benchmark configuration at full size: 128^3 leaf grid (2.1 M leaves, 268 MB of SH9
+    records), half of the leaves zeroed.  query_vertical on 4 Mi uniform points (svox_kernel.cu:120-143)
+    and render_persp of one 800x800 image from a radius-4 orbit with thresholds 0 (svox/renderer.py:290-322,
+    rt_kernel.cu:799-819): leaf ids, values, picture and visit counts equal to the oracle's; gradients of
+    the image (marching with and without a workspace, and replayed from the forward pass's notes) within
+    1e-4 relative of the oracle's exact sum.  Every ray that hits shades about 57 leaves, twice what a
+    ray's share of the notes' workspace holds."""
+    tree = synth.dense_tree(6, "SH9", seed=0, sigma="lognormal", coeff_std=0.5, zero_fraction=0.5)
+    assert tree.n_leaves == 128 ** 3
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    dev = tree.to(gpu)
+    threads = min(16, oracle_mod.max_threads())
+
+    Q = 1 << 22
+    pts = torch.rand(Q, 3, generator=torch.Generator().manual_seed(3))
+    ref_vals, ref_ids = oracle_mod.query_vertical(ot, pts)
+    vals, ids = dev(pts.to(gpu), want_node_ids=True)
+    assert np.array_equal(ids.cpu().numpy(), ref_ids)
+    assert np.array_equal(vals.detach().cpu().numpy(), ref_vals)
+    del vals, ids, ref_vals, ref_ids
+
+    W = H = 800
+    fx = 1111.111
+    c2w = synth.orbit_poses(1, seed=1, radius=4.0)[0]
+    r = svox.VolumeRenderer(dev)
+    opt = r._get_options(False)
+    assert opt.sigma_thresh == 0.0 and opt.stop_thresh == 0.0
+    ref, ref_stats = oracle_mod.volume_render_image(ot, c2w, fx, fx, W, H, opt, want_stats=True, n_threads=threads)
+    with torch.no_grad():
+        img = r.render_persp(c2w.to(gpu), width=W, height=H, fx=fx)
+    assert np.array_equal(img.cpu().numpy(), ref)
+    from svox_amd.renderer import _make_camera_spec
+    cam = _make_camera_spec(c2w.to(gpu).contiguous(), W, H, fx, fx)
+    stats = C.volume_render_stats(dev._spec(), cam, opt)
+    for k in ("rays", "rays_hit", "samples", "samples_shaded", "levels"):
+        assert stats[k] == ref_stats[k], k
+    assert stats["rays_hit"] > 100_000 and stats["samples_shaded"] > 50 * stats["rays_hit"]
+
+    go = torch.randn(H, W, 3, generator=torch.Generator().manual_seed(1)) * 1e-2
+    ref_grad = oracle_mod.volume_render_image_backward(ot, c2w, fx, fx, W, H, opt, go, n_threads=threads)
+    spec = dev._spec()
+    for workspace in (True, False):
+        grad = C.volume_render_image_backward(spec, cam, opt, go.to(gpu), workspace=workspace)
+        err, ok = grad_close(grad.cpu().numpy(), ref_grad)
+        assert ok, (workspace, err)
+    del grad
+    # through autograd: the noted forward pass (notes overflow for most rays that hit) and its backward
+    dev.data.grad = None
+    out = r.render_persp(c2w.to(gpu), width=W, height=H, fx=fx)
+    assert np.array_equal(out.detach().cpu().numpy(), ref)
+    out.backward(go.to(gpu))
+    err, ok = grad_close(dev.data.grad.cpu().numpy(), ref_grad)
+    assert ok, ("autograd", err)
