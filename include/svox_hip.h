@@ -226,8 +226,8 @@ int svox_volume_render_backward_static(const SvoxTreeSpec* tree, const SvoxRaysS
  * svox_volume_render_backward_noted, called with the same tree, rays, options and workspace, gives
  * the gradient of svox_volume_render_backward without walking the tree: it replays the notes twice.
  * A ray whose notes did not fit is marched twice as in svox_volume_render_backward; so is every ray
- * if the workspace does not carry the stamp (ray count, tree->data, rays->origins, step size,
- * sigma_thresh) the first call left.  The caller must not change tree->data, the rays or the
+ * if the workspace does not carry the stamp (ray count, tree->data, tree->child, rays->origins,
+ * rays->dirs, step size, sigma_thresh) the first call left.  The caller must not change tree->data, the rays or the
  * workspace between the two calls.  Workspace as for svox_volume_render_backward_ws (same size
  * function).  Where notes cannot be taken (fp64 or generic kernels, a weight accumulator, a negative
  * sigma_thresh, a workspace with fewer than n_rays chunks) the two calls are svox_volume_render and

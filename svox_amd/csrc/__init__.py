@@ -41,6 +41,7 @@ class TreeSpec:
         self._weight_accum = None
         self._weight_accum_max = False
         self.child_marks = None   # optional: what mark_empty_leaves returned for this tree (no reference counterpart)
+        self.owner = None         # optional: the N3Tree this spec was made from (its write counter)
 
 
 class CameraSpec:
@@ -451,23 +452,38 @@ def _check_grad(grad_output, shape, dtype):
         raise RuntimeError(f"grad_output must have shape {tuple(shape)}, got {tuple(grad_output.shape)}")
 
 
-# Leaves per ray (on average) the backward's workspace has room for, and the most memory it may take.
+# Leaves per ray (on average) the backward's workspace has room for, and the most memory it may take:
+# BACKWARD_WORKSPACE_LIMIT bytes, and of what is free on the device at the time (memory torch holds
+# in its cache counted as free) no more than BACKWARD_WORKSPACE_FREE_FRACTION.
 BACKWARD_RECORDS_PER_RAY = 30
 BACKWARD_WORKSPACE_LIMIT = 4 << 30
+BACKWARD_WORKSPACE_FREE_FRACTION = 0.25
+_ASK_DEVICE_ABOVE = 64 << 20   # smaller workspaces are taken without asking the device what is free
 
 
 def _backward_workspace(tree, n_rays):
-    """(tensor, bytes) of the backward's workspace for n_rays rays, or (None, 0)."""
+    """(tensor, bytes) of the backward's workspace for n_rays rays, or (None, 0): for a tree that is
+    not fp32, where the limits leave no room for 15 leaves per ray, and where the allocation fails
+    (the caller then runs without a workspace: same results, more marching)."""
     if n_rays <= 0 or tree.data.dtype != torch.float32:
         return None, 0
     size_of = _abi.load_library().svox_volume_render_backward_workspace_bytes
     per_ray = int(BACKWARD_RECORDS_PER_RAY)
-    while per_ray > 0 and size_of(n_rays, per_ray) > BACKWARD_WORKSPACE_LIMIT:
+    limit = BACKWARD_WORKSPACE_LIMIT
+    if size_of(n_rays, per_ray) > _ASK_DEVICE_ABOVE:
+        device = tree.data.device
+        free, _ = torch.cuda.mem_get_info(device)
+        cached = torch.cuda.memory_reserved(device) - torch.cuda.memory_allocated(device)
+        limit = min(limit, int((free + cached) * BACKWARD_WORKSPACE_FREE_FRACTION))
+    while per_ray > 0 and size_of(n_rays, per_ray) > limit:
         per_ray -= 15
     nbytes = int(size_of(n_rays, per_ray)) if per_ray > 0 else 0
     if nbytes <= 0:
         return None, 0
-    return torch.empty(nbytes // 8, dtype=torch.float64, device=tree.data.device), nbytes
+    try:
+        return torch.empty(nbytes // 8, dtype=torch.float64, device=tree.data.device), nbytes
+    except torch.cuda.OutOfMemoryError:
+        return None, 0
 
 
 def volume_render_backward(tree, rays, opt, grad_output, workspace=True):

@@ -1110,6 +1110,7 @@ static_assert(offsetof(ShadeSharedProbe, who) == sizeof(int32_t) * kQueue * kMar
 // from the rest of the workspace, of which a wavefront takes a stock of 64 chunks at a time through
 // one atomic counter (a heavy image tile needs hundreds, most tiles none); the lanes that need a
 // chunk in the same step are ranked by ballot.
+constexpr int kStampWords = 6;   // ray count; tree data, child; ray origins, directions; step size and threshold
 struct ReplaySpace {
     float2* base;          // chunk c starts at base + c * kChunkFloat2
     int64_t first_shared;  // chunks [0, first_shared) are the rays' first chunks
@@ -1118,13 +1119,21 @@ struct ReplaySpace {
     // kForwardNoted writes `stamp` (what the notes belong to) to stamp_at; replay_backward_kernel uses
     // the notes only if it finds its own stamp there
     unsigned long long* stamp_at;
-    unsigned long long stamp[4];
+    unsigned long long stamp[kStampWords];
     // one bit per ray (ray i: bit i % 64 of word i / 64).  replay_backward_kernel sets the bits of the
     // rays it could not do from their notes; a launch of render_backward_kernel that is given the
     // bitmap as `only` does those rays and no others
     unsigned long long* undone;
     const unsigned long long* only;
 };
+
+// whether the workspace carries the stamp this launch expects
+__device__ __forceinline__ bool stamp_matches(const ReplaySpace& ws) {
+    bool same = true;
+#pragma unroll
+    for (int i = 0; i < kStampWords; ++i) same = same && ws.stamp_at[i] == ws.stamp[i];
+    return same;
+}
 
 // The first ray at or after `next` (a wavefront-uniform ray number below `end`) whose 64-ray word of
 // the bitmap `only` is not zero, found 64 words at a time; a value >= end if there is none.
@@ -1190,7 +1199,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
     if constexpr (kMode == kForwardNoted) {
-        if (blockIdx.x == 0 && lane < 4) ws.stamp_at[lane] = ws.stamp[lane];
+        if (blockIdx.x == 0 && lane < kStampWords) ws.stamp_at[lane] = ws.stamp[lane];
     }
 
     enum { kMarch1 = 0, kMarch2 = 1, kReplaying = 2 };
@@ -1501,8 +1510,7 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
     __shared__ ShadeShared<D, true> sh;
     const int lane = threadIdx.x;
     const int64_t ray = blockIdx.x * (int64_t)kMarchThreads + lane;
-    const bool stamped = ws.stamp_at[0] == ws.stamp[0] && ws.stamp_at[1] == ws.stamp[1] &&
-                         ws.stamp_at[2] == ws.stamp[2] && ws.stamp_at[3] == ws.stamp[3];
+    const bool stamped = stamp_matches(ws);
     const float2* first = ws.base + ray * kChunkFloat2;
     int count = 0;
     int32_t first_link = 0;
@@ -2000,8 +2008,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
     __shared__ GroupScratch group;
     const int lane = threadIdx.x;
     const int64_t ray = blockIdx.x * (int64_t)kMarchThreads + lane;
-    const bool stamped = ws.stamp_at[0] == ws.stamp[0] && ws.stamp_at[1] == ws.stamp[1] &&
-                         ws.stamp_at[2] == ws.stamp[2] && ws.stamp_at[3] == ws.stamp[3];
+    const bool stamped = stamp_matches(ws);
     const float2* first = ws.base + ray * kChunkFloat2;
     int count = 0;
     int32_t first_link = 0;

@@ -335,7 +335,7 @@ constexpr int64_t kChunkBytes = (int64_t)kChunkFloat2 * 8;   // 384: 15 records 
 
 // What the notes in a workspace belong to (ReplaySpace::stamp).
 struct NoteStamp {
-    unsigned long long word[4];
+    unsigned long long word[kStampWords];
 };
 NoteStamp stamp_of(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxRenderOptions* opt) {
     NoteStamp st;
@@ -346,6 +346,8 @@ NoteStamp stamp_of(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const Svo
     st.word[1] = (unsigned long long)(uintptr_t)tree->data;
     st.word[2] = (unsigned long long)(uintptr_t)rays->origins;
     st.word[3] = ((unsigned long long)thresh_bits << 32) | step_bits;
+    st.word[4] = (unsigned long long)(uintptr_t)tree->child;
+    st.word[5] = (unsigned long long)(uintptr_t)rays->dirs;
     return st;
 }
 
@@ -356,7 +358,7 @@ constexpr int64_t kStampOffset = 0;
 constexpr int64_t kStockCounterOffset = 128;
 int64_t bitmap_bytes(int64_t n_slots) { return ((n_slots + 63) / 64 * 8 + 15) / 16 * 16; }
 bool carve_workspace(void* workspace, int64_t workspace_bytes, int64_t n_slots, ReplaySpace* ws) {
-    *ws = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0}, nullptr, nullptr};
+    *ws = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0, 0, 0}, nullptr, nullptr};
     const int64_t chunks = workspace && n_slots > 0
                                ? (workspace_bytes - kTailBytes - bitmap_bytes(n_slots)) / kChunkBytes : 0;
     if (n_slots <= 0 || chunks < n_slots || chunks >= 0x7fffffffll || ((uintptr_t)workspace & 15u) != 0) return false;
@@ -500,6 +502,7 @@ NoteStamp stamp_of_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, in
                                 const SvoxRenderOptions* opt) {
     SvoxRaysSpec as_rays;
     as_rays.origins = cam->c2w;
+    as_rays.dirs = nullptr;
     as_rays.n_rays = ((int64_t)n_images * cam->height * cam->width) ^ ((int64_t)cam->width << 40);
     return stamp_of(tree, &as_rays, opt);
 }
@@ -519,7 +522,7 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
                                                stream, all, *opt, (const float*)grad_output, (float*)grad_data_out, ws));
     int rc = check_launch("volume_render_backward_noted");
     if (rc) return rc;
-    ReplaySpace only = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0}, nullptr, ws.undone};
+    ReplaySpace only = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0, 0, 0}, nullptr, ws.undone};
     const unsigned blocks = blocks_for(total_items_of(rest), rest.per_wave);
     if (rest.per_wave > kMarchThreads) {
         SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, true, kBackwardPlain>), dim3(blocks),

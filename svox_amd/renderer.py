@@ -57,9 +57,9 @@ class _VolumeRenderFunction(torch.autograd.Function):
     def forward(ctx, data, tree, rays, opt, keep_notes=False):
         ctx.tree, ctx.rays, ctx.opt = tree, rays, opt
         ctx.notes = None
+        ctx.versions = _versions(tree, rays)
         if keep_notes:
             out, ctx.notes = _C.volume_render_noted(tree, rays, opt)
-            ctx.versions = _versions(tree, rays)
             return out
         return _C.volume_render(tree, rays, opt)
 
@@ -68,16 +68,28 @@ class _VolumeRenderFunction(torch.autograd.Function):
         if not ctx.needs_input_grad[0]:
             return None, None, None, None, None
         notes, ctx.notes = ctx.notes, None
-        if notes is not None and ctx.versions == _versions(ctx.tree, ctx.rays):
+        if ctx.versions != _versions(ctx.tree, ctx.rays):
+            # the tree or the rays were written to since the forward pass: its notes and the marks of
+            # the empty leaves it ran with describe the old values; march through the tree as it is
+            notes, ctx.tree.child_marks = None, None
+        if notes is not None:
             grad = _C.volume_render_backward_noted(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous(), notes)
         else:
             grad = _C.volume_render_backward(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous())
         return grad, None, None, None, None
 
 
+def _tree_versions(tree):
+    """What tells that a tree was written to: torch's version counters of data and child and, for
+    writes those do not see (kernels of this package, N3TreeView.set, tree.touch()), the write
+    counter of the N3Tree the spec was made from."""
+    owner = getattr(tree, "owner", None)
+    return (tree.data._version, tree.child._version, getattr(owner, "_writes", 0), getattr(owner, "_ver", 0))
+
+
 def _versions(tree, rays):
-    """Version counters of the tensors the notes of a forward pass depend on."""
-    return tuple(t._version for t in (tree.data, tree.child, rays.origins, rays.dirs, rays.vdirs))
+    """Version counters of everything the notes of a forward pass depend on."""
+    return _tree_versions(tree) + tuple(t._version for t in (rays.origins, rays.dirs, rays.vdirs))
 
 
 class _VolumeRenderImageFunction(torch.autograd.Function):
@@ -88,9 +100,9 @@ class _VolumeRenderImageFunction(torch.autograd.Function):
     def forward(ctx, data, tree, cam, opt, keep_notes=False):
         ctx.tree, ctx.cam, ctx.opt = tree, cam, opt
         ctx.notes = None
+        ctx.versions = _image_versions(tree, cam)
         if keep_notes:
             out, ctx.notes = _C.volume_render_images_noted(tree, cam, opt)
-            ctx.versions = _image_versions(tree, cam)
             return out
         return _C.volume_render_image(tree, cam, opt) if cam.c2w.dim() == 2 else _C.volume_render_images(tree, cam, opt)
 
@@ -99,8 +111,8 @@ class _VolumeRenderImageFunction(torch.autograd.Function):
         if not ctx.needs_input_grad[0]:
             return None, None, None, None, None
         notes, ctx.notes = ctx.notes, None
-        if notes is not None and ctx.versions != _image_versions(ctx.tree, ctx.cam):
-            notes = None
+        if ctx.versions != _image_versions(ctx.tree, ctx.cam):
+            notes, ctx.tree.child_marks = None, None     # as in _VolumeRenderFunction.backward
         grad = _C.volume_render_images_backward_noted(ctx.tree, ctx.cam, ctx.opt, grad_out.contiguous(), notes)
         return grad, None, None, None, None
 
@@ -109,7 +121,7 @@ _VolumeRenderImagesFunction = _VolumeRenderImageFunction
 
 
 def _image_versions(tree, cam):
-    return tuple(t._version for t in (tree.data, tree.child, cam.c2w))
+    return _tree_versions(tree) + (cam.c2w._version,)
 
 
 def convert_to_ndc(origins, directions, focal, w, h, near=1.0):
@@ -137,6 +149,27 @@ class VolumeRenderer(nn.Module):
            min_comp > max_comp renders 0.5 grey
     :param density_softplus: apply log(1 + exp(sigma - 1)) to the stored density
     :param rgb_padding: colours become sigmoid * (1 + 2 p) - p
+
+    Memory and state beyond the reference's renderer (which holds nothing between calls):
+
+    * A forward pass that will be differentiated (gradient mode on, `tree.data.requires_grad`) keeps
+      notes of the leaves its rays met until `backward()` has run: 768 bytes per ray (30 leaves per ray
+      on average; 3.9 GB for eight 800x800 images), at most `csrc.BACKWARD_WORKSPACE_LIMIT` (4 GiB) and
+      at most a quarter of the device memory that is free at the time.  Where that leaves no room, or
+      the allocation fails, the pass runs without notes and the backward pass marches through the tree
+      twice, as the reference does: same results, slower.  The noted forward pass follows every ray to
+      its end (no early stop), so it is slower than a forward pass under `torch.no_grad()`.  The notes
+      are used once: a second `backward()` through a retained graph marches.  `renderer.KEEP_NOTES =
+      False` switches the notes off.  If `tree.data`, the tree's structure, the rays or the camera are
+      written to between the two passes -- through torch (version counters), a method of the tree or a
+      view, or `tree.touch()` -- the backward pass drops the notes and any marks of empty leaves and
+      marches through the tree as it then is, which is what the reference's backward pass sees.
+      Only a write through `tree.data.data[...]` that is not followed by `tree.touch()` goes unseen.
+    * A call of `render_persp` on a stack of poses with at least `csrc.AUTO_MARK_RAYS_PER_CELL` (0.7)
+      rays per cell of the tree first marks the empty leaves (one int32 per cell, freed after the
+      call; 25 MB and 0.125 ms for a 512^3 tree of 774 k nodes) so that the march passes through them
+      without reading their density.  Smaller calls do not; `N3Tree.mark_empty_leaves()` keeps marks
+      on the tree for all of them.  Pictures are bit-identical either way.
     """
 
     def __init__(self, tree, step_size=1e-3, background_brightness=1.0, ndc=None, min_comp=0,

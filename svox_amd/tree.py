@@ -119,7 +119,7 @@ class N3Tree(nn.Module):
         if not cuda or not self.data.is_cuda:
             _no_fallback("N3Tree.set")
         _C.assign_vertical(self._spec(), indices.contiguous(), values.contiguous())
-        self._leaf_marks = None   # densities may have changed under the marks
+        self.touch()   # a write torch's version counter of `data` has not seen
 
     def forward(self, indices, cuda=True, want_node_ids=False, world=True):
         """Leaf values at the points `indices` (Q, 3); differentiable w.r.t. `data`.
@@ -610,8 +610,18 @@ class N3Tree(nn.Module):
 
     def _invalidate(self):
         self._ver += 1
+        self._writes = getattr(self, "_writes", 0) + 1
         self._last_all_leaves = None
         self._last_frontier = None
+
+    def touch(self):
+        """Tells the tree that its values were written in a way torch's version counters do not see
+        (a kernel of this package, or `tree.data.data[...] = ...`): kept marks of the empty leaves
+        are dropped, and a backward pass that follows does not use notes its forward pass took of
+        the old values.  Every write path of this package calls it; a caller that writes through
+        `tree.data.data` itself must (no reference counterpart)."""
+        self._writes = getattr(self, "_writes", 0) + 1
+        self._leaf_marks = None
 
     def _spec(self, world=True):
         """The TreeSpec handed to the operators (svox/svox.py:1084-1103).  For tree-local queries
@@ -625,6 +635,7 @@ class N3Tree(nn.Module):
         spec.scaling = self.invradius if world else None
         spec._weight_accum = getattr(self, "_weight_accum", None)
         spec._weight_accum_max = getattr(self, "_weight_accum_op", None) == "max"
+        spec.owner = self    # lets the autograd functions see the tree's write counter
         if getattr(self, "_leaf_marks", None) is not None:
             if self._leaf_marks_key == self._marks_key():
                 spec.child_marks = self._leaf_marks
@@ -641,8 +652,8 @@ class N3Tree(nn.Module):
         The marks describe the tree as it is now.  They are dropped by every method of the tree and
         its views that writes values or changes the structure, and by in-place torch operations on
         `tree.data` / `tree.child` (their version counters tell).  A write that bypasses both --
-        `tree.data.data -= ...` as in svox's own toy example -- does not: call `clear_leaf_marks()`
-        (or this method again) after such a write."""
+        `tree.data.data -= ...` as in svox's own toy example -- does not: call `tree.touch()`
+        (or `clear_leaf_marks()`, or this method again) after such a write."""
         self._leaf_marks = None
         self._leaf_marks = _C.mark_empty_leaves(self._spec())
         self._leaf_marks_key = self._marks_key()
@@ -652,7 +663,8 @@ class N3Tree(nn.Module):
         self._leaf_marks = None
 
     def _marks_key(self):
-        return (self._ver, self.data._version, self.child._version, self.data.data_ptr(), self.child.data_ptr())
+        return (self._ver, getattr(self, "_writes", 0), self.data._version, self.child._version,
+                self.data.data_ptr(), self.child.data_ptr())
 
     def _maybe_auto_data_dim(self):
         fmt_dim = self.data_format.data_dim if self.data_format is not None else None

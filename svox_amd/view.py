@@ -64,7 +64,7 @@ class N3TreeView:
         if isinstance(value, N3TreeView):
             value = value.values_nograd
         data = self.tree.data.data
-        self.tree.clear_leaf_marks()      # the write below goes past data's version counter
+        self.tree.touch()      # the write below goes past data's version counter
         if self._needs_two_step():
             rows = data[self.key[:-1]]
             rows[..., self.key[-1]] = value

@@ -596,3 +596,151 @@ def test_training_step_in_a_hip_graph(gpu):
         assert torch.equal(g_out, want_out), step
         err, ok = grad_close(g_grad.cpu().numpy(), want_grad.cpu().numpy())
         assert ok, (step, err)
+
+
+def test_writes_past_the_version_counters_between_forward_and_backward(gpu, oracle_mod):
+    """Writes torch's version counters do not see (svox's own idiom, docs/source/ex_opt_toy.py:26, and the
+    views' `set`) between forward and backward: through a view or followed by tree.touch() the backward
+    pass drops the forward pass's notes -- and marks of empty leaves kept on the tree -- and marches
+    through the tree as it then is, which is what the reference's backward pass sees
+    (svox/renderer.py:57-72 keeps nothing of the forward pass)."""
+    tree = on_gpu(synth.shell_tree(depth=6, n_spheres=6, data_format="SH4", seed=31, sigma_range=(20.0, 200.0)), gpu)
+    rays = synth.sphere_rays(3000, seed=3)
+    rays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.dirs.clone().to(gpu))
+    c2w = synth.orbit_poses(1, seed=4, radius=2.5)[0].to(gpu)
+    r = svox.VolumeRenderer(tree, step_size=1e-3)
+    go = (torch.randn(3000, 3, generator=torch.Generator().manual_seed(1)) * 1e-2).to(gpu)
+    gi = (torch.randn(48, 64, 3, generator=torch.Generator().manual_seed(2)) * 1e-2).to(gpu)
+    opt = r._get_options(True)
+    pts = torch.rand(4000, 3, generator=torch.Generator().manual_seed(1)).to(gpu)
+
+    def oracle_grads():
+        ot = oracle_mod.Tree.from_n3tree(tree)      # the tree as it is now
+        a = oracle_mod.volume_render_backward(ot, rays.origins.cpu(), rays.dirs.cpu(), rays.viewdirs.cpu(), opt, go.cpu())
+        b = oracle_mod.volume_render_image_backward(ot, c2w.cpu(), 50.0, 50.0, 64, 48, opt, gi.cpu())
+        return a, b
+
+    def check(write):
+        tree.data.grad = None
+        out = r(rays, fast=True)
+        img = r.render_persp(c2w, width=64, height=48, fx=50.0, fast=True)
+        versions = (tree.data._version, tree.child._version)
+        write()
+        assert (tree.data._version, tree.child._version) == versions    # torch has not seen the write
+        want_batch, want_image = oracle_grads()
+        out.backward(go)
+        err, ok = grad_close(tree.data.grad.cpu().numpy(), want_batch)
+        assert ok, err
+        tree.data.grad = None
+        img.backward(gi)
+        err, ok = grad_close(tree.data.grad.cpu().numpy(), want_image)
+        assert ok, err
+
+    def view_write():
+        tree[pts, -1:] = 150.0           # N3TreeView.set: empty leaves become dense
+
+    def raw_write_then_touch():
+        tree.data.data[..., -1] *= 0.25
+        tree.touch()
+
+    def kernel_write():
+        tree.set(pts[:500], torch.full((500, tree.data_dim), 0.3, device=gpu))
+
+    for marked in (False, True):
+        for write in (view_write, raw_write_then_touch, kernel_write):
+            if marked:
+                tree.mark_empty_leaves()
+                assert tree._spec().child_marks is not None
+            check(write)
+            assert tree._spec().child_marks is None      # every such write also drops kept marks
+
+    # kept marks + a view write: the next picture is the one an unmarked tree gives
+    tree.mark_empty_leaves()
+    tree[pts[:100], -1:] = 0.0
+    tree[pts[100:200], -1:] = 90.0
+    with torch.no_grad():
+        after = r.render_persp(c2w, width=64, height=48, fx=50.0, fast=True)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    assert np.array_equal(after.cpu().numpy(), oracle_mod.volume_render_image(ot, c2w.cpu(), 50.0, 50.0, 64, 48, opt))
+
+
+def test_notes_are_not_replayed_for_other_directions_or_another_structure(gpu, oracle_mod):
+    """The stamp of the notes in a workspace names the ray directions and the child table as well:
+    svox_volume_render_backward_noted called with other directions (same origins), or with another
+    child table (same data), marches instead of replaying notes that do not belong to the call."""
+    tree = on_gpu(synth.shell_tree(depth=5, n_spheres=5, data_format="SH4", seed=8, sigma_range=(20.0, 200.0)), gpu)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    n = 2000
+    rays = synth.sphere_rays(n, seed=6)
+    other = synth.sphere_rays(n, seed=7)
+    opt = options(tree, step_size=1e-3)
+    go = (torch.randn(n, 3, generator=torch.Generator().manual_seed(3)) * 1e-2).to(gpu)
+    spec = tree._spec()
+    rs = rays_spec(rays, gpu)
+    out, notes = C.volume_render_noted(spec, rs, opt)
+    assert notes is not None
+    # same origins tensor, other directions
+    rs2 = C.RaysSpec()
+    rs2.origins = rs.origins
+    rs2.dirs = other.dirs.to(gpu)
+    # (aim the new directions from the old origins at the cube again)
+    tgt = torch.rand(n, 3, generator=torch.Generator().manual_seed(9)).to(gpu)
+    d = tgt - rs.origins
+    rs2.dirs = (d / d.norm(dim=1, keepdim=True)).contiguous()
+    rs2.vdirs = rs2.dirs.clone()
+    got = C.volume_render_backward_noted(spec, rs2, opt, go, notes)
+    want = oracle_mod.volume_render_backward(ot, rs2.origins.cpu(), rs2.dirs.cpu(), rs2.vdirs.cpu(), opt, go.cpu())
+    err, ok = grad_close(got.cpu().numpy(), want)
+    assert ok, err
+    # same data tensor, another child table (every leaf of the first node's children merged away is
+    # not needed: a table of the same shape in which the root's cells are leaves is enough)
+    out, notes = C.volume_render_noted(spec, rs, opt)
+    flat = tree._spec()
+    flat.child = torch.zeros_like(tree.child)
+    got = C.volume_render_backward_noted(flat, rs, opt, go, notes)
+    flat_tree = oracle_mod.Tree(tree.data.detach().cpu().numpy(), flat.child.cpu().numpy(), tree.parent_depth.cpu().numpy(),
+                                tree.offset.cpu().numpy(), tree.invradius.cpu().numpy())
+    want = oracle_mod.volume_render_backward(flat_tree, rays.origins, rays.dirs, rays.viewdirs, opt, go.cpu())
+    err, ok = grad_close(got.cpu().numpy(), want)
+    assert ok, err
+
+
+def test_workspace_and_marking_thresholds_from_both_sides(gpu, monkeypatch):
+    """The two size heuristics of the shim: the backward workspace (notes) shrinks to what the byte
+    limit and the free device memory allow and is left out below 15 leaves per ray; a multi-pose call
+    marks the empty leaves from AUTO_MARK_RAYS_PER_CELL rays per cell on.  Results do not depend on
+    either."""
+    tree = on_gpu(synth.shell_tree(depth=5, n_spheres=4, data_format="SH4", seed=5, sigma_range=(20.0, 200.0)), gpu)
+    n = 4096
+    size_of = C._abi.load_library().svox_volume_render_backward_workspace_bytes
+    assert C._backward_workspace(tree, n)[1] == size_of(n, 30)
+    monkeypatch.setattr(C, "BACKWARD_WORKSPACE_LIMIT", size_of(n, 30) - 1)
+    assert C._backward_workspace(tree, n)[1] == size_of(n, 15)
+    monkeypatch.setattr(C, "BACKWARD_WORKSPACE_LIMIT", size_of(n, 15))
+    assert C._backward_workspace(tree, n)[1] == size_of(n, 15)
+    monkeypatch.setattr(C, "BACKWARD_WORKSPACE_LIMIT", size_of(n, 15) - 1)
+    assert C._backward_workspace(tree, n) == (None, 0)
+    # no room: the differentiable forward pass runs without notes, the gradient is the same
+    rays = synth.sphere_rays(n, seed=2)
+    rays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.dirs.clone().to(gpu))
+    r = svox.VolumeRenderer(tree, step_size=1e-3)
+    go = torch.randn(n, 3, device=gpu)
+    r(rays).backward(go)
+    without_notes = tree.data.grad.clone()
+    tree.data.grad = None
+    monkeypatch.setattr(C, "BACKWARD_WORKSPACE_LIMIT", 4 << 30)
+    r(rays).backward(go)
+    err, ok = grad_close(tree.data.grad.cpu().numpy(), without_notes.cpu().numpy())
+    assert ok, err
+    # the share of the free memory: a large request is cut down to it
+    monkeypatch.setattr(C, "_ASK_DEVICE_ABOVE", 0)
+    monkeypatch.setattr(C, "BACKWARD_WORKSPACE_FREE_FRACTION", 1e-9)
+    assert C._backward_workspace(tree, n) == (None, 0)
+    monkeypatch.setattr(C, "BACKWARD_WORKSPACE_FREE_FRACTION", 0.25)
+    assert C._backward_workspace(tree, n)[1] == size_of(n, 30)
+    # marking: exactly at the threshold the call marks, one ray below it does not
+    cells = tree.child.numel()
+    opt = options(tree, step_size=1e-3, fast=True)
+    monkeypatch.setattr(C, "AUTO_MARK_RAYS_PER_CELL", 1000 / cells)
+    assert C._marks_for_this_call(tree._spec(), opt, 1000) is not None
+    assert C._marks_for_this_call(tree._spec(), opt, 999) is None
