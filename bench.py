@@ -56,6 +56,7 @@ def main():
     ap.add_argument("--no-bwd", action="store_true", help="skip the forward+backward leg")
     ap.add_argument("--no-query", action="store_true", help="skip the point-query leg")
     ap.add_argument("--no-large", action="store_true", help="skip the depth-10 SH25 NDC leg")
+    ap.add_argument("--no-generic", action="store_true", help="skip the fp64 / SG / softplus leg (generic kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (rays would shard "
@@ -170,14 +171,35 @@ def main():
     copy_gbs = 5 * 2 * src.numel() * 4 / (a.elapsed_time(b) * 1e-3) / 1e9
     del src, dst
 
-    # HBM bytes per launch of the dominant kernel come from rocprofv3 counters (two separate --pmc runs), not
-    # from this process: the committed summary carries the figure for the default workload
-    traffic = None
+    # the ceiling this gather-bound launch runs against: random 128-byte lines out of a buffer of the
+    # size of tree.data (index_select of 8 Mi rows of 32 floats), in lines per microsecond
+    rows = data_bytes // 128
+    table = torch.empty(rows, 32, dtype=torch.float32, device=dev)
+    idx = torch.randint(0, rows, (1 << 23,), generator=torch.Generator().manual_seed(11)).to(dev)
+    torch.index_select(table, 0, idx)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(3):
+        torch.index_select(table, 0, idx)
+    b.record()
+    torch.cuda.synchronize()
+    gather_lines_per_us = 3 * idx.numel() / (a.elapsed_time(b) * 1e3)
+    del table, idx
+
+    # HBM bytes and L2 requests per launch of the dominant kernel come from rocprofv3 counters (separate
+    # --pmc runs), not from this process: the committed summary carries the figures for the default workload
+    traffic = l2_requests = l2_misses = None
     prof = os.path.join(ROOT, "profiles", "hbm_traffic_sparse512_sh16.txt")
     if args.depth == 9 and args.size == 800 and args.poses == 8 and os.path.exists(prof):
         import re
-        m = re.search(r"traffic_bytes_per_launch:\s*(\d+)", open(prof).read())
+        text = open(prof).read()
+        m = re.search(r"traffic_bytes_per_launch:\s*(\d+)", text)
         traffic = int(m.group(1)) if m else None
+        m = re.search(r"l2_requests_per_launch:\s*(\d+)", text)
+        l2_requests = int(m.group(1)) if m else None
+        m = re.search(r"l2_misses_per_launch:\s*(\d+)", text)
+        l2_misses = int(m.group(1)) if m else None
 
     roofline = {
         "bound": "hbm", "kernel": "render_forward_kernel<OctreePolicy<SH,16>, ImageSource>",
@@ -189,11 +211,26 @@ def main():
         "empty_leaves_marked_per_call": bool(C.AUTO_MARK_RAYS_PER_CELL is not None
                                              and n_rays_step >= C.AUTO_MARK_RAYS_PER_CELL * tree.child.numel()),
         "copy_ceiling_gbs": round(copy_gbs, 1),
+        "rays_hit": int(sum(s["rays_hit"] for s in pose_stats)),
+        "samples": int(sum(s["samples"] for s in pose_stats)),
+        "samples_shaded": int(sum(s["samples_shaded"] for s in pose_stats)),
         "samples_per_ray": round(sum(s["samples"] for s in pose_stats) / n_rays_step, 2),
         "shaded_per_ray": round(sum(s["samples_shaded"] for s in pose_stats) / n_rays_step, 2),
+        "msamples_s": round(sum(s["samples"] for s in pose_stats) / (durs.mean() * 1e3), 1),
+        # the launch as a stream of scattered cache lines: its L2 requests (rocprofv3 TCC_REQ, from the
+        # committed profile) per microsecond against a plain gather of random 128-byte lines measured here
+        "scattered_lines": {
+            "l2_requests_per_launch": l2_requests, "l2_misses_per_launch": l2_misses,
+            "l2_requests_per_us": round(l2_requests / (durs.mean() * 1e3), 1) if l2_requests else None,
+            "l2_misses_per_us": round(l2_misses / (durs.mean() * 1e3), 1) if l2_misses else None,
+            "torch_index_select_lines_per_us": round(gather_lines_per_us, 1),
+            # filled in by the query leg: what this library's own gather kernel reaches on random records
+            "gather_ceiling_lines_per_us": None, "misses_over_gather_ceiling": None,
+        },
     }
     per_call = {"value": round(n_rays_step / (per_call_ms * 1e-3) / 1e6, 3), "unit": "Mrays/s",
-                "ms_per_step": round(per_call_ms, 4),
+                "ms_per_step": round(per_call_ms, 4), "ms_per_pose": round(per_call_ms / args.poses, 4),
+                "mrays_hit_s": round(roofline["rays_hit"] / (per_call_ms * 1e-3) / 1e6, 1),
                 "note": "same step as one render_persp call (one launch) per pose, the reference's calling pattern"}
     log(f"[bench] forward {fwd_ms:.2f} ms/step, {fwd_mrays:.1f} Mrays/s (one call per pose: {per_call}), roofline {roofline}")
 
@@ -373,6 +410,15 @@ def main():
             "calc_corners": {"mleaves_s": round(leaves.shape[0] / c_ms / 1e3, 1), "ms": round(c_ms, 4),
                              "algorithmic_gbs": round(c_bytes / c_ms / 1e6, 1)},
         }
+        # the gather kernel as a ceiling for scattered lines: a 112-byte record at a 112-byte stride lies in
+        # 1 + 111/128 lines of 128 bytes on average, and every point reads one (the child reads hit in L2)
+        lines_per_point = 1.0 + (4 * Kq - 1) / 128.0
+        sl = roofline["scattered_lines"]
+        sl["gather_ceiling_lines_per_us"] = round(Q * lines_per_point / (q_ms * 1e3), 1)
+        sl["gather_ceiling_note"] = (f"query_vertical, {Q} random points, {4 * Kq}-byte records of a 268 MB tree: "
+                                     f"{lines_per_point:.2f} lines read per point")
+        if sl["l2_misses_per_us"]:
+            sl["misses_over_gather_ceiling"] = round(sl["l2_misses_per_us"] / sl["gather_ceiling_lines_per_us"], 4)
         # render_persp of the same dense tree: one 800x800 pose from the radius-4 orbit, thresholds 0
         # (every ray that hits shades some 57 leaves; the tree and its child table sit in the 256 MB
         # Infinity Cache, so bytes fetched from HBM are far below the algorithmic ones here)
@@ -412,6 +458,59 @@ def main():
             del qot, qref
         del qtree, pts, go, leaves, qimg, qgo
         log(f"[bench] query {query}")
+
+    # ---------------------------------------------------------------- what the generic kernels do
+    # (fp64 data, spherical-Gaussian lobes, density_softplus: one ray per lane, the reference's loop)
+    generic = None
+    if not args.no_generic:
+        def ev_time(fn, n=3):
+            fn()
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(n):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b) / n
+
+        generic = {"workload": f"dense 128^3 tree (SH9 / SG9 records), one {W}x{H} pose, thresholds 0; "
+                               "4M-point query in fp64"}
+        gtree = synth.dense_tree(6, "SH9", seed=0, sigma="lognormal", coeff_std=0.5, zero_fraction=0.5).to(dev)
+        gcam = _make_camera_spec(poses[0].contiguous(), W, H, fx, fx)
+        with torch.no_grad():
+            base_ms = ev_time(lambda: C.volume_render_image(gtree._spec(), gcam, svox.VolumeRenderer(gtree)._get_options(False)))
+            soft_opt = svox.VolumeRenderer(gtree, density_softplus=True)._get_options(False)
+            soft_ms = ev_time(lambda: C.volume_render_image(gtree._spec(), gcam, soft_opt))
+            C.set_debug_flags(1)
+            try:
+                forced_ms = ev_time(lambda: C.volume_render_image(gtree._spec(), gcam, svox.VolumeRenderer(gtree)._get_options(False)))
+            finally:
+                C.set_debug_flags(0)
+        generic["fp32_sh9_octree_kernel_ms"] = round(base_ms, 4)
+        generic["fp32_sh9_generic_kernel_ms"] = round(forced_ms, 4)
+        generic["fp32_sh9_density_softplus_ms"] = round(soft_ms, 4)
+        # SG lobes on the same records (extra_data: lambda, mu)
+        lobes = torch.cat([torch.rand(9, 1, generator=torch.Generator().manual_seed(2)) * 4 + 0.5,
+                           synth.unit_vectors(9, torch.Generator().manual_seed(3))], dim=1).to(dev)
+        sgtree = svox.N3Tree(N=2, data_format="SG9", init_refine=0, extra_data=lobes, device=dev)
+        sgtree.data, sgtree.child, sgtree.parent_depth = gtree.data, gtree.child, gtree.parent_depth
+        sgtree._n_internal.fill_(gtree.n_internal)
+        with torch.no_grad():
+            sg_opt = svox.VolumeRenderer(sgtree)._get_options(False)
+            generic["fp32_sg9_ms"] = round(ev_time(lambda: C.volume_render_image(sgtree._spec(), gcam, sg_opt)), 4)
+        del sgtree
+        gtree64 = gtree.double()
+        g64cam = _make_camera_spec(poses[0].double().contiguous(), W, H, fx, fx)
+        pts64 = torch.rand(1 << 22, 3, generator=torch.Generator().manual_seed(3), dtype=torch.float64).to(dev)
+        with torch.no_grad():
+            opt64 = svox.VolumeRenderer(gtree64)._get_options(False)
+            generic["fp64_sh9_ms"] = round(ev_time(lambda: C.volume_render_image(gtree64._spec(), g64cam, opt64)), 4)
+            generic["fp64_query_4M_ms"] = round(ev_time(lambda: C.query_vertical(gtree64._spec(), pts64)), 4)
+        generic["mrays_s"] = {k[:-3]: round(W * H / v / 1e3, 1) for k, v in generic.items() if k.endswith("_ms") and "query" not in k}
+        del gtree, gtree64, pts64
+        torch.cuda.empty_cache()
+        log(f"[bench] generic kernels {generic}")
 
     # ---------------------------------------------------------------- depth-10 SH25 tree, NDC camera
     large = None
@@ -536,6 +635,8 @@ def main():
         "value": round(fwd_mrays, 3), "unit": "Mrays/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(fwd_ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "rays_hit": roofline["rays_hit"], "mrays_hit_s": round(roofline["rays_hit"] / (fwd_ms * 1e-3) / 1e6, 1),
+        "msamples_s": round(roofline["samples"] / (fwd_ms * 1e-3) / 1e6, 1),
         "config": {"workload": "sparse512_sh16: 8 poses x 800x800, step 5e-4, sigma/stop thresh 1e-2",
                    "depth": args.depth, "image": [W, H], "poses": args.poses, "nodes": tree.info["nodes"],
                    "leaves": tree.info["leaves"], "occupancy": round(tree.info["occupancy"], 5),
@@ -546,6 +647,7 @@ def main():
         "fwd_bwd": fwd_bwd,
         "query": query,
         "large": large,
+        "generic_kernels": generic,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)

@@ -699,6 +699,10 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         // ---- sigma
         float q_sigma[kQueue];
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+        if (opt.density_softplus) {   // rt_kernel.cu:276-277 (the launcher passes no marks with this option)
+#pragma unroll
+            for (int q = 0; q < kQueue; ++q) q_sigma[q] = q_leaf[q] >= 0 ? softplus_m1(q_sigma[q]) : 0.0f;
+        }
         // ---- shade list
         const int n_entries = build_shade_list(sh, q_leaf, q_sigma, sigma_thresh, lane);
         bool stopped = false;

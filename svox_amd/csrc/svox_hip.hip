@@ -176,8 +176,9 @@ int check_rays(const SvoxRaysSpec* rays) {
 }
 
 // default options on an fp32 octree whose record matches the format: the specialised kernels
-int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
-    if (!octree_fast_ok(tree) || opt->density_softplus) return -1;
+// (density_softplus only in the forward kernel: `softplus_ok`)
+int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, bool softplus_ok = false) {
+    if (!octree_fast_ok(tree) || (opt->density_softplus && !softplus_ok)) return -1;
     if (opt->format == SVOX_FORMAT_RGBA) return tree->data_dim == 4 ? 0 : -1;
     if (opt->format != SVOX_FORMAT_SH) return -1;
     const int D = opt->basis_dim;
@@ -190,7 +191,8 @@ int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
 // of the child table where they apply (no leaf with sigma <= 0 may contribute: sigma_thresh >= 0).
 TreeDev<float> march_tree(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
     TreeDev<float> d = make_tree<float>(tree);
-    if (tree->child_marks && opt->sigma_thresh >= 0.0f) d.child = tree->child_marks;
+    // (softplus of any stored density is > 0: no leaf is empty then)
+    if (tree->child_marks && opt->sigma_thresh >= 0.0f && !opt->density_softplus) d.child = tree->child_marks;
     return d;
 }
 
@@ -306,7 +308,7 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
                     void* out, hipStream_t stream) {
     const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
-        const int D = fast_basis(tree, opt);
+        const int D = fast_basis(tree, opt, true);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
             const Source dealt = dealt_out(src, blocks);

@@ -744,3 +744,83 @@ def test_workspace_and_marking_thresholds_from_both_sides(gpu, monkeypatch):
     monkeypatch.setattr(C, "AUTO_MARK_RAYS_PER_CELL", 1000 / cells)
     assert C._marks_for_this_call(tree._spec(), opt, 1000) is not None
     assert C._marks_for_this_call(tree._spec(), opt, 999) is None
+
+
+def test_render_of_a_saved_and_loaded_tree(gpu, oracle_mod, tmp_path):
+    """save -> load -> render (svox/svox.py:835-865, 899-938): the file stores float16 records, so the
+    picture of the loaded tree is, bit for bit, the picture of the original tree with its records
+    rounded to float16 -- on the GPU and in the oracle.  (Interoperability with a file written by the
+    reference itself cannot be pinned: the reference ships none.)"""
+    tree = synth.shell_tree(depth=6, n_spheres=5, data_format="SH9", seed=12, sigma_range=(20.0, 200.0))
+    path = str(tmp_path / "scene.npz")
+    tree.save(path)
+    loaded = svox.N3Tree.load(path, device=gpu)
+    assert loaded.data.is_cuda and loaded.child.is_cuda and repr(loaded.data_format) == "SH9"
+    rounded = on_gpu(tree, gpu)
+    with torch.no_grad():
+        rounded.data.copy_(rounded.data.half().float())
+    c2w = synth.orbit_poses(1, seed=2, radius=2.5)[0]
+    kw = dict(width=120, height=90, fx=100.0, fast=True)
+    with torch.no_grad():
+        a = svox.VolumeRenderer(loaded, step_size=1e-3).render_persp(c2w.to(gpu), **kw)
+        b = svox.VolumeRenderer(rounded, step_size=1e-3).render_persp(c2w.to(gpu), **kw)
+        c = svox.VolumeRenderer(on_gpu(tree, gpu), step_size=1e-3).render_persp(c2w.to(gpu), **kw)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    ot = oracle_mod.Tree.from_n3tree(loaded)
+    ref = oracle_mod.volume_render_image(ot, c2w, 100.0, 100.0, 120, 90, options(loaded, step_size=1e-3, fast=True))
+    assert np.array_equal(a.cpu().numpy(), ref)
+    pts = torch.rand(5000, 3, generator=torch.Generator().manual_seed(1)).to(gpu)
+    va, ia = loaded(pts, want_node_ids=True)
+    vb, ib = rounded(pts, want_node_ids=True)
+    assert torch.equal(ia, ib) and torch.equal(va, vb)
+
+
+@pytest.mark.parametrize("fmt", ["SH9", "RGBA"])
+def test_density_softplus_on_the_octree_forward_kernel(gpu, oracle_mod, fmt):
+    """density_softplus (rt_kernel.cu:276-277) in the specialised forward kernel: bit for bit what the
+    generic kernel gives (one softplus routine on the device), 1e-5 from the oracle (another logf),
+    for a ray batch handled both ways and for an image; marks of empty leaves play no part (the
+    softplus of any stored density is > 0).  The backward pass of this option stays on the generic kernels."""
+    tree = synth.shell_tree(depth=6, n_spheres=5, data_format=fmt, seed=17, sigma_range=(0.5, 30.0))
+    with torch.no_grad():
+        tree.data[..., -1] -= 3.0                 # stored densities of both signs
+    rays = synth.sphere_rays(3000, seed=4)
+    opt = options(tree, step_size=1e-3, density_softplus=True, fast=True, rgb_padding=0.001)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    ref = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    marked = dev._spec()
+    marked.child_marks = C.mark_empty_leaves(dev._spec())
+    C.set_debug_flags(1)
+    try:
+        generic = C.volume_render(dev._spec(), rs, opt)
+    finally:
+        C.set_debug_flags(0)
+    assert np.abs(generic.cpu().numpy() - ref).max() <= 1e-5
+    for flags in (0, 2):
+        C.set_debug_flags(flags)
+        try:
+            assert torch.equal(C.volume_render(dev._spec(), rs, opt), generic), flags
+            assert torch.equal(C.volume_render(marked, rs, opt), generic), flags
+        finally:
+            C.set_debug_flags(0)
+    c2w = synth.orbit_poses(1, seed=4, radius=2.5)[0]
+    cam = cam_spec(c2w, 75, 53, 60.0, device=gpu)
+    img = C.volume_render_image(dev._spec(), cam, opt)
+    want = oracle_mod.volume_render_image(ot, c2w, 60.0, 60.0, 75, 53, opt)
+    assert np.abs(img.cpu().numpy() - want).max() <= 1e-5
+    C.set_debug_flags(1)
+    try:
+        assert torch.equal(C.volume_render_image(dev._spec(), cam, opt), img)
+    finally:
+        C.set_debug_flags(0)
+    # through the renderer: forward on the octree kernel, gradient by the generic backward kernel
+    r = svox.VolumeRenderer(dev, step_size=1e-3, density_softplus=True, rgb_padding=0.001)
+    go = (torch.randn(3000, 3, generator=torch.Generator().manual_seed(2)) * 1e-2).to(gpu)
+    out = r(svox.Rays(rs.origins, rs.dirs, rs.vdirs), fast=True)
+    assert torch.equal(out.detach(), generic)
+    out.backward(go)
+    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go.cpu())
+    err, ok = grad_close(dev.data.grad.cpu().numpy(), want_g, rel=2e-4)   # (logf and its derivative from two libraries)
+    assert ok, err

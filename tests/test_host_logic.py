@@ -196,14 +196,60 @@ def test_no_cpu_fallback_and_argument_checks():
 
 
 def test_save_load_round_trip(tmp_path):
+    """npz persistence (svox/svox.py:835-865, 899-938): the file holds the reference's keys, `data` as
+    float16; load gives back exactly the float16-rounded tree."""
     tree = synth.shell_tree(depth=4, n_spheres=2, data_format="SH4", seed=3)
+    original = tree.data.data.clone()
     path = str(tmp_path / "tree.npz")
     tree.save(path)
+    z = np.load(path)
+    assert sorted(z.files) == sorted(["data_dim", "child", "parent_depth", "n_internal", "n_free", "invradius3",
+                                      "offset", "depth_limit", "geom_resize_fact", "data", "data_format"])
+    assert z["data"].dtype == np.float16 and z["child"].dtype == np.int32 and str(z["data_format"]) == "SH4"
     back = svox.N3Tree.load(path)
     assert torch.equal(back.child, tree.child) and torch.equal(back.parent_depth, tree.parent_depth)
     assert back.n_internal == tree.n_internal and repr(back.data_format) == "SH4"
-    assert torch.allclose(back.data.data, tree.data.data.half().float())      # stored as float16
-    assert torch.equal(back.invradius, tree.invradius) and back.check_integrity()
+    assert back.data.dtype == torch.float32
+    assert torch.equal(back.data.data, original[:tree.n_internal].half().float())      # exactly the fp16 rounding
+    assert not torch.equal(back.data.data, original[:tree.n_internal])                 # ... which is lossy
+    assert torch.equal(back.invradius, tree.invradius) and torch.equal(back.offset, tree.offset)
+    assert back.depth_limit == tree.depth_limit and back.geom_resize_fact == tree.geom_resize_fact
+    assert int(back._n_free) == 0 and back.check_integrity()
+    # saving what was loaded is a fixed point: float16 values survive float16 storage
+    path2 = str(tmp_path / "again.npz")
+    back.save(path2, compress=False)
+    again = svox.N3Tree.load(path2, dtype=torch.float64)
+    assert again.data.dtype == torch.float64 and torch.equal(again.data.data.float(), back.data.data)
+    # an SG tree keeps its lobes
+    sg = svox.N3Tree(data_format="SG2", init_refine=1, extra_data=torch.rand(2, 4))
+    sg.save(str(tmp_path / "sg.npz"))
+    assert torch.equal(svox.N3Tree.load(str(tmp_path / "sg.npz")).extra_data, sg.extra_data)
+
+
+def test_load_reads_the_legacy_file_layout(tmp_path):
+    """Files written before `invradius3`, `n_free` and `data_format` existed (svox/svox.py:920-934):
+    a scalar `invradius` fills all three axes, `n_free` defaults to 0, the format to None (the
+    renderer then infers SH from data_dim, svox/renderer.py:171-176)."""
+    tree = synth.dense_tree(2, "SH4", seed=4, sigma="lognormal")
+    n = tree.n_internal
+    path = str(tmp_path / "legacy.npz")
+    np.savez(path, data_dim=np.int64(tree.data_dim), child=tree.child[:n].numpy(), parent_depth=tree.parent_depth[:n].numpy(),
+             n_internal=np.int64(n), invradius=np.float64(0.25), offset=np.array([0.5, 0.25, 0.125]),
+             depth_limit=np.int64(7), geom_resize_fact=np.float64(1.5), data=tree.data.data[:n].numpy().astype(np.float16))
+    back = svox.N3Tree.load(path)
+    assert torch.equal(back.invradius, torch.full((3,), 0.25)) and back.invradius.dtype == torch.float32
+    assert torch.equal(back.offset, torch.tensor([0.5, 0.25, 0.125])) and back.offset.dtype == torch.float32
+    assert int(back._n_free) == 0 and back.data_format is None and back.depth_limit == 7
+    assert back.geom_resize_fact == 1.5 and back.N == 2 and back.data_dim == 13 and back.n_internal == n
+    assert torch.equal(back.data.data, tree.data.data[:n].half().float()) and back.check_integrity()
+    with pytest.warns(UserWarning, match="Legacy N3Tree"):
+        r = svox.VolumeRenderer(back)
+    assert repr(r.data_format) == "SH4"
+    # a freed node count that is stored is honoured
+    blob = dict(np.load(path))
+    blob["n_free"] = np.int64(2)
+    np.savez(str(tmp_path / "freed.npz"), **blob)
+    assert int(svox.N3Tree.load(str(tmp_path / "freed.npz"))._n_free) == 2
 
 
 def test_generators_are_seeded():
