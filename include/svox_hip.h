@@ -125,7 +125,9 @@ const char* svox_status_string(int status);
 /* Debugging aid without a counterpart in the reference.  Bit 0: route every call to the generic
  * kernels (any N, any dtype) even where a specialised octree kernel exists.  Bit 1: ray batches of
  * any size run the way batches of 512 Ki rays and more do (several 64-ray chunks per wavefront, idle
- * lanes refilled), so that small test batches reach those kernels. */
+ * lanes refilled), so that small test batches reach those kernels.  Bit 2: forward renders never take
+ * the kernel that walks and shades on two wavefronts; bit 3: they always do where it applies (launches
+ * of one 64-ray wavefront per tile or chunk, no weight accumulator), whatever their size. */
 void svox_set_debug_flags(int flags);
 
 /* query_vertical(TreeSpec&, Tensor indices) -> (values, node_ids); svox/csrc/svox_kernel.cu:120-143.

@@ -693,5 +693,6 @@ def volume_render_stats(tree, rays_or_cam, opt):
 
 
 def set_debug_flags(flags):
-    """bit 0: route every call to the generic kernels; bit 1: small ray batches run like large ones"""
+    """bit 0: route every call to the generic kernels; bit 1: small ray batches run like large ones;
+    bit 2 / bit 3: forward renders never / always take the two-wavefront kernel"""
     _abi.load_library().svox_set_debug_flags(int(flags))

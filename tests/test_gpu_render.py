@@ -107,6 +107,12 @@ def test_image_render_and_backward(gpu, oracle_mod, ndc):
     out = C.volume_render_image(dev._spec(), cam, opt)
     assert out.shape == (H, W, 3)
     assert np.array_equal(out.cpu().numpy(), ref)
+    for flags in (4, 8):     # either forward kernel for launches of this size, whatever the choice would be
+        C.set_debug_flags(flags)
+        try:
+            assert torch.equal(C.volume_render_image(dev._spec(), cam, opt), out), flags
+        finally:
+            C.set_debug_flags(0)
     assert ref_stats["rays_hit"] > 0.2 * W * H
     stats = C.volume_render_stats(dev._spec(), cam, opt)
     assert stats["samples"] == ref_stats["samples"] and stats["rays"] == W * H
@@ -302,12 +308,13 @@ def test_pathological_rays_end_and_match_the_oracle(gpu, oracle_mod, fmt):
         out, ref, stats, ref_stats, dev, ot = render_both(gpu, oracle_mod, tree, rays, opt)
         assert np.array_equal(out, ref, equal_nan=True)
         assert stats["samples"] == ref_stats["samples"]
-        C.set_debug_flags(1)
-        try:
-            out_generic = C.volume_render(dev._spec(), rays_spec(rays, gpu), opt).cpu().numpy()
-        finally:
-            C.set_debug_flags(0)
-        assert np.array_equal(out_generic, ref, equal_nan=True)
+        for flags in (1, 2, 4, 8):     # generic kernel; refilling kernel; one wavefront per 64 rays; two
+            C.set_debug_flags(flags)
+            try:
+                other = C.volume_render(dev._spec(), rays_spec(rays, gpu), opt).cpu().numpy()
+            finally:
+                C.set_debug_flags(0)
+            assert np.array_equal(other, ref, equal_nan=True), flags
         go = torch.ones(rays.origins.shape[0], 3)
         ref_grad = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
         grad = C.volume_render_backward(dev._spec(), rays_spec(rays, gpu), opt, go.to(gpu)).cpu().numpy()
