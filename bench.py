@@ -281,6 +281,7 @@ def main():
         grad_out = (torch.randn(B, 3, generator=g) * 1e-2).to(dev)
         lr = 1e-3
         train_stats = C.volume_render_stats(spec, _rays_spec_from_rays(rays), opt)
+        data_before = tree.data.data.clone()   # the SGD steps below change the tree; put back afterwards
         ev = []
 
         def train_step(record=False):
@@ -367,6 +368,34 @@ def main():
             "includes": "zero-fill of gradient and Hessian diagonal (2 x data); one march that takes notes, "
                         "then residual, gradient and Hessian from the notes"}
         del target
+        with torch.no_grad():
+            tree.data.data.copy_(data_before)
+        del data_before
+        # the gradient of one whole pose (every pixel a ray): neighbouring rays share leaves, unlike the random rays above
+        igo = (torch.randn(H, W, 3, generator=g) * 1e-2).to(dev)
+        icam = _make_camera_spec(poses[0].contiguous(), W, H, fx, fx)
+
+        def image_step():
+            tree.data.grad = None
+            renderer.render_persp(poses[0], width=W, height=H, fx=fx, fast=True).backward(igo)
+
+        def timed(fn, n=3):
+            fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) * 1e3 / n
+
+        fwd_bwd["image_pose"] = {
+            "forward_backward_ms": round(timed(image_step), 3),
+            "backward_marching_ms": round(timed(lambda: C.volume_render_image_backward(spec, icam, opt, igo,
+                                                                                        workspace=False)), 3),
+            "note": f"render_persp of pose 0 ({W}x{H}) and its gradient through autograd; then the stateless "
+                    "backward operator without a workspace (zero-fill of the gradient included in both)"}
+        tree.data.grad = None
+        del igo
         log(f"[bench] fwd+bwd {fwd_bwd}")
 
     # ---------------------------------------------------------------- point queries (dense 128^3 SH9 tree)
@@ -436,6 +465,20 @@ def main():
             qrend.render_persp(poses[0], width=W, height=H, fx=fx).backward(qgo)
 
         qrb_ms = ev_time(dense_train, n=3)
+        qrm_ms = ev_time(lambda: C.volume_render_image_backward(qspec, qcam, qopt, qgo, workspace=False), n=3)
+        # the same tree from close by (a finest voxel covers some 12x12 pixels): the rays of a wavefront
+        # share their leaves, so the backward pass sums the records of a leaf before its atomics
+        near = synth.orbit_poses(1, seed=3, radius=1.2)[0].to(dev)
+        ncam = _make_camera_spec(near.contiguous(), W, H, fx, fx)
+        with torch.no_grad():
+            nr_ms = ev_time(lambda: qrend.render_persp(near, width=W, height=H, fx=fx), n=3)
+
+        def near_train():
+            qtree.data.grad = None
+            qrend.render_persp(near, width=W, height=H, fx=fx).backward(qgo)
+
+        nrb_ms = ev_time(near_train, n=3)
+        nrm_ms = ev_time(lambda: C.volume_render_image_backward(qspec, ncam, qopt, qgo, workspace=False), n=3)
         qtree.data.grad = None
         qr_bytes = forward_bytes(qstats, W * H, Kq, 12)
         query["render_persp"] = {
@@ -448,6 +491,10 @@ def main():
             "algorithmic_gbs": round(qr_bytes / qr_ms / 1e6, 1),
             "frac_of_peak": round(qr_bytes / qr_ms / 1e6 / PEAK_HBM_GBS, 4),
             "forward_backward_ms": round(qrb_ms, 4),
+            "backward_marching_ms": round(qrm_ms, 4),
+            "close_up": {"workload": "the same tree from radius 1.2: about 12 pixels across a finest voxel",
+                         "ms": round(nr_ms, 4), "forward_backward_ms": round(nrb_ms, 4),
+                         "backward_marching_ms": round(nrm_ms, 4)},
         }
         if not args.no_cpu:
             from oracle import oracle as _oracle
