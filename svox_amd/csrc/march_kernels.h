@@ -787,6 +787,17 @@ struct SplitBox {
     int32_t taken[kMarchThreads];          // set by the shading: leaves taken out so far (| kEndedBit)
 };
 
+// The two counters are read and written as relaxed atomics of the workgroup: the compiler then neither
+// keeps them in registers nor moves them across one another, and, unlike a volatile access (which it
+// leaves on the generic address path: a flat instruction with a wait for every store), it still knows
+// that they live in LDS and issues plain LDS reads and writes.
+__device__ __forceinline__ int32_t box_read(const int32_t* at) {
+    return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void box_write(int32_t* at, int32_t value) {
+    __hip_atomic_store(at, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 template <class P, class Source>
 __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(TreeDev<float> tr, Source src,
                                                                              SvoxRenderOptions opt,
@@ -829,12 +840,10 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         }
     }
     if (!__any(active)) return;   // (both wavefronts see the same rays: both leave or both stay)
-    volatile int32_t* written_box = box.written;
-    volatile int32_t* taken_box = box.taken;
     if (walks)
-        written_box[lane] = 0;
+        box.written[lane] = 0;
     else
-        taken_box[lane] = active ? 0 : kEndedBit;
+        box.taken[lane] = active ? 0 : kEndedBit;
     __syncthreads();
 
     if (walks) {
@@ -850,10 +859,10 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         while (true) {
             // (reading the shading's count only every few turns was measured slower: rays that have
             // stopped are then walked further)
-            const int32_t taken = taken_box[lane];
+            const int32_t taken = box_read(&box.taken[lane]);
             live = live && !(taken & kEndedBit);
             if (live && (broken || !(r.t < r.tmax))) {   // the walk of this ray is over: say so once
-                written_box[lane] = written | kEndedBit;
+                box_write(&box.written[lane], written | kEndedBit);
                 live = false;
             }
             if (!__any(live)) break;
@@ -877,7 +886,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
             // (a wavefront's LDS operations are carried out in order: the leaf is in the ring before the
             // count says so; only the compiler has to be told)
             asm volatile("" ::: "memory");
-            if (put) written_box[lane] = written;
+            if (put) box_write(&box.written[lane], written);
         }
         return;
     }
@@ -888,7 +897,8 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
     int32_t taken = 0;
     int spins = 0;
     while (true) {
-        const int32_t w = written_box[lane];
+        const int32_t w = box_read(&box.written[lane]);
+        asm volatile("" ::: "memory");   // the ring is read after the count, not before
         const int32_t avail = (w & ~kEndedBit) - taken;
         if (active && (w & kEndedBit) && avail == 0) {
             // the ray left the tree: the background shows through what is left of the light
@@ -902,7 +912,11 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         // (waiting for fuller hands -- two or four leaves per lane, a few looks of patience -- and a ring
         // of 16 were measured: no gain, the larger ring costs LDS)
         if (!__any(n_take > 0)) {   // the walk has found nothing new yet
-            if (++spins > kSpinLimit) break;
+            if (++spins > kSpinLimit) {
+                // cannot happen while the walk runs; a picture with NaN in it says so if it ever does
+                if (active) out[slot * 3] = out[slot * 3 + 1] = out[slot * 3 + 2] = __int_as_float(0x7fc00000);
+                break;
+            }
             __builtin_amdgcn_s_sleep(1);
             continue;
         }
@@ -917,7 +931,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         }
         wave_lds_sync();   // the leaves are out of the ring before the count gives their places back
         taken += n_take;
-        if (n_take > 0) taken_box[lane] = taken;
+        if (n_take > 0) box_write(&box.taken[lane], taken);
         float q_sigma[kQueue];
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);
         if (opt.density_softplus) {
@@ -956,7 +970,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
             out[slot * 3 + 1] = acc[1] * scale;
             out[slot * 3 + 2] = acc[2] * scale;
             active = false;
-            taken_box[lane] = taken | kEndedBit;
+            box_write(&box.taken[lane], taken | kEndedBit);
         }
     }
 }

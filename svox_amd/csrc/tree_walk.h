@@ -108,6 +108,19 @@ __device__ __forceinline__ int cell_at(uint32_t ix, uint32_t iy, uint32_t iz, in
     return (int)((((bx << 1) | by) << 1) | bz);
 }
 
+// One child entry for the point queries: from the rows staged in LDS for nodes below lds_nodes, else
+// from memory.  Written as an LDS read that every lane makes (of entry 0 where the node is not
+// staged) and a memory read under a condition: a choice between the two pointers would leave the
+// compiler with one load through the generic address path, which is the slower way into LDS.
+__device__ __forceinline__ int32_t child_entry(const int32_t* __restrict__ child, const int32_t* lds_child,
+                                               int32_t lds_nodes, int32_t node, int32_t cell) {
+    const bool staged = node < lds_nodes;
+    int32_t skip = lds_child[staged ? cell : 0];
+    asm volatile("" : "+v"(skip));   // (keeps the two reads apart)
+    if (!staged) skip = child[cell];
+    return skip;
+}
+
 // Octree walk over integer coordinates with no path memory (point queries).
 // `lds_child` holds the child rows of nodes [0, lds_nodes); deeper nodes are read from memory.
 // Returns the leaf cell index node*8 + cell (or -1) and the number of levels visited.
@@ -118,7 +131,7 @@ __device__ __forceinline__ int32_t descend_octree(const int32_t* __restrict__ ch
     int32_t node = 0;
     for (int level = 1; level <= kCoordBits; ++level) {
         const int32_t cell = node * 8 + cell_at(ix, iy, iz, level);
-        const int32_t skip = node < lds_nodes ? lds_child[cell] : child[cell];
+        const int32_t skip = child_entry(child, lds_child, lds_nodes, node, cell);
         if (skip == 0) {
             *levels = level;
             return cell;
@@ -153,7 +166,7 @@ __device__ __forceinline__ void descend_octree_multi(const int32_t* __restrict__
         for (int u = 0; u < kPts; ++u) {
             cell[u] = node[u] * 8 + cell_at(ix[u], iy[u], iz[u], level);
             skip[u] = 0;
-            if (live[u]) skip[u] = node[u] < lds_nodes ? lds_child[cell[u]] : child[cell[u]];
+            if (live[u]) skip[u] = child_entry(child, lds_child, lds_nodes, node[u], cell[u]);
         }
         any_live = false;
 #pragma unroll
