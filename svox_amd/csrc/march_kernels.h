@@ -1213,7 +1213,10 @@ __device__ __forceinline__ void add_records_by_leaf(int n, int lane, const int32
     }
 }
 
-constexpr int kEmitCap = 60;   // 60 * (leaf 4 + g_sigma 4 + tmp2 12 + owner 1) = 1260 of 1280 bytes
+// One record per lane of a wavefront: a step in which all 64 lanes emit fills the list once.  Leaves,
+// density terms and colour factors (20 bytes a record) fill ShadeShared::leaf and ::who exactly; the
+// owners follow the GroupScratch in ShadeShared::colour.
+constexpr int kEmitCap = kMarchThreads;
 template <class P, int D, bool kByRecord = false>
 struct RecordList {
     static constexpr int K = P::kRecord;
@@ -1224,30 +1227,93 @@ struct RecordList {
     int n = 0;   // wavefront-uniform
 
     __device__ __forceinline__ int32_t* leaves() const { return sh.leaf; }
-    __device__ __forceinline__ float* g_sigmas() const { return (float*)(sh.leaf + kEmitCap); }
-    __device__ __forceinline__ float* tmp2s() const { return (float*)(sh.leaf + 2 * kEmitCap); }
-    __device__ __forceinline__ uint8_t* owners() const { return (uint8_t*)(sh.leaf + 5 * kEmitCap); }
+    // per record four factors: the three colour factors tmp2[c], then the density term
+    __device__ __forceinline__ float* factors() const { return (float*)(sh.leaf + kEmitCap); }
+    __device__ __forceinline__ uint8_t* owners() const { return (uint8_t*)sh.colour + sizeof(GroupScratch); }
 
     // element e of record rec: basis[i] * tmp2[c] for a colour coefficient, g_sigma for the density
     __device__ __forceinline__ float element(int rec, int e) const {
         const int c = P::kFormat == SVOX_FORMAT_RGBA ? e : e / D;
         if (c < 3) {
-            const float v = tmp2s()[rec * 3 + c];
+            const float v = factors()[rec * 4 + c];
             return P::kFormat == SVOX_FORMAT_RGBA ? v : sh.basis[owners()[rec] * D + (e - c * D)] * v;
         }
-        return g_sigmas()[rec];
+        return factors()[rec * 4 + 3];
     }
 
     // The colours of the round are in registers by the time records are added: their LDS is free.
     __device__ __forceinline__ GroupScratch& scratch() const { return *(GroupScratch*)sh.colour; }
 
+    // add_records_by_leaf for records longer than half a wavefront (one record at a time, lane e on
+    // element e).  What the lanes need to find a record's values -- its place in the list, its leaf,
+    // its owner -- is first taken into registers, record r by lane r, and then handed round by
+    // readlane: per record that leaves two LDS reads (the factor of the lane's channel, the owner's
+    // basis value) whose addresses come from scalars, so the reads of kHeldBlock records are in flight
+    // together.  (Through LDS alone a record costs three reads that wait for one another: place, owner,
+    // basis.)  order: the records' adding order (grouped by leaf), or nullptr for the list's own.
+    static constexpr bool kHeld = K > kMarchThreads / 2;
+    static constexpr int kHeldBlock = 4;
+    __device__ __forceinline__ void add_held(const uint8_t* order) {
+        const bool mine = lane < n;
+        const int rec = mine ? (order ? order[lane] : lane) : 0;
+        int my_rec = rec;
+        int my_leaf = leaves()[rec];
+        int my_owner = owners()[rec];
+        // Every lane must hold its record before any lane reads it by readlane.  The compiler does not
+        // know that readlane looks into other lanes: without this it moves the reads above into the loop
+        // below, which the lanes beyond K never enter, and their registers stay unset.
+        asm volatile("" : "+v"(my_rec), "+v"(my_leaf), "+v"(my_owner));
+        for (int e = lane; e < K; e += kMarchThreads) {
+            const int c = P::kFormat == SVOX_FORMAT_RGBA ? e : e / D;
+            const int i = P::kFormat == SVOX_FORMAT_RGBA ? 0 : e - c * D;
+            const bool with_basis = P::kFormat != SVOX_FORMAT_RGBA && c < 3;
+            int32_t cur = -1;
+            float acc = 0.0f;
+            for (int at = 0; at < n; at += kHeldBlock) {
+                int32_t leaf[kHeldBlock];
+                float val[kHeldBlock], leaf_basis[kHeldBlock];
+#pragma unroll
+                for (int u = 0; u < kHeldBlock; ++u) {
+                    const int a = at + u < n ? at + u : n - 1;   // (past the end: the last record again, unused)
+                    leaf[u] = __builtin_amdgcn_readlane(my_leaf, a);
+                    const int owner = __builtin_amdgcn_readlane(my_owner, a);
+                    const float t = factors()[__builtin_amdgcn_readlane(my_rec, a) * 4 + c];
+                    // (every lane reads, also the lane of the density element, whose i is 0: a read under a
+                    // condition would be waited for on the spot)
+                    float basis_value = 1.0f;
+                    if constexpr (P::kFormat != SVOX_FORMAT_RGBA) basis_value = sh.basis[owner * D + i];
+                    leaf_basis[u] = basis_value;
+                    val[u] = t;
+                }
+#pragma unroll
+                for (int u = 0; u < kHeldBlock; ++u) val[u] = with_basis ? leaf_basis[u] * val[u] : val[u];
+#pragma unroll
+                for (int u = 0; u < kHeldBlock; ++u) {
+                    if (at + u < n) {
+                        if (leaf[u] != cur) {
+                            if (cur >= 0) atomicAdd(grad_data + (int64_t)cur * K + e, acc);
+                            cur = leaf[u];
+                            acc = 0.0f;
+                        }
+                        acc += val[u];
+                    }
+                }
+            }
+            if (cur >= 0) atomicAdd(grad_data + (int64_t)cur * K + e, acc);
+        }
+    }
+
     // Adds the list with the records of every leaf summed first, if enough records share a leaf.
     __device__ __forceinline__ bool flush_grouped() {
         GroupScratch& gs = scratch();
         if (!group_by_leaf(gs, merge, leaves(), n, lane)) return false;
-        add_records_by_leaf<K, 1>(
-            n, lane, gs.leaf, [&](int at, int e, float* t) { t[0] = element(gs.order[at], e); },
-            [&](int32_t leaf, int e, const float* sum) { atomicAdd(grad_data + (int64_t)leaf * K + e, sum[0]); });
+        if constexpr (kHeld) {
+            add_held(gs.order);
+        } else {
+            add_records_by_leaf<K, 1>(
+                n, lane, gs.leaf, [&](int at, int e, float* t) { t[0] = element(gs.order[at], e); },
+                [&](int32_t leaf, int e, const float* sum) { atomicAdd(grad_data + (int64_t)leaf * K + e, sum[0]); });
+        }
         wave_lds_sync();
         n = 0;
         return true;
@@ -1266,13 +1332,13 @@ struct RecordList {
             const int rec = f / K, e = f - rec * K;
             float val;
             if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                val = e < 3 ? tmp2s()[rec * 3 + e] : g_sigmas()[rec];
+                val = factors()[rec * 4 + e];
             } else {
                 if (e < 3 * D) {
                     const int c = e / D;
-                    val = sh.basis[owners()[rec] * D + (e - c * D)] * tmp2s()[rec * 3 + c];
+                    val = sh.basis[owners()[rec] * D + (e - c * D)] * factors()[rec * 4 + c];
                 } else {
-                    val = g_sigmas()[rec];
+                    val = factors()[rec * 4 + 3];
                 }
             }
             atomicAdd(grad_data + (int64_t)leaves()[rec] * K + e, val);
@@ -1287,9 +1353,13 @@ struct RecordList {
         if (n == 0) return;
         wave_lds_sync();
         if (flush_grouped()) return;
-        add_records_by_leaf<K, 1>(
-            n, lane, leaves(), [&](int rec, int e, float* t) { t[0] = element(rec, e); },
-            [&](int32_t leaf, int e, const float* sum) { atomicAdd(grad_data + (int64_t)leaf * K + e, sum[0]); });
+        if constexpr (kHeld) {
+            add_held(nullptr);
+        } else {
+            add_records_by_leaf<K, 1>(
+                n, lane, leaves(), [&](int rec, int e, float* t) { t[0] = element(rec, e); },
+                [&](int32_t leaf, int e, const float* sum) { atomicAdd(grad_data + (int64_t)leaf * K + e, sum[0]); });
+        }
         wave_lds_sync();
         n = 0;
     }
@@ -1305,10 +1375,10 @@ struct RecordList {
             if (take) {
                 leaves()[slot] = leaf;
                 owners()[slot] = (uint8_t)lane;
-                g_sigmas()[slot] = g_sigma;
-                tmp2s()[slot * 3] = tmp2[0];
-                tmp2s()[slot * 3 + 1] = tmp2[1];
-                tmp2s()[slot * 3 + 2] = tmp2[2];
+                factors()[slot * 4] = tmp2[0];
+                factors()[slot * 4 + 1] = tmp2[1];
+                factors()[slot * 4 + 2] = tmp2[2];
+                factors()[slot * 4 + 3] = g_sigma;
             }
             const unsigned long long taken = __ballot(take);
             n += __popcll(taken);
@@ -1316,9 +1386,10 @@ struct RecordList {
         }
     }
 };
-static_assert(5 * kEmitCap * 4 + kEmitCap <= kQueue * kMarchThreads * 5, "record list exceeds the shade list");
+static_assert(5 * kEmitCap * 4 <= kQueue * kMarchThreads * 5, "record list exceeds the shade list");
 static_assert(kEmitCap <= kMarchThreads, "group_by_leaf holds one record per lane");
-static_assert(sizeof(GroupScratch) <= sizeof(float) * kQueue * kMarchThreads * 3, "GroupScratch lives in ShadeShared::colour");
+static_assert(sizeof(GroupScratch) + kEmitCap <= sizeof(float) * kQueue * kMarchThreads * 3,
+              "GroupScratch and the owners live in ShadeShared::colour");
 using ShadeSharedProbe = ShadeShared<1, true>;
 static_assert(offsetof(ShadeSharedProbe, who) == sizeof(int32_t) * kQueue * kMarchThreads,
               "the record list runs from ShadeShared::leaf into ShadeShared::who");
@@ -1724,24 +1795,37 @@ template <class P, class Source>
 __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3))) void replay_backward_kernel(Source src, SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
                                                                         float* __restrict__ grad_data,
-                                                                        ReplaySpace ws) {
+                                                                        ReplaySpace ws, int ray_shift) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     __shared__ ShadeShared<D, true> sh;
     const int lane = threadIdx.x;
-    const int64_t ray = blockIdx.x * (int64_t)kMarchThreads + lane;
+    // A wavefront takes 2^ray_shift consecutive rays (64, 32 or 16), one per lane from lane 0.  Adding a
+    // step's records is work of the whole wavefront, one record after the other; where the rays of a
+    // wavefront are neighbours (the pixels of an image) they are all long or all short together, and
+    // fewer of them per wavefront spread a long run of pixels over several wavefronts.
+    const int64_t ray = ((int64_t)blockIdx.x << ray_shift) + lane;
+    const bool seated = lane < (1 << ray_shift);
     const bool stamped = stamp_matches(ws);
     const float2* first = ws.base + ray * kChunkFloat2;
     int count = 0;
     int32_t first_link = 0;
     float dscale = 0.0f;
-    if (ray < src.n_slots()) {
+    if (seated && ray < src.n_slots()) {
         const float2 head = first[kHeadFloat2], tail = first[kHeadFloat2 + 1];
         first_link = __float_as_int(head.x);
         count = stamped ? __float_as_int(head.y) : -1;
         dscale = tail.x;
     }
+    // (the wavefront's part of the bitmap: a word, half a word or a quarter of one)
     const unsigned long long undone = __ballot(count < 0);
-    if (lane == 0) ws.undone[blockIdx.x] = undone;
+    if (lane == 0) {
+        if (ray_shift == 6)
+            ws.undone[blockIdx.x] = undone;
+        else if (ray_shift == 5)
+            ((uint32_t*)ws.undone)[blockIdx.x] = (uint32_t)undone;
+        else
+            ((uint16_t*)ws.undone)[blockIdx.x] = (uint16_t)undone;
+    }
     const bool work = count > 0;
     if (!__any(work)) return;
 

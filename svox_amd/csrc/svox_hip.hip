@@ -550,12 +550,20 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
                                const void* grad_output, void* grad_data_out, void* workspace, int64_t workspace_bytes,
                                int64_t n_slots, const NoteStamp& stamp, hipStream_t stream) {
     const int D = fast_basis(tree, opt);
-    const unsigned words = blocks_for(n_slots, kMarchThreads);
+    // rays per wavefront of the replay: 16 for the pixels of images (neighbours, long together), 64 for ray
+    // batches (SVOX_REPLAY_SHIFT = 4, 5 or 6 overrides)
+    static const int forced_shift = [] {
+        const char* e = getenv("SVOX_REPLAY_SHIFT");
+        return e ? atoi(e) : -1;
+    }();
+    const int ray_shift = forced_shift >= 4 && forced_shift <= 6 ? forced_shift : (is_image_source(all) ? 4 : 6);
+    const unsigned waves = blocks_for(n_slots, 1 << ray_shift);
     ReplaySpace ws;
     carve_workspace(workspace, workspace_bytes, n_slots, &ws);
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
-    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P, Source>), dim3(words), dim3(kMarchThreads), 0,
-                                               stream, all, *opt, (const float*)grad_output, (float*)grad_data_out, ws));
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P, Source>), dim3(waves), dim3(kMarchThreads), 0,
+                                               stream, all, *opt, (const float*)grad_output, (float*)grad_data_out, ws,
+                                               ray_shift));
     int rc = check_launch("volume_render_backward_noted");
     if (rc) return rc;
     ReplaySpace only = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0, 0, 0}, nullptr, ws.undone};
