@@ -761,221 +761,6 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
 }
 
 // ------------------------------------------------------------------------------------------------
-// forward, walk and shading on two wavefronts
-// ------------------------------------------------------------------------------------------------
-// The round of render_forward_kernel is one chain per wavefront: four turns of the walk (child reads
-// that hit in L2), then the densities and the records of the leaves found (reads that go to HBM), then
-// the colours, then the next walk.  The walk does not depend on what the leaves hold, but a
-// wavefront's loads come back in the order they were issued, so within one wavefront the next walk
-// cannot run while the records are on their way.  Here a block is two wavefronts that share the 64
-// rays of a tile: the first only walks and hands every leaf it finds (that is not marked empty) to
-// the second through a ring in LDS, a few leaves per lane deep; the second takes the leaves as they
-// come, fetches densities and records, evaluates colours and composites exactly as
-// render_forward_kernel does, and tells the walk which rays have stopped.  Same arithmetic, same
-// pictures.  Each wavefront sets the rays up for itself (the same instructions give the same rays).
-// A wavefront that finds nothing to do sleeps a few cycles and looks again; after kSpinLimit looks in a
-// row it gives up, so that a launch ends whatever happens.
-constexpr int kSplitThreads = 2 * kMarchThreads;
-constexpr int kRing = 8;               // leaves a lane's walk may be ahead of its shading (a power of two)
-constexpr int kSpinLimit = 1 << 22;
-constexpr int32_t kEndedBit = 1 << 30;   // in SplitBox::written: the ray's walk is over; in ::taken: the ray wants no more leaves
-
-struct SplitBox {
-    int32_t leaf[kRing * kMarchThreads];   // [place in the ring][lane]
-    float dt[kRing * kMarchThreads];
-    int32_t written[kMarchThreads];        // set by the walk: leaves put into the lane's ring so far (| kEndedBit)
-    int32_t taken[kMarchThreads];          // set by the shading: leaves taken out so far (| kEndedBit)
-};
-
-// The two counters are read and written as relaxed atomics of the workgroup: the compiler then neither
-// keeps them in registers nor moves them across one another, and, unlike a volatile access (which it
-// leaves on the generic address path: a flat instruction with a wait for every store), it still knows
-// that they live in LDS and issues plain LDS reads and writes.
-__device__ __forceinline__ int32_t box_read(const int32_t* at) {
-    return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-}
-__device__ __forceinline__ void box_write(int32_t* at, int32_t value) {
-    __hip_atomic_store(at, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-}
-
-template <class P, class Source>
-__global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(TreeDev<float> tr, Source src,
-                                                                             SvoxRenderOptions opt,
-                                                                             float* __restrict__ out) {
-    constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
-    constexpr int K = P::kRecord;
-    __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
-    __shared__ ShadeShared<D, false> sh;
-    __shared__ SplitBox box;
-    const int lane = threadIdx.x & (kMarchThreads - 1);
-    const bool walks = threadIdx.x < kMarchThreads;   // uniform in a wavefront
-    float offset[3], scaling[3];
-    load_transform(tr, offset, scaling);
-    const float bg = opt.background_brightness;
-    const float pad = opt.rgb_padding;
-    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
-    const float step = opt.step_size, sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
-
-    const int64_t item = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)kMarchThreads + lane;
-    RayState<float> r;
-    int64_t slot = -1;
-    bool active = false;
-    {
-        float origin[3], dir[3], vdir[3];
-        if (item < src.total()) slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
-        if (slot >= 0) active = setup_ray(r, origin, dir, scaling);
-        if (!walks) {
-            if (slot >= 0 && !active) {
-                out[slot * 3] = bg;
-                out[slot * 3 + 1] = bg;
-                out[slot * 3 + 2] = bg;
-            }
-            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
-                if (active) {
-                    sh.vdir[lane * 3] = vdir[0];
-                    sh.vdir[lane * 3 + 1] = vdir[1];
-                    sh.vdir[lane * 3 + 2] = vdir[2];
-                }
-            }
-        }
-    }
-    if (!__any(active)) return;   // (both wavefronts see the same rays: both leave or both stay)
-    if (walks)
-        box.written[lane] = 0;
-    else
-        box.taken[lane] = active ? 0 : kEndedBit;
-    __syncthreads();
-
-    if (walks) {
-        // ---- the walk: one leaf per live lane and turn, into the ring
-        OctreeCursor cur;
-        cur.reset(path + lane, kMarchThreads);
-        int32_t written = 0;
-        bool live = active, broken = false;
-        int spins = 0;
-        // the walk is the longest chain of a tile: it goes first where wavefronts share a SIMD
-        // (measured: -10 % on a dense image, nothing elsewhere)
-        __builtin_amdgcn_s_setprio(3);
-        while (true) {
-            // (reading the shading's count only every few turns was measured slower: rays that have
-            // stopped are then walked further)
-            const int32_t taken = box_read(&box.taken[lane]);
-            live = live && !(taken & kEndedBit);
-            if (live && (broken || !(r.t < r.tmax))) {   // the walk of this ray is over: say so once
-                box_write(&box.written[lane], written | kEndedBit);
-                live = false;
-            }
-            if (!__any(live)) break;
-            const bool go = live && written - (taken & ~kEndedBit) < kRing;
-            if (!__any(go)) {   // every ring is full: the shading is behind
-                if (++spins > kSpinLimit) break;
-                __builtin_amdgcn_s_sleep(1);
-                continue;
-            }
-            spins = 0;
-            int32_t leaf;
-            float dt;
-            walk_turn_flat(tr, r, cur, step, go, broken, leaf, dt);
-            const bool put = go && leaf >= 0 && !(leaf & kEmptyLeafBit);
-            if (put) {
-                const int at = (written & (kRing - 1)) * kMarchThreads + lane;
-                box.leaf[at] = leaf;
-                box.dt[at] = dt;
-                written += 1;
-            }
-            // (a wavefront's LDS operations are carried out in order: the leaf is in the ring before the
-            // count says so; only the compiler has to be told)
-            asm volatile("" ::: "memory");
-            if (put) box_write(&box.written[lane], written);
-        }
-        return;
-    }
-
-    // ---- the shading: takes up to kQueue leaves per lane at a time, as render_forward_kernel's round
-    float acc[3] = {0.f, 0.f, 0.f};
-    float light = 1.0f;
-    int32_t taken = 0;
-    int spins = 0;
-    while (true) {
-        const int32_t w = box_read(&box.written[lane]);
-        asm volatile("" ::: "memory");   // the ring is read after the count, not before
-        const int32_t avail = (w & ~kEndedBit) - taken;
-        if (active && (w & kEndedBit) && avail == 0) {
-            // the ray left the tree: the background shows through what is left of the light
-            out[slot * 3] = fma_(light, bg, acc[0]);
-            out[slot * 3 + 1] = fma_(light, bg, acc[1]);
-            out[slot * 3 + 2] = fma_(light, bg, acc[2]);
-            active = false;
-        }
-        if (!__any(active)) break;
-        const int n_take = active ? (avail < kQueue ? avail : kQueue) : 0;
-        // (waiting for fuller hands -- two or four leaves per lane, a few looks of patience -- and a ring
-        // of 16 were measured: no gain, the larger ring costs LDS)
-        if (!__any(n_take > 0)) {   // the walk has found nothing new yet
-            if (++spins > kSpinLimit) {
-                // cannot happen while the walk runs; a picture with NaN in it says so if it ever does
-                if (active) out[slot * 3] = out[slot * 3 + 1] = out[slot * 3 + 2] = __int_as_float(0x7fc00000);
-                break;
-            }
-            __builtin_amdgcn_s_sleep(1);
-            continue;
-        }
-        spins = 0;
-        int32_t q_leaf[kQueue];
-        float q_dt[kQueue];
-#pragma unroll
-        for (int q = 0; q < kQueue; ++q) {
-            const int at = ((taken + q) & (kRing - 1)) * kMarchThreads + lane;
-            q_leaf[q] = q < n_take ? box.leaf[at] : -1;
-            q_dt[q] = q < n_take ? box.dt[at] : 0.0f;
-        }
-        wave_lds_sync();   // the leaves are out of the ring before the count gives their places back
-        taken += n_take;
-        if (n_take > 0) box_write(&box.taken[lane], taken);
-        float q_sigma[kQueue];
-        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
-        if (opt.density_softplus) {
-#pragma unroll
-            for (int q = 0; q < kQueue; ++q) q_sigma[q] = q_leaf[q] >= 0 ? softplus_m1(q_sigma[q]) : 0.0f;
-        }
-        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, sigma_thresh, lane);
-        bool stopped = false;
-        if (n_entries > 0) {
-            wave_lds_sync();
-            shade_entries<P, false>(tr.data, sh, n_entries, lane);
-            wave_lds_sync();
-            float q_att[kQueue], q_rgb[kQueue][3];
-#pragma unroll
-            for (int q = 0; q < kQueue; ++q) {
-                q_att[q] = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
-                const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
-#pragma unroll
-                for (int c = 0; c < 3; ++c) q_rgb[q][c] = fma_(s[c], d_rgb_pad, -pad);
-            }
-#pragma unroll
-            for (int q = 0; q < kQueue; ++q) {
-                const bool take = active && q_leaf[q] >= 0 && !stopped && q_sigma[q] > sigma_thresh;
-                const float weight = light * (1.0f - q_att[q]);
-#pragma unroll
-                for (int c = 0; c < 3; ++c) acc[c] = take ? fma_(weight, q_rgb[q][c], acc[c]) : acc[c];
-                light = take ? light * q_att[q] : light;
-                stopped = stopped || (take && light <= stop_thresh);
-            }
-            wave_lds_sync();   // the colours are read before the next list overwrites them
-        }
-        if (active && stopped) {
-            // rt_kernel.cu:306-313: rescale and leave without the background; the walk may stop
-            const float scale = (float)(1.0 / (1.0 - (double)light));
-            out[slot * 3] = acc[0] * scale;
-            out[slot * 3 + 1] = acc[1] * scale;
-            out[slot * 3 + 2] = acc[2] * scale;
-            active = false;
-            box_write(&box.taken[lane], taken | kEndedBit);
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 // backward
 // ------------------------------------------------------------------------------------------------
 // trace_ray_backward, rt_kernel.cu:323-477, generic flavour: two marches, the colour gradients in
@@ -1459,6 +1244,303 @@ constexpr int kChunkRecords = 15;
 constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
 constexpr int kHeadFloat2 = kChunkRecords * 3;          // float2 index of {link, count}, then {delta_scale, -}
 constexpr int kChunkStock = 64;   // further chunks a wavefront takes at a time (at most 64 lanes ask at once)
+
+// ------------------------------------------------------------------------------------------------
+// forward, walk and shading on two wavefronts
+// ------------------------------------------------------------------------------------------------
+// The round of render_forward_kernel is one chain per wavefront: four turns of the walk (child reads
+// that hit in L2), then the densities and the records of the leaves found (reads that go to HBM), then
+// the colours, then the next walk.  The walk does not depend on what the leaves hold, but a
+// wavefront's loads come back in the order they were issued, so within one wavefront the next walk
+// cannot run while the records are on their way.  Here a block is two wavefronts that share the 64
+// rays of a tile: the first only walks and hands every leaf it finds (that is not marked empty) to
+// the second through a ring in LDS, a few leaves per lane deep; the second takes the leaves as they
+// come, fetches densities and records, evaluates colours and composites exactly as
+// render_forward_kernel does, and tells the walk which rays have stopped.  Same arithmetic, same
+// pictures.  Each wavefront sets the rays up for itself (the same instructions give the same rays).
+// A wavefront that finds nothing to do sleeps a few cycles and looks again; after kSpinLimit looks in a
+// row it gives up, so that a launch ends whatever happens.
+//
+// kNoted: the launch also leaves, for the backward pass, the notes render_backward_kernel<kForwardNoted>
+// leaves (same workspace, same format): every leaf with sigma > 0 of the whole ray, so the walk goes on
+// after the picture's early stop, and the colours of leaves below sigma_thresh are evaluated too; the
+// picture itself is composed as without notes.
+constexpr int kSplitThreads = 2 * kMarchThreads;
+constexpr int kRing = 8;               // leaves a lane's walk may be ahead of its shading (a power of two)
+constexpr int kSpinLimit = 1 << 22;
+constexpr int32_t kEndedBit = 1 << 30;   // in SplitBox::written: the ray's walk is over; in ::taken: the ray wants no more leaves
+constexpr int32_t kBrokenBit = 1 << 29;  // in SplitBox::written, beside kEndedBit: the walk ended in a malformed tree
+
+struct SplitBox {
+    int32_t leaf[kRing * kMarchThreads];   // [place in the ring][lane]
+    float dt[kRing * kMarchThreads];
+    int32_t written[kMarchThreads];        // set by the walk: leaves put into the lane's ring so far (| kEndedBit)
+    int32_t taken[kMarchThreads];          // set by the shading: leaves taken out so far (| kEndedBit)
+};
+
+// The two counters are read and written as relaxed atomics of the workgroup: the compiler then neither
+// keeps them in registers nor moves them across one another, and, unlike a volatile access (which it
+// leaves on the generic address path: a flat instruction with a wait for every store), it still knows
+// that they live in LDS and issues plain LDS reads and writes.
+__device__ __forceinline__ int32_t box_read(const int32_t* at) {
+    return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void box_write(int32_t* at, int32_t value) {
+    __hip_atomic_store(at, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+template <class P, class Source, bool kNoted = false>
+__global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(TreeDev<float> tr, Source src,
+                                                                             SvoxRenderOptions opt,
+                                                                             float* __restrict__ out, ReplaySpace ws) {
+    constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
+    constexpr int K = P::kRecord;
+    __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
+    __shared__ ShadeShared<D, false> sh;
+    __shared__ SplitBox box;
+    if constexpr (kNoted) {
+        if (blockIdx.x == 0 && threadIdx.x < kStampWords) ws.stamp_at[threadIdx.x] = ws.stamp[threadIdx.x];
+    }
+    const int lane = threadIdx.x & (kMarchThreads - 1);
+    const bool walks = threadIdx.x < kMarchThreads;   // uniform in a wavefront
+    float offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    const float bg = opt.background_brightness;
+    const float pad = opt.rgb_padding;
+    const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
+    const float step = opt.step_size, sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
+
+    const int64_t item = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)kMarchThreads + lane;
+    RayState<float> r;
+    int64_t slot = -1;
+    bool active = false;
+    {
+        float origin[3], dir[3], vdir[3];
+        if (item < src.total()) slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+        if (slot >= 0) active = setup_ray(r, origin, dir, scaling);
+        if (!walks) {
+            if (slot >= 0 && !active) {
+                out[slot * 3] = bg;
+                out[slot * 3 + 1] = bg;
+                out[slot * 3 + 2] = bg;
+                if constexpr (kNoted) {
+                    ws.base[slot * kChunkFloat2 + kHeadFloat2] = make_float2(0.0f, __int_as_float(0));   // no notes
+                    ws.base[slot * kChunkFloat2 + kHeadFloat2 + 1] = make_float2(0.0f, 1.0f);            // missed
+                }
+            }
+            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+                if (active) {
+                    sh.vdir[lane * 3] = vdir[0];
+                    sh.vdir[lane * 3 + 1] = vdir[1];
+                    sh.vdir[lane * 3 + 2] = vdir[2];
+                }
+            }
+        }
+    }
+    if (!__any(active)) return;   // (both wavefronts see the same rays: both leave or both stay)
+    if (walks)
+        box.written[lane] = 0;
+    else
+        box.taken[lane] = active ? 0 : kEndedBit;
+    __syncthreads();
+
+    if (walks) {
+        // ---- the walk: one leaf per live lane and turn, into the ring
+        OctreeCursor cur;
+        cur.reset(path + lane, kMarchThreads);
+        int32_t written = 0;
+        bool live = active, broken = false;
+        int spins = 0;
+        // the walk is the longest chain of a tile: it goes first where wavefronts share a SIMD
+        // (measured: -10 % on a dense image, nothing elsewhere)
+        __builtin_amdgcn_s_setprio(3);
+        while (true) {
+            // (reading the shading's count only every few turns was measured slower: rays that have
+            // stopped are then walked further)
+            const int32_t taken = box_read(&box.taken[lane]);
+            live = live && !(taken & kEndedBit);
+            if (live && (broken || !(r.t < r.tmax))) {   // the walk of this ray is over: say so once
+                box_write(&box.written[lane], written | kEndedBit | (broken ? kBrokenBit : 0));
+                live = false;
+            }
+            if (!__any(live)) break;
+            const bool go = live && written - (taken & ~kEndedBit) < kRing;
+            if (!__any(go)) {   // every ring is full: the shading is behind
+                if (++spins > kSpinLimit) break;
+                __builtin_amdgcn_s_sleep(1);
+                continue;
+            }
+            spins = 0;
+            int32_t leaf;
+            float dt;
+            walk_turn_flat(tr, r, cur, step, go, broken, leaf, dt);
+            const bool put = go && leaf >= 0 && !(leaf & kEmptyLeafBit);
+            if (put) {
+                const int at = (written & (kRing - 1)) * kMarchThreads + lane;
+                box.leaf[at] = leaf;
+                box.dt[at] = dt;
+                written += 1;
+            }
+            // (a wavefront's LDS operations are carried out in order: the leaf is in the ring before the
+            // count says so; only the compiler has to be told)
+            asm volatile("" ::: "memory");
+            if (put) box_write(&box.written[lane], written);
+        }
+        return;
+    }
+
+    // ---- the shading: takes up to kQueue leaves per lane at a time, as render_forward_kernel's round
+    float acc[3] = {0.f, 0.f, 0.f};
+    float light = 1.0f;
+    int32_t taken = 0;
+    int spins = 0;
+    // kNoted: the picture of a ray may be finished (early stop) while its notes go on
+    bool painted = false;
+    // the notes of this lane's ray: their number, the chunk being written and the place in it
+    int rec_count = 0, rec_pos = 0;
+    bool rec_lost = false;   // the workspace ran out: this ray's backward pass will march
+    float2* rec_first = ws.base;
+    float2* rec_chunk = ws.base;
+    int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of further chunks (uniform)
+    if constexpr (kNoted) {
+        if (active) {
+            rec_first = ws.base + slot * kChunkFloat2;
+            rec_chunk = rec_first;
+        }
+    }
+    while (true) {
+        const int32_t w = box_read(&box.written[lane]);
+        asm volatile("" ::: "memory");   // the ring is read after the count, not before
+        const int32_t avail = (w & ~(kEndedBit | kBrokenBit)) - taken;
+        if (active && (w & kEndedBit) && avail == 0) {
+            // the ray left the tree: the background shows through what is left of the light
+            if (!painted) {
+                out[slot * 3] = fma_(light, bg, acc[0]);
+                out[slot * 3 + 1] = fma_(light, bg, acc[1]);
+                out[slot * 3 + 2] = fma_(light, bg, acc[2]);
+            }
+            if constexpr (kNoted) {
+                // the head of the notes: the count beside the link (written when the first chunk filled
+                // up), then delta_scale
+                ((float*)(rec_first + kHeadFloat2))[1] = __int_as_float(rec_lost || (w & kBrokenBit) ? -1 : rec_count);
+                rec_first[kHeadFloat2 + 1] = make_float2(r.dscale, 0.0f);
+            }
+            active = false;
+        }
+        if (!__any(active)) break;
+        const int n_take = active ? (avail < kQueue ? avail : kQueue) : 0;
+        // (waiting for fuller hands -- two or four leaves per lane, a few looks of patience -- and a ring
+        // of 16 were measured: no gain, the larger ring costs LDS)
+        if (!__any(n_take > 0)) {   // the walk has found nothing new yet
+            if (++spins > kSpinLimit) {
+                // cannot happen while the walk runs; a picture with NaN in it says so if it ever does
+                if (active) out[slot * 3] = out[slot * 3 + 1] = out[slot * 3 + 2] = __int_as_float(0x7fc00000);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+            continue;
+        }
+        spins = 0;
+        int32_t q_leaf[kQueue];
+        float q_dt[kQueue];
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q) {
+            const int at = ((taken + q) & (kRing - 1)) * kMarchThreads + lane;
+            q_leaf[q] = q < n_take ? box.leaf[at] : -1;
+            q_dt[q] = q < n_take ? box.dt[at] : 0.0f;
+        }
+        wave_lds_sync();   // the leaves are out of the ring before the count gives their places back
+        taken += n_take;
+        if (n_take > 0) box_write(&box.taken[lane], taken);
+        float q_sigma[kQueue];
+        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+        if (opt.density_softplus) {
+#pragma unroll
+            for (int q = 0; q < kQueue; ++q) q_sigma[q] = q_leaf[q] >= 0 ? softplus_m1(q_sigma[q]) : 0.0f;
+        }
+        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, kNoted ? 0.0f : sigma_thresh, lane);
+        bool stopped = false;
+        if (n_entries > 0) {
+            wave_lds_sync();
+            shade_entries<P, false>(tr.data, sh, n_entries, lane);
+            wave_lds_sync();
+            float q_att[kQueue], q_rgb[kQueue][3], q_s[kQueue][3];
+#pragma unroll
+            for (int q = 0; q < kQueue; ++q) {
+                q_att[q] = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
+                const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+#pragma unroll
+                for (int c = 0; c < 3; ++c) {
+                    q_s[q][c] = s[c];
+                    q_rgb[q][c] = fma_(s[c], d_rgb_pad, -pad);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < kQueue; ++q) {
+                const bool take = active && !painted && q_leaf[q] >= 0 && !stopped && q_sigma[q] > sigma_thresh;
+                const float weight = light * (1.0f - q_att[q]);
+#pragma unroll
+                for (int c = 0; c < 3; ++c) acc[c] = take ? fma_(weight, q_rgb[q][c], acc[c]) : acc[c];
+                light = take ? light * q_att[q] : light;
+                stopped = stopped || (take && light <= stop_thresh);
+                if constexpr (kNoted) {
+                    // the note of this leaf; lanes whose chunk is full take the next chunks of the
+                    // wavefront's stock, in lane order (as render_backward_kernel does)
+                    const bool note = active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
+                    const bool need = note && !rec_lost && rec_pos == kChunkRecords;
+                    const unsigned long long m = __ballot(need);
+                    if (m) {
+                        if (shared_next + __popcll(m) > shared_end) {
+                            unsigned long long t = 0;
+                            if (lane == 0) t = atomicAdd(ws.stocks_taken, 1ull);
+                            const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)t);
+                            const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(t >> 32));
+                            const int64_t stock = (int64_t)(((unsigned long long)hi << 32) | lo);
+                            shared_next = ws.first_shared + stock * kChunkStock;
+                            shared_end = shared_next + kChunkStock < ws.n_chunks ? shared_next + kChunkStock : ws.n_chunks;
+                            if (shared_next > shared_end) shared_next = shared_end;
+                        }
+                        const int64_t mine = shared_next + rank_in(m);
+                        if (need) {
+                            if (mine < shared_end) {
+                                rec_chunk[kHeadFloat2] = make_float2(__int_as_float((int32_t)mine), 0.0f);
+                                rec_chunk = ws.base + mine * kChunkFloat2;
+                                rec_pos = 0;
+                            } else {
+                                rec_lost = true;
+                            }
+                        }
+                        shared_next += __popcll(m);
+                    }
+                    if (note) {
+                        if (!rec_lost) {
+                            float2* e = rec_chunk + rec_pos * 3;
+                            e[0] = make_float2(__int_as_float(q_leaf[q]), q_dt[q]);
+                            e[1] = make_float2(q_sigma[q], q_s[q][0]);
+                            e[2] = make_float2(q_s[q][1], q_s[q][2]);
+                            rec_pos += 1;
+                        }
+                        rec_count += 1;
+                    }
+                }
+            }
+            wave_lds_sync();   // the colours are read before the next list overwrites them
+        }
+        if (active && stopped) {
+            // rt_kernel.cu:306-313: rescale and leave without the background; the walk may stop
+            const float scale = (float)(1.0 / (1.0 - (double)light));
+            out[slot * 3] = acc[0] * scale;
+            out[slot * 3 + 1] = acc[1] * scale;
+            out[slot * 3 + 2] = acc[2] * scale;
+            if constexpr (kNoted) {
+                painted = true;   // the picture is done; the notes go on to the end of the ray
+            } else {
+                active = false;
+                box_write(&box.taken[lane], taken | kEndedBit);
+            }
+        }
+    }
+}
 
 // kReplay: during march 1 a lane notes, for every leaf with sigma > 0, what march 2 needs of it; if
 // the notes fit into the workspace, march 2 does not walk the tree again but replays them (a ray

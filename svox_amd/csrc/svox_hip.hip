@@ -346,9 +346,9 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
                                                *opt, (float*)out))
             const bool refill = src.per_wave > kMarchThreads;
             if (!refill && !tree->weight_accum && use_split_forward(blocks, is_image_source(src))) {
-                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source>), dim3(blocks),
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false>), dim3(blocks),
                                                            dim3(kSplitThreads), 0, stream, march_tree(tree, opt), dealt,
-                                                           *opt, (float*)out));
+                                                           *opt, (float*)out, ReplaySpace{}));
                 return;
             }
             if (tree->weight_accum) {
@@ -433,6 +433,13 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
                                                dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt,     \
                                                *opt, (const float*)grad_out, (float*)grad_data, ws, (float*)out))
             const bool refill = src.per_wave > kMarchThreads;
+            if (mode == kForwardNoted && !refill && use_split_forward(blocks, is_image_source(src))) {
+                // a launch that does not fill the GPU: the walk and the shading (with the notes) on two wavefronts
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, true>), dim3(blocks),
+                                                           dim3(kSplitThreads), 0, stream, march_tree(tree, opt), dealt,
+                                                           *opt, (float*)out, ws));
+                return;
+            }
             if (mode == kBackwardReplay) {
                 if (refill) { SVOX_LAUNCH_BACKWARD(true, kBackwardReplay); } else { SVOX_LAUNCH_BACKWARD(false, kBackwardReplay); }
             } else if (mode == kForwardNoted) {

@@ -4,7 +4,8 @@ Per case: shell / dense / deep-chain tree, 100-5000 sphere rays, random step siz
 thresholds, random background.  Paths: forward, marching backward with and without a workspace, noted
 forward + replayed backward, se_grad with and without a workspace -- each with the rays handled as a
 small batch and as a large one (debug flag 2), on the plain tree and with the empty leaves marked; the
-forward pass also on either of its small-launch kernels (debug flags 4 and 8).
+forward pass, the noted forward pass and se_grad also on either of the small-launch kernels (debug
+flags 4 and 8).
 
 Bars: pictures equal to the oracle's bit for bit; gradients within 1e-4 relative of the oracle's exact
 sum (fp32 terms added in float64) beyond the order slack of fp32 additions, elements below 1e-3 of the
@@ -86,9 +87,10 @@ def test_every_render_path_against_the_exact_sum_oracle(gpu, oracle_mod, case):
     failures = []
     paths = ("fwd", "bwd", "bwd_nows", "noted", "se", "se_nows")
     combos = list(itertools.product((0, 2), ((plain, "plain"), (marked, "marked")), paths))
-    # the forward pass once more on each of its two small-launch kernels (one wavefront per 64 rays that
-    # walks and shades; two wavefronts, one for each), whatever the launch size would choose
-    combos += list(itertools.product((4, 8), ((plain, "plain"), (marked, "marked")), ("fwd",)))
+    # the forward pass, the noted forward pass and se_grad's noting march once more on each of the two
+    # small-launch kernels (one wavefront per 64 rays that walks and shades; two wavefronts, one for
+    # each), whatever the launch size would choose
+    combos += list(itertools.product((4, 8), ((plain, "plain"), (marked, "marked")), ("fwd", "noted", "se")))
     for flags, (spec, spec_name), name in combos:
         tag = f"{name}/flags{flags}/{spec_name}"
         C.set_debug_flags(flags)
