@@ -608,6 +608,141 @@ __device__ __forceinline__ int build_shade_list(Shared& sh, const int32_t* q_lea
     return n_entries;
 }
 
+// Workspace of the replaying backward: chunks of kChunkRecords records of 3 float2 (leaf and step
+// length, density and first sigmoid, the other two sigmoids) followed by one float2 whose x
+// holds the index of the ray's next chunk.  Ray number i starts in chunk i; further chunks come
+// from the rest of the workspace, of which a wavefront takes a stock of 64 chunks at a time through
+// one atomic counter (a heavy image tile needs hundreds, most tiles none); the lanes that need a
+// chunk in the same step are ranked by ballot.
+constexpr int kStampWords = 6;   // ray count; tree data, child; ray origins, directions; step size and threshold
+struct ReplaySpace {
+    float2* base;          // chunk c starts at base + c * kChunkFloat2
+    int64_t first_shared;  // chunks [0, first_shared) are the rays' first chunks
+    int64_t n_chunks;      // chunks [first_shared, n_chunks) are handed out in stocks of kChunkStock
+    unsigned long long* stocks_taken;   // counter of the stocks handed out (zero when the launch starts)
+    // the noting forward kernels write `stamp` (what the notes belong to) to stamp_at; replay_backward_kernel uses
+    // the notes only if it finds its own stamp there
+    unsigned long long* stamp_at;
+    unsigned long long stamp[kStampWords];
+    // one bit per ray (ray i: bit i % 64 of word i / 64).  replay_backward_kernel sets the bits of the
+    // rays it could not do from their notes; a launch of render_backward_kernel that is given the
+    // bitmap as `only` does those rays and no others
+    unsigned long long* undone;
+    const unsigned long long* only;
+};
+
+// whether the workspace carries the stamp this launch expects
+__device__ __forceinline__ bool stamp_matches(const ReplaySpace& ws) {
+    bool same = true;
+#pragma unroll
+    for (int i = 0; i < kStampWords; ++i) same = same && ws.stamp_at[i] == ws.stamp[i];
+    return same;
+}
+
+// The first ray at or after `next` (a wavefront-uniform ray number below `end`) whose 64-ray word of
+// the bitmap `only` is not zero, found 64 words at a time; a value >= end if there is none.
+__device__ __forceinline__ int64_t skip_clear_words(const unsigned long long* __restrict__ only, int64_t next,
+                                                    int64_t end, int lane) {
+    while (next < end) {
+        const int64_t word = next >> 6, last_word = (end - 1) >> 6;
+        const bool some = word + lane <= last_word && only[word + lane] != 0ull;
+        const unsigned long long nz = __ballot(some);
+        if (nz == 0ull) {
+            next = (word + kMarchThreads) << 6;
+            continue;
+        }
+        const int64_t first = (word + __builtin_ctzll(nz)) << 6;
+        if (first > next) next = first;
+        break;
+    }
+    return next;
+}
+
+// What a launch of render_backward_kernel does:
+//   kBackwardPlain   both marches walk the tree;
+//   kBackwardReplay  march 1 leaves notes in the workspace, march 2 replays them.
+// (The notes a forward pass leaves for a later backward pass are taken by render_forward_kernel and
+// render_forward_split_kernel with kNoted, and used by replay_backward_kernel.)
+enum BackwardMode { kBackwardPlain = 0, kBackwardReplay = 1 };
+
+// Head of a ray's notes, kept in the spare floats of its first chunk (after the 15 records): the
+// link to the next chunk, the number of notes (-1: they did not fit; 0 also for a ray that misses
+// the tree), the ray's delta_scale (rt_kernel.cu:228) and 1.0f if the ray misses the tree, else 0.0f.
+constexpr int kChunkRecords = 15;
+constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
+constexpr int kHeadFloat2 = kChunkRecords * 3;          // float2 index of {link, count}, then {delta_scale, -}
+constexpr int kChunkStock = 64;   // further chunks a wavefront takes at a time (at most 64 lanes ask at once)
+
+// The notes of one lane's ray while they are taken (by the forward kernels, for replay_backward_kernel
+// and replay_se_grad_kernel): every leaf with sigma > 0, in the order the ray meets them.
+struct NoteTaker {
+    int count, pos;     // notes so far; place in the chunk being written
+    bool lost;          // the workspace ran out: the backward pass of this ray will march
+    float2* first;      // the ray's own chunk, which also holds the head of its notes
+    float2* chunk;      // the chunk being written
+
+    __device__ __forceinline__ void begin(const ReplaySpace& ws, int64_t slot) {
+        count = 0;
+        pos = 0;
+        lost = false;
+        first = ws.base + slot * kChunkFloat2;
+        chunk = first;
+    }
+    // A ray that misses the tree: no notes, flagged as a miss.
+    static __device__ __forceinline__ void missed(const ReplaySpace& ws, int64_t slot) {
+        ws.base[slot * kChunkFloat2 + kHeadFloat2] = make_float2(0.0f, __int_as_float(0));
+        ws.base[slot * kChunkFloat2 + kHeadFloat2 + 1] = make_float2(0.0f, 1.0f);
+    }
+    // Called by all lanes of the wavefront together; `note`: this lane has a leaf to note.  Lanes whose
+    // chunk is full take the next chunks of the wavefront's stock [shared_next, shared_end), in lane
+    // order; a new stock costs one atomic on the workspace's counter (what is left of the old one is
+    // given up).
+    __device__ __forceinline__ void take(const ReplaySpace& ws, int64_t& shared_next, int64_t& shared_end, int lane,
+                                         bool note, int32_t leaf, float dt, float sigma, const float* s) {
+        const bool need = note && !lost && pos == kChunkRecords;
+        const unsigned long long m = __ballot(need);
+        if (m) {
+            if (shared_next + __popcll(m) > shared_end) {
+                unsigned long long t = 0;
+                if (lane == 0) t = atomicAdd(ws.stocks_taken, 1ull);
+                const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)t);
+                const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(t >> 32));
+                const int64_t stock = (int64_t)(((unsigned long long)hi << 32) | lo);
+                shared_next = ws.first_shared + stock * kChunkStock;
+                shared_end = shared_next + kChunkStock < ws.n_chunks ? shared_next + kChunkStock : ws.n_chunks;
+                if (shared_next > shared_end) shared_next = shared_end;
+            }
+            const int64_t mine = shared_next + rank_in(m);
+            if (need) {
+                if (mine < shared_end) {
+                    chunk[kHeadFloat2] = make_float2(__int_as_float((int32_t)mine), 0.0f);
+                    chunk = ws.base + mine * kChunkFloat2;
+                    pos = 0;
+                } else {
+                    lost = true;
+                }
+            }
+            shared_next += __popcll(m);
+        }
+        if (note) {
+            if (!lost) {
+                float2* e = chunk + pos * 3;
+                e[0] = make_float2(__int_as_float(leaf), dt);
+                e[1] = make_float2(sigma, s[0]);
+                e[2] = make_float2(s[1], s[2]);
+                pos += 1;
+            }
+            count += 1;
+        }
+    }
+    // The head of the notes: the count beside the link (written when the first chunk filled up), -1 if
+    // the notes are incomplete; then the ray's delta_scale.
+    __device__ __forceinline__ void finish(bool broken, float dscale) {
+        ((float*)(first + kHeadFloat2))[1] = __int_as_float(lost || broken ? -1 : count);
+        first[kHeadFloat2 + 1] = make_float2(dscale, 0.0f);
+    }
+};
+
 // trace_ray, octree flavour: a persistent wavefront working in rounds.
 //
 //   refill    lanes whose ray has ended take the next rays of the wavefront's range (ranked by
@@ -629,10 +764,14 @@ __device__ __forceinline__ int build_shade_list(Shared& sh, const int32_t* q_lea
 // tr.weight_accum at the leaf's cell index (rt_kernel.cu:298-304).
 // kRefill: the wavefront owns more than 64 rays and refills idle lanes; without it the 64 rays are
 // set up once before the loop, and nothing the set-up needs stays live inside it.
-template <class P, class Source, bool kAccum, bool kRefill>
+// kNoted: the forward pass of a training step.  The picture is composed as without it; beside it the
+// launch leaves in the workspace the notes the backward pass works from (NoteTaker): every leaf with
+// sigma > 0 of the whole ray, so a ray is walked to its end also after its picture stopped early, and
+// the colours of the leaves at or below sigma_thresh are evaluated too.
+template <class P, class Source, bool kAccum, bool kRefill, bool kNoted = false>
 __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<float> tr, Source src,
                                                                        SvoxRenderOptions opt,
-                                                                       float* __restrict__ out) {
+                                                                       float* __restrict__ out, ReplaySpace ws) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
@@ -649,11 +788,18 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     const int64_t total = src.total();
     const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
+    if constexpr (kNoted) {
+        if (blockIdx.x == 0 && lane < kStampWords) ws.stamp_at[lane] = ws.stamp[lane];
+    }
+
     RayState<float> r;
     float acc[3] = {0.f, 0.f, 0.f};
     float light = 1.0f;
     int64_t slot = -1;
     bool active = false;
+    bool painted = false;   // kNoted: the ray's picture is finished (early stop), its notes go on
+    NoteTaker notes;
+    int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of chunks for notes (uniform)
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
 
@@ -672,10 +818,15 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
             light = 1.0f;
             cur.restart();
             active = true;
+            if constexpr (kNoted) {
+                painted = false;
+                notes.begin(ws, slot);
+            }
         } else {
             out[slot * 3] = bg;
             out[slot * 3 + 1] = bg;
             out[slot * 3 + 2] = bg;
+            if constexpr (kNoted) NoteTaker::missed(ws, slot);
         }
     };
     if constexpr (!kRefill) {
@@ -704,7 +855,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
             for (int q = 0; q < kQueue; ++q) q_sigma[q] = q_leaf[q] >= 0 ? softplus_m1(q_sigma[q]) : 0.0f;
         }
         // ---- shade list
-        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, sigma_thresh, lane);
+        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, kNoted ? 0.0f : sigma_thresh, lane);
         bool stopped = false;
         if (n_entries > 0) {   // most rounds of a ray pass through empty space: nothing to shade
             wave_lds_sync();   // list and view directions are visible to every lane
@@ -713,17 +864,20 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
             // ---- composite
             // the attenuations and padded colours of the four slots do not depend on one another: they
             // are evaluated side by side, and only the products with the transmittance form a chain
-            float q_att[kQueue], q_rgb[kQueue][3];
+            float q_att[kQueue], q_rgb[kQueue][3], q_s[kQueue][3];
 #pragma unroll
             for (int q = 0; q < kQueue; ++q) {
                 q_att[q] = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
                 const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
 #pragma unroll
-                for (int c = 0; c < 3; ++c) q_rgb[q][c] = fma_(s[c], d_rgb_pad, -pad);
+                for (int c = 0; c < 3; ++c) {
+                    q_s[q][c] = s[c];
+                    q_rgb[q][c] = fma_(s[c], d_rgb_pad, -pad);
+                }
             }
 #pragma unroll
             for (int q = 0; q < kQueue; ++q) {
-                const bool take = active && q_leaf[q] >= 0 && !stopped && q_sigma[q] > sigma_thresh;
+                const bool take = active && !painted && q_leaf[q] >= 0 && !stopped && q_sigma[q] > sigma_thresh;
                 const float weight = light * (1.0f - q_att[q]);
 #pragma unroll
                 for (int c = 0; c < 3; ++c) acc[c] = take ? fma_(weight, q_rgb[q][c], acc[c]) : acc[c];
@@ -737,23 +891,32 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                     }
                 }
                 stopped = stopped || (take && light <= stop_thresh);
+                if constexpr (kNoted) {
+                    notes.take(ws, shared_next, shared_end, lane, active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f,
+                               q_leaf[q], q_dt[q], q_sigma[q], q_s[q]);
+                }
             }
         }
         if (active) {
-            if (stopped || broken || !(r.t < r.tmax)) {
-                if (stopped) {
-                    // rt_kernel.cu:306-313: rescale and leave without the background (done here, once
-                    // per round, with the transmittance the ray stopped at)
-                    const float scale = (float)(1.0 / (1.0 - (double)light));
-#pragma unroll
-                    for (int c = 0; c < 3; ++c) acc[c] *= scale;
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 3; ++c) acc[c] = fma_(light, bg, acc[c]);
+            if (stopped) {
+                // rt_kernel.cu:306-313: rescale and leave without the background (done here, once
+                // per round, with the transmittance the ray stopped at)
+                const float scale = (float)(1.0 / (1.0 - (double)light));
+                out[slot * 3] = acc[0] * scale;
+                out[slot * 3 + 1] = acc[1] * scale;
+                out[slot * 3 + 2] = acc[2] * scale;
+                if constexpr (kNoted)
+                    painted = true;   // the notes go on to the end of the ray
+                else
+                    active = false;
+            }
+            if (active && (broken || !(r.t < r.tmax))) {
+                if (!painted) {
+                    out[slot * 3] = fma_(light, bg, acc[0]);
+                    out[slot * 3 + 1] = fma_(light, bg, acc[1]);
+                    out[slot * 3 + 2] = fma_(light, bg, acc[2]);
                 }
-                out[slot * 3] = acc[0];
-                out[slot * 3 + 1] = acc[1];
-                out[slot * 3 + 2] = acc[2];
+                if constexpr (kNoted) notes.finish(broken, r.dscale);
                 active = false;
             }
         }
@@ -1179,71 +1342,6 @@ using ShadeSharedProbe = ShadeShared<1, true>;
 static_assert(offsetof(ShadeSharedProbe, who) == sizeof(int32_t) * kQueue * kMarchThreads,
               "the record list runs from ShadeShared::leaf into ShadeShared::who");
 
-// Workspace of the replaying backward: chunks of kChunkRecords records of 3 float2 (leaf and step
-// length, density and first sigmoid, the other two sigmoids) followed by one float2 whose x
-// holds the index of the ray's next chunk.  Ray number i starts in chunk i; further chunks come
-// from the rest of the workspace, of which a wavefront takes a stock of 64 chunks at a time through
-// one atomic counter (a heavy image tile needs hundreds, most tiles none); the lanes that need a
-// chunk in the same step are ranked by ballot.
-constexpr int kStampWords = 6;   // ray count; tree data, child; ray origins, directions; step size and threshold
-struct ReplaySpace {
-    float2* base;          // chunk c starts at base + c * kChunkFloat2
-    int64_t first_shared;  // chunks [0, first_shared) are the rays' first chunks
-    int64_t n_chunks;      // chunks [first_shared, n_chunks) are handed out in stocks of kChunkStock
-    unsigned long long* stocks_taken;   // counter of the stocks handed out (zero when the launch starts)
-    // kForwardNoted writes `stamp` (what the notes belong to) to stamp_at; replay_backward_kernel uses
-    // the notes only if it finds its own stamp there
-    unsigned long long* stamp_at;
-    unsigned long long stamp[kStampWords];
-    // one bit per ray (ray i: bit i % 64 of word i / 64).  replay_backward_kernel sets the bits of the
-    // rays it could not do from their notes; a launch of render_backward_kernel that is given the
-    // bitmap as `only` does those rays and no others
-    unsigned long long* undone;
-    const unsigned long long* only;
-};
-
-// whether the workspace carries the stamp this launch expects
-__device__ __forceinline__ bool stamp_matches(const ReplaySpace& ws) {
-    bool same = true;
-#pragma unroll
-    for (int i = 0; i < kStampWords; ++i) same = same && ws.stamp_at[i] == ws.stamp[i];
-    return same;
-}
-
-// The first ray at or after `next` (a wavefront-uniform ray number below `end`) whose 64-ray word of
-// the bitmap `only` is not zero, found 64 words at a time; a value >= end if there is none.
-__device__ __forceinline__ int64_t skip_clear_words(const unsigned long long* __restrict__ only, int64_t next,
-                                                    int64_t end, int lane) {
-    while (next < end) {
-        const int64_t word = next >> 6, last_word = (end - 1) >> 6;
-        const bool some = word + lane <= last_word && only[word + lane] != 0ull;
-        const unsigned long long nz = __ballot(some);
-        if (nz == 0ull) {
-            next = (word + kMarchThreads) << 6;
-            continue;
-        }
-        const int64_t first = (word + __builtin_ctzll(nz)) << 6;
-        if (first > next) next = first;
-        break;
-    }
-    return next;
-}
-
-// What a launch of render_backward_kernel does:
-//   kBackwardPlain   both marches walk the tree;
-//   kBackwardReplay  march 1 leaves notes in the workspace, march 2 replays them;
-//   kForwardNoted    march 1 only: it renders the ray (the output of render_forward_kernel, thresholds
-//                    and early stop included) and leaves the notes and their count in the workspace,
-//                    for replay_backward_kernel.
-enum BackwardMode { kBackwardPlain = 0, kBackwardReplay = 1, kForwardNoted = 2 };
-
-// Head of a ray's notes, kept in the spare floats of its first chunk (after the 15 records): the
-// link to the next chunk, the number of notes (-1: they did not fit; 0 also for a ray that misses
-// the tree), the ray's delta_scale (rt_kernel.cu:228) and 1.0f if the ray misses the tree, else 0.0f.
-constexpr int kChunkRecords = 15;
-constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
-constexpr int kHeadFloat2 = kChunkRecords * 3;          // float2 index of {link, count}, then {delta_scale, -}
-constexpr int kChunkStock = 64;   // further chunks a wavefront takes at a time (at most 64 lanes ask at once)
 
 // ------------------------------------------------------------------------------------------------
 // forward, walk and shading on two wavefronts
@@ -1261,10 +1359,10 @@ constexpr int kChunkStock = 64;   // further chunks a wavefront takes at a time 
 // A wavefront that finds nothing to do sleeps a few cycles and looks again; after kSpinLimit looks in a
 // row it gives up, so that a launch ends whatever happens.
 //
-// kNoted: the launch also leaves, for the backward pass, the notes render_backward_kernel<kForwardNoted>
-// leaves (same workspace, same format): every leaf with sigma > 0 of the whole ray, so the walk goes on
-// after the picture's early stop, and the colours of leaves below sigma_thresh are evaluated too; the
-// picture itself is composed as without notes.
+// kNoted: as in render_forward_kernel, the launch also leaves the notes of every ray for the backward
+// pass: every leaf with sigma > 0 of the whole ray, so the walk goes on after the picture's early stop,
+// and the colours of leaves below sigma_thresh are evaluated too; the picture itself is composed as
+// without notes.
 constexpr int kSplitThreads = 2 * kMarchThreads;
 constexpr int kRing = 8;               // leaves a lane's walk may be ahead of its shading (a power of two)
 constexpr int kSpinLimit = 1 << 22;
@@ -1323,10 +1421,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
                 out[slot * 3] = bg;
                 out[slot * 3 + 1] = bg;
                 out[slot * 3 + 2] = bg;
-                if constexpr (kNoted) {
-                    ws.base[slot * kChunkFloat2 + kHeadFloat2] = make_float2(0.0f, __int_as_float(0));   // no notes
-                    ws.base[slot * kChunkFloat2 + kHeadFloat2 + 1] = make_float2(0.0f, 1.0f);            // missed
-                }
+                if constexpr (kNoted) NoteTaker::missed(ws, slot);
             }
             if constexpr (P::kFormat == SVOX_FORMAT_SH) {
                 if (active) {
@@ -1396,18 +1491,9 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
     int spins = 0;
     // kNoted: the picture of a ray may be finished (early stop) while its notes go on
     bool painted = false;
-    // the notes of this lane's ray: their number, the chunk being written and the place in it
-    int rec_count = 0, rec_pos = 0;
-    bool rec_lost = false;   // the workspace ran out: this ray's backward pass will march
-    float2* rec_first = ws.base;
-    float2* rec_chunk = ws.base;
-    int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of further chunks (uniform)
-    if constexpr (kNoted) {
-        if (active) {
-            rec_first = ws.base + slot * kChunkFloat2;
-            rec_chunk = rec_first;
-        }
-    }
+    NoteTaker notes;
+    int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of chunks for notes (uniform)
+    if constexpr (kNoted) notes.begin(ws, active ? slot : 0);
     while (true) {
         const int32_t w = box_read(&box.written[lane]);
         asm volatile("" ::: "memory");   // the ring is read after the count, not before
@@ -1419,12 +1505,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
                 out[slot * 3 + 1] = fma_(light, bg, acc[1]);
                 out[slot * 3 + 2] = fma_(light, bg, acc[2]);
             }
-            if constexpr (kNoted) {
-                // the head of the notes: the count beside the link (written when the first chunk filled
-                // up), then delta_scale
-                ((float*)(rec_first + kHeadFloat2))[1] = __int_as_float(rec_lost || (w & kBrokenBit) ? -1 : rec_count);
-                rec_first[kHeadFloat2 + 1] = make_float2(r.dscale, 0.0f);
-            }
+            if constexpr (kNoted) notes.finish((w & kBrokenBit) != 0, r.dscale);
             active = false;
         }
         if (!__any(active)) break;
@@ -1484,44 +1565,8 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
                 light = take ? light * q_att[q] : light;
                 stopped = stopped || (take && light <= stop_thresh);
                 if constexpr (kNoted) {
-                    // the note of this leaf; lanes whose chunk is full take the next chunks of the
-                    // wavefront's stock, in lane order (as render_backward_kernel does)
-                    const bool note = active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
-                    const bool need = note && !rec_lost && rec_pos == kChunkRecords;
-                    const unsigned long long m = __ballot(need);
-                    if (m) {
-                        if (shared_next + __popcll(m) > shared_end) {
-                            unsigned long long t = 0;
-                            if (lane == 0) t = atomicAdd(ws.stocks_taken, 1ull);
-                            const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)t);
-                            const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(t >> 32));
-                            const int64_t stock = (int64_t)(((unsigned long long)hi << 32) | lo);
-                            shared_next = ws.first_shared + stock * kChunkStock;
-                            shared_end = shared_next + kChunkStock < ws.n_chunks ? shared_next + kChunkStock : ws.n_chunks;
-                            if (shared_next > shared_end) shared_next = shared_end;
-                        }
-                        const int64_t mine = shared_next + rank_in(m);
-                        if (need) {
-                            if (mine < shared_end) {
-                                rec_chunk[kHeadFloat2] = make_float2(__int_as_float((int32_t)mine), 0.0f);
-                                rec_chunk = ws.base + mine * kChunkFloat2;
-                                rec_pos = 0;
-                            } else {
-                                rec_lost = true;
-                            }
-                        }
-                        shared_next += __popcll(m);
-                    }
-                    if (note) {
-                        if (!rec_lost) {
-                            float2* e = rec_chunk + rec_pos * 3;
-                            e[0] = make_float2(__int_as_float(q_leaf[q]), q_dt[q]);
-                            e[1] = make_float2(q_sigma[q], q_s[q][0]);
-                            e[2] = make_float2(q_s[q][1], q_s[q][2]);
-                            rec_pos += 1;
-                        }
-                        rec_count += 1;
-                    }
+                    notes.take(ws, shared_next, shared_end, lane, active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f,
+                               q_leaf[q], q_dt[q], q_sigma[q], q_s[q]);
                 }
             }
             wave_lds_sync();   // the colours are read before the next list overwrites them
@@ -1551,7 +1596,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                                                                         SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
                                                                         float* __restrict__ grad_data,
-                                                                        ReplaySpace ws, float* __restrict__ out) {
+                                                                        ReplaySpace ws) {
     constexpr bool kReplay = kMode != kBackwardPlain;
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
@@ -1564,25 +1609,15 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     const float pad = opt.rgb_padding;
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     const float step = opt.step_size;
-    const float sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
 
     int64_t next = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)src.per_wave;
     const int64_t total = src.total();
     const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
-    if constexpr (kMode == kForwardNoted) {
-        if (blockIdx.x == 0 && lane < kStampWords) ws.stamp_at[lane] = ws.stamp[lane];
-    }
-
     enum { kMarch1 = 0, kMarch2 = 1, kReplaying = 2 };
     RayState<float> r;
     float go[3] = {0.f, 0.f, 0.f};
     float light = 1.0f, accum = 0.0f, tmin = 0.0f;
-    // kForwardNoted: the rendered colour, composited as render_forward_kernel does
-    float acc[3] = {0.f, 0.f, 0.f};
-    float light_f = 1.0f;
-    bool stopped_f = false;
-    int64_t out_slot = 0;
     bool active = false;
     int phase = kMarch1;
     // notes of march 1: total count, the chunk being written / read and the position in it
@@ -1610,16 +1645,9 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
-            if constexpr (kMode == kForwardNoted) {
-                acc[0] = acc[1] = acc[2] = 0.0f;
-                light_f = 1.0f;
-                stopped_f = false;
-                out_slot = slot;
-            } else {
-                go[0] = grad_out[slot * 3];
-                go[1] = grad_out[slot * 3 + 1];
-                go[2] = grad_out[slot * 3 + 2];
-            }
+            go[0] = grad_out[slot * 3];
+            go[1] = grad_out[slot * 3 + 1];
+            go[2] = grad_out[slot * 3 + 2];
             light = 1.0f;
             accum = 0.0f;
             tmin = r.t;
@@ -1633,12 +1661,6 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                 rec_first = ws.base + slot * kChunkFloat2;
                 rec_chunk = rec_first;
             }
-        } else if (kMode == kForwardNoted && slot >= 0) {
-            out[slot * 3] = bg;
-            out[slot * 3 + 1] = bg;
-            out[slot * 3 + 2] = bg;
-            ws.base[slot * kChunkFloat2 + kHeadFloat2] = make_float2(0.0f, __int_as_float(0));   // no notes
-            ws.base[slot * kChunkFloat2 + kHeadFloat2 + 1] = make_float2(0.0f, 1.0f);            // missed
         }
     };
     if constexpr (!kRefill) {
@@ -1705,9 +1727,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         }
         // ---- shade list (walking lanes only)
         const int n_entries = any_walk ? build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane, replaying) : 0;
-        // a round of kForwardNoted without a leaf to shade (most rounds of a ray pass through empty
-        // space) has nothing to compose and nothing to note
-        if (kMode != kForwardNoted || n_entries > 0) {
+        {
             wave_lds_sync();
             if (n_entries > 0) shade_entries<P, true>(tr.data, sh, n_entries, lane);
             wave_lds_sync();
@@ -1739,17 +1759,6 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                     const float* s = q_s[q];
                     const float total_color = q_total[q];
                     light *= att;
-                    if constexpr (kMode == kForwardNoted) {
-                        // rt_kernel.cu:278-313 on this leaf, as render_forward_kernel composes it
-                        if (!stopped_f && q_sigma[q] > sigma_thresh) {
-                            const float att_f = expf_fixed(-q_dt[q] * r.dscale * q_sigma[q]);
-                            const float weight_f = light_f * (1.0f - att_f);
-#pragma unroll
-                            for (int c = 0; c < 3; ++c) acc[c] = fma_(weight_f, fma_(s[c], d_rgb_pad, -pad), acc[c]);
-                            light_f *= att_f;
-                            if (light_f <= stop_thresh) stopped_f = true;
-                        }
-                    }
                     if (phase == kMarch1) {
                         accum = fma_(weight, total_color, accum);
                         if constexpr (kReplay) {
@@ -1812,33 +1821,15 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                         rec_count += 1;
                     }
                 }
-                if constexpr (kMode != kForwardNoted) records.append(emit, q_leaf[q], tmp2, g_sigma);
+                records.append(emit, q_leaf[q], tmp2, g_sigma);
             }
-            if constexpr (kMode != kForwardNoted) records.flush();
+            records.flush();
         }
         // ---- end of a march
         if (active) {
             if (replaying) {
                 rec_next += kQueue;
                 if (rec_next >= rec_count) active = false;
-            } else if (kMode == kForwardNoted && (broken || !(r.t < r.tmax))) {
-                // the ray's colour (rt_kernel.cu:306-319) and the count of its notes
-                if (stopped_f) {
-                    const float scale = (float)(1.0 / (1.0 - (double)light_f));
-#pragma unroll
-                    for (int c = 0; c < 3; ++c) acc[c] *= scale;
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 3; ++c) acc[c] = fma_(light_f, bg, acc[c]);
-                }
-                out[out_slot * 3] = acc[0];
-                out[out_slot * 3 + 1] = acc[1];
-                out[out_slot * 3 + 2] = acc[2];
-                // the head of the notes: the count beside the link (written when the first chunk filled
-                // up), then delta_scale
-                ((float*)(rec_first + kHeadFloat2))[1] = __int_as_float(rec_lost || broken ? -1 : rec_count);
-                rec_first[kHeadFloat2 + 1] = make_float2(r.dscale, 0.0f);
-                active = false;
             } else if (broken || !(r.t < r.tmax)) {
                 if (phase == kMarch1 && !broken) {
                     const float total_grad = (go[0] + go[1]) + go[2];
@@ -1863,7 +1854,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     }
 }
 
-// The backward pass from the notes render_backward_kernel<kForwardNoted> left: one lane per ray, no
+// The backward pass from the notes a noting forward kernel left (NoteTaker): one lane per ray, no
 // tree walk.  The notes of a ray (leaf, step length, sigma, the three sigmoids of every leaf with
 // sigma > 0) are read twice, five at a time: first for the sum the reference's first march forms
 // (rt_kernel.cu:358-419), then for the gradient records of its second march (:421-475), which the
@@ -1881,7 +1872,7 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     __shared__ ShadeShared<D, true> sh;
     const int lane = threadIdx.x;
-    // A wavefront takes 2^ray_shift consecutive rays (64, 32 or 16), one per lane from lane 0.  Adding a
+    // A wavefront takes 2^ray_shift consecutive rays (64 or 16), one per lane from lane 0.  Adding a
     // step's records is work of the whole wavefront, one record after the other; where the rays of a
     // wavefront are neighbours (the pixels of an image) they are all long or all short together, and
     // fewer of them per wavefront spread a long run of pixels over several wavefronts.
@@ -1898,13 +1889,11 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
         count = stamped ? __float_as_int(head.y) : -1;
         dscale = tail.x;
     }
-    // (the wavefront's part of the bitmap: a word, half a word or a quarter of one)
+    // (the wavefront's part of the bitmap: a word or a quarter of one)
     const unsigned long long undone = __ballot(count < 0);
     if (lane == 0) {
         if (ray_shift == 6)
             ws.undone[blockIdx.x] = undone;
-        else if (ray_shift == 5)
-            ((uint32_t*)ws.undone)[blockIdx.x] = (uint32_t)undone;
         else
             ((uint16_t*)ws.undone)[blockIdx.x] = (uint16_t)undone;
     }
@@ -2364,7 +2353,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
     }
 }
 
-// se_grad from the notes render_backward_kernel<kForwardNoted> left (taken with both thresholds at
+// se_grad from the notes a noting forward kernel left (NoteTaker; taken with both thresholds at
 // zero): one lane per ray, no tree walk.  The first pass over a ray's notes forms the residual and the
 // rendered colour as march 1 of se_grad_kernel does, the second pass the gradient and Hessian records
 // of its march 2, term by term the same values; the wavefront adds the records of its rays together,

@@ -343,7 +343,7 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
 #define SVOX_LAUNCH_FORWARD(ACCUM, REFILL)                                                                     \
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, ACCUM, REFILL>), dim3(blocks), \
                                                dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt,    \
-                                               *opt, (float*)out))
+                                               *opt, (float*)out, ReplaySpace{}))
             const bool refill = src.per_wave > kMarchThreads;
             if (!refill && !tree->weight_accum && use_split_forward(blocks, is_image_source(src))) {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false>), dim3(blocks),
@@ -407,14 +407,12 @@ bool carve_workspace(void* workspace, int64_t workspace_bytes, int64_t n_slots, 
     return true;
 }
 
-// mode: kBackwardPlain asks for the backward pass with whatever the workspace allows (replay if it is
-// large enough); kForwardNoted needs a usable workspace and the octree kernels, which noted_ok() tells
-// beforehand.
+// The backward pass, with whatever the workspace allows: march 2 replayed from notes of march 1 if it
+// is large enough, else two marches.
 template <class Source, typename T>
 void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, int out_dim,
                      const void* grad_out, void* grad_data, void* workspace, int64_t workspace_bytes,
-                     int64_t n_slots, hipStream_t stream, int mode = kBackwardPlain, void* out = nullptr,
-                     const NoteStamp* stamp = nullptr) {
+                     int64_t n_slots, hipStream_t stream) {
     const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
         const int D = fast_basis(tree, opt);
@@ -423,27 +421,15 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
             const Source dealt = dealt_out(src, blocks);
             // every ray owns one chunk; the wavefronts draw on what is left of the workspace
             ReplaySpace ws;
-            if (carve_workspace(workspace, workspace_bytes, n_slots, &ws) &&
-                zero_fill(ws.stocks_taken, 16, stream) == SVOX_OK) {
-                if (stamp) memcpy(ws.stamp, stamp->word, sizeof(ws.stamp));
-                if (mode == kBackwardPlain) mode = kBackwardReplay;
-            }
+            const bool replay = carve_workspace(workspace, workspace_bytes, n_slots, &ws) &&
+                                zero_fill(ws.stocks_taken, 16, stream) == SVOX_OK;
 #define SVOX_LAUNCH_BACKWARD(REFILL, MODE)                                                                      \
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, REFILL, MODE>), dim3(blocks),  \
                                                dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt,     \
-                                               *opt, (const float*)grad_out, (float*)grad_data, ws, (float*)out))
+                                               *opt, (const float*)grad_out, (float*)grad_data, ws))
             const bool refill = src.per_wave > kMarchThreads;
-            if (mode == kForwardNoted && !refill && use_split_forward(blocks, is_image_source(src))) {
-                // a launch that does not fill the GPU: the walk and the shading (with the notes) on two wavefronts
-                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, true>), dim3(blocks),
-                                                           dim3(kSplitThreads), 0, stream, march_tree(tree, opt), dealt,
-                                                           *opt, (float*)out, ws));
-                return;
-            }
-            if (mode == kBackwardReplay) {
+            if (replay) {
                 if (refill) { SVOX_LAUNCH_BACKWARD(true, kBackwardReplay); } else { SVOX_LAUNCH_BACKWARD(false, kBackwardReplay); }
-            } else if (mode == kForwardNoted) {
-                if (refill) { SVOX_LAUNCH_BACKWARD(true, kForwardNoted); } else { SVOX_LAUNCH_BACKWARD(false, kForwardNoted); }
             } else {
                 if (refill) { SVOX_LAUNCH_BACKWARD(true, kBackwardPlain); } else { SVOX_LAUNCH_BACKWARD(false, kBackwardPlain); }
             }
@@ -454,6 +440,49 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
     hipLaunchKernelGGL((render_backward_generic_kernel<T, Source>), dim3(blocks_for(items, kMarchThreads)),
                        dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (const T*)grad_out,
                        (T*)grad_data);
+}
+
+// The launch shape of the noting forward pass for the rays of `s`: that of a forward pass (a batch
+// source made for a backward pass gives its wavefronts more rays than the forward kernels like).
+template <typename T>
+BatchSource<T> noting_shape(BatchSource<T> s) {
+    s.per_wave = pick_per_wave(s.rays.n_rays, false);
+    return s;
+}
+template <typename T>
+ImageSource<T> noting_shape(const ImageSource<T>& s) { return s; }
+
+// The forward pass of a training step: the picture into `out` and, in the workspace, the notes of
+// every ray under `stamp`.  Needs a usable workspace and the octree kernels, which noted_ok() tells
+// beforehand.  A launch that does not fill the GPU runs on two wavefronts per 64 rays.
+template <class Source>
+int launch_noted(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, void* out,
+                 void* workspace, int64_t workspace_bytes, int64_t n_slots, const NoteStamp& stamp,
+                 hipStream_t stream) {
+    const int D = fast_basis(tree, opt);
+    const unsigned blocks = blocks_for(total_items_of(src), src.per_wave);
+    const Source dealt = dealt_out(src, blocks);
+    ReplaySpace ws;
+    if (D < 0 || !carve_workspace(workspace, workspace_bytes, n_slots, &ws))
+        return fail(SVOX_ERR_BAD_SHAPE, "notes asked for where they cannot be taken");
+    const int rc = zero_fill(ws.stocks_taken, 16, stream);
+    if (rc) return rc;
+    memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
+    const bool refill = src.per_wave > kMarchThreads;
+    if (!refill && use_split_forward(blocks, is_image_source(src))) {
+        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, true>), dim3(blocks),
+                                                   dim3(kSplitThreads), 0, stream, march_tree(tree, opt), dealt, *opt,
+                                                   (float*)out, ws));
+    } else if (refill) {
+        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, false, true, true>), dim3(blocks),
+                                                   dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt, *opt,
+                                                   (float*)out, ws));
+    } else {
+        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, false, false, true>), dim3(blocks),
+                                                   dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt, *opt,
+                                                   (float*)out, ws));
+    }
+    return SVOX_OK;
 }
 
 // The device address of `scratch` on the current device, looked up once per device (every GPU holds
@@ -530,7 +559,7 @@ int se_grad_prepare(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, void
 // wavefronts that look after the rays of a batch that replay_backward_kernel leaves undone (normally none)
 constexpr int kUndoneWaves = 256;
 
-// Can notes be taken (kForwardNoted) and used (replay_backward_kernel)?  The octree kernels, a forward
+// Can notes be taken (launch_noted) and used (replay_backward_kernel)?  The octree kernels, a forward
 // pass whose threshold does not admit leaves the backward pass ignores, no weight accumulator, and a
 // workspace with a chunk for every ray.
 bool noted_ok(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, int64_t n_slots, void* workspace,
@@ -558,12 +587,12 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
                                int64_t n_slots, const NoteStamp& stamp, hipStream_t stream) {
     const int D = fast_basis(tree, opt);
     // rays per wavefront of the replay: 16 for the pixels of images (neighbours, long together), 64 for ray
-    // batches (SVOX_REPLAY_SHIFT = 4, 5 or 6 overrides)
+    // batches (SVOX_REPLAY_SHIFT = 4 or 6 overrides)
     static const int forced_shift = [] {
         const char* e = getenv("SVOX_REPLAY_SHIFT");
         return e ? atoi(e) : -1;
     }();
-    const int ray_shift = forced_shift >= 4 && forced_shift <= 6 ? forced_shift : (is_image_source(all) ? 4 : 6);
+    const int ray_shift = forced_shift == 4 || forced_shift == 6 ? forced_shift : (is_image_source(all) ? 4 : 6);
     const unsigned waves = blocks_for(n_slots, 1 << ray_shift);
     ReplaySpace ws;
     carve_workspace(workspace, workspace_bytes, n_slots, &ws);
@@ -578,13 +607,11 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
     if (rest.per_wave > kMarchThreads) {
         SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, true, kBackwardPlain>), dim3(blocks),
                                                    dim3(kMarchThreads), 0, stream, march_tree(tree, opt), rest, *opt,
-                                                   (const float*)grad_output, (float*)grad_data_out, only,
-                                                   (float*)nullptr));
+                                                   (const float*)grad_output, (float*)grad_data_out, only));
     } else {
         SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, false, kBackwardPlain>), dim3(blocks),
                                                    dim3(kMarchThreads), 0, stream, march_tree(tree, opt), rest, *opt,
-                                                   (const float*)grad_output, (float*)grad_data_out, only,
-                                                   (float*)nullptr));
+                                                   (const float*)grad_output, (float*)grad_data_out, only));
     }
     return check_launch("volume_render_backward_noted");
 }
@@ -598,9 +625,9 @@ int se_grad_from_notes(const SvoxTreeSpec* tree, const Source& all, const Source
                        const void* color_ref, void* color_out, void* grad, void* hess, void* workspace,
                        int64_t workspace_bytes, int64_t n_slots, const NoteStamp& stamp, hipStream_t stream) {
     const int D = fast_basis(tree, opt);
-    launch_backward<Source, float>(tree, all, opt, 3, nullptr, nullptr, workspace, workspace_bytes, n_slots, stream,
-                                   kForwardNoted, color_out, &stamp);
-    int rc = check_launch("se_grad");
+    int rc = launch_noted(tree, noting_shape(all), opt, color_out, workspace, workspace_bytes, n_slots, stamp, stream);
+    if (rc) return rc;
+    rc = check_launch("se_grad");
     if (rc) return rc;
     ReplaySpace ws;
     carve_workspace(workspace, workspace_bytes, n_slots, &ws);
@@ -742,9 +769,9 @@ int svox_volume_render_noted(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
     if (!noted_ok(tree, opt, rays->n_rays, workspace, workspace_bytes))
         return svox_volume_render(tree, rays, opt, out, stream);
     const NoteStamp stamp = stamp_of(tree, rays, opt);
-    launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays, true), opt, od, nullptr, nullptr,
-                                               workspace, workspace_bytes, rays->n_rays, (hipStream_t)stream,
-                                               kForwardNoted, out, &stamp);
+    rc = launch_noted(tree, batch_source<float>(rays, false), opt, out, workspace, workspace_bytes, rays->n_rays, stamp,
+                      (hipStream_t)stream);
+    if (rc) return rc;
     return check_launch("volume_render_noted");
 }
 
@@ -790,9 +817,9 @@ int svox_volume_render_images_noted(const SvoxTreeSpec* tree, const SvoxCameraSp
     if (!noted_ok(tree, opt, n_slots, workspace, workspace_bytes))
         return svox_volume_render_images(tree, cam, n_images, pose_stride, opt, out, stream);
     const NoteStamp stamp = stamp_of_image(tree, cam, n_images, opt);
-    launch_backward<ImageSource<float>, float>(tree, image_source<float>(cam, n_images, pose_stride), opt, od, nullptr,
-                                               nullptr, workspace, workspace_bytes, n_slots, (hipStream_t)stream,
-                                               kForwardNoted, out, &stamp);
+    rc = launch_noted(tree, image_source<float>(cam, n_images, pose_stride), opt, out, workspace, workspace_bytes,
+                      n_slots, stamp, (hipStream_t)stream);
+    if (rc) return rc;
     return check_launch("volume_render_images_noted");
 }
 
