@@ -477,7 +477,13 @@ def main():
             qtree.data.grad = None
             qrend.render_persp(near, width=W, height=H, fx=fx).backward(qgo)
 
+        # (the renderer gives the notes of later steps more room when those of a step ran out: a few
+        # untimed steps let it settle, as the first steps of a training run would)
+        for _ in range(5):
+            near_train()
+            torch.cuda.synchronize()
         nrb_ms = ev_time(near_train, n=3)
+        near_notes = qrend.notes_budget.records_per_ray()
         nrm_ms = ev_time(lambda: C.volume_render_image_backward(qspec, ncam, qopt, qgo, workspace=False), n=3)
         qtree.data.grad = None
         qr_bytes = forward_bytes(qstats, W * H, Kq, 12)
@@ -494,6 +500,7 @@ def main():
             "backward_marching_ms": round(qrm_ms, 4),
             "close_up": {"workload": "the same tree from radius 1.2: about 12 pixels across a finest voxel",
                          "ms": round(nr_ms, 4), "forward_backward_ms": round(nrb_ms, 4),
+                         "notes_room_leaves_per_ray": near_notes,
                          "backward_marching_ms": round(nrm_ms, 4)},
         }
         if not args.no_cpu:

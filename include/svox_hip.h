@@ -255,6 +255,15 @@ int svox_volume_render_images_backward_noted(const SvoxTreeSpec* tree, const Svo
                                              int64_t workspace_bytes, void* stream);
 int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray);
 
+/* No counterpart in the reference.  How full a workspace of notes ran: after a call that takes notes
+ * (svox_volume_render_noted, svox_volume_render_images_noted, the _ws calls) the 64-bit word at byte
+ * *counter_offset of the workspace holds the number of 64-chunk stocks its wavefronts asked for
+ * beyond the rays' own chunks, and the workspace has *pool_stocks of them (rounded up).  A count at
+ * or above that number says the shared chunks ran out: some rays' notes are incomplete (those rays are
+ * marched by the backward pass: correct, slower) and a larger workspace would serve the same rays
+ * better.  Returns 0, or SVOX_ERR_BAD_SHAPE for a workspace too small to hold n_rays chunks. */
+int svox_notes_pool_info(int64_t n_rays, int64_t workspace_bytes, int64_t* counter_offset, int64_t* pool_stocks);
+
 /* The same for svox_volume_render_images_backward: one ray per pixel, n_rays = n_images * H * W. */
 int svox_volume_render_images_backward_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam,
                                           int32_t n_images, int64_t pose_stride,

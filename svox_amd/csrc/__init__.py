@@ -403,7 +403,7 @@ def volume_render_images_backward(tree, cam, opt, grad_output, workspace=True):
     return grad
 
 
-def volume_render_images_noted(tree, cam, opt):
+def volume_render_images_noted(tree, cam, opt, records_per_ray=None):
     """(images, notes): volume_render_images that also leaves the notes
     volume_render_images_backward_noted works from (see volume_render_noted).  cam.c2w is
     (n, 3, 4) / (n, 4, 4), or one pose (3, 4) / (4, 4), which gives (H, W, out_dim)."""
@@ -415,7 +415,7 @@ def volume_render_images_noted(tree, cam, opt):
     shape = (cspec.height, cspec.width, od) if single else (n, cspec.height, cspec.width, od)
     out = torch.empty(shape, dtype=tree.data.dtype, device=tree.data.device)
     copt = opt._pack()
-    ws, ws_bytes = _backward_workspace(tree, n * cspec.height * cspec.width)
+    ws, ws_bytes = _backward_workspace(tree, n * cspec.height * cspec.width, records_per_ray)
     marks = _attach_marks(spec, tree, opt, n * cspec.height * cspec.width)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_images_noted", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
@@ -461,14 +461,16 @@ BACKWARD_WORKSPACE_FREE_FRACTION = 0.25
 _ASK_DEVICE_ABOVE = 64 << 20   # smaller workspaces are taken without asking the device what is free
 
 
-def _backward_workspace(tree, n_rays):
+def _backward_workspace(tree, n_rays, records_per_ray=None):
     """(tensor, bytes) of the backward's workspace for n_rays rays, or (None, 0): for a tree that is
     not fp32, where the limits leave no room for 15 leaves per ray, and where the allocation fails
-    (the caller then runs without a workspace: same results, more marching)."""
+    (the caller then runs without a workspace: same results, more marching).  records_per_ray: room
+    for that many leaves per ray on average (default BACKWARD_RECORDS_PER_RAY), as far as the limits
+    allow."""
     if n_rays <= 0 or tree.data.dtype != torch.float32:
         return None, 0
     size_of = _abi.load_library().svox_volume_render_backward_workspace_bytes
-    per_ray = int(BACKWARD_RECORDS_PER_RAY)
+    per_ray = int(BACKWARD_RECORDS_PER_RAY if records_per_ray is None else records_per_ray)
     limit = BACKWARD_WORKSPACE_LIMIT
     if size_of(n_rays, per_ray) > _ASK_DEVICE_ABOVE:
         device = tree.data.device
@@ -528,9 +530,21 @@ def volume_render_backward_static(tree, rays, opt, grad_output, grad_data_out, a
     return grad_data_out
 
 
-def volume_render_noted(tree, rays, opt):
+def notes_pool_use(notes, n_rays):
+    """(counter, pool) of the notes a noted forward pass left for n_rays rays: `counter` is a
+    one-element int64 view into `notes` (on the device) that holds how many 64-chunk stocks the pass
+    asked for beyond the rays' own chunks, `pool` how many the workspace had.  counter >= pool: the
+    workspace ran out and some rays will be marched by the backward pass."""
+    offset, pool = ctypes.c_int64(0), ctypes.c_int64(0)
+    _call("svox_notes_pool_info", int(n_rays), notes.numel() * notes.element_size(), ctypes.byref(offset),
+          ctypes.byref(pool))
+    return notes.view(torch.int64)[offset.value // 8: offset.value // 8 + 1], int(pool.value)
+
+
+def volume_render_noted(tree, rays, opt, records_per_ray=None):
     """(out, notes): volume_render, which in the same march leaves in `notes` (a workspace tensor, or
     None where the library cannot take notes) what volume_render_backward_noted needs of the rays.
+    records_per_ray: room for that many leaves per ray on average (default BACKWARD_RECORDS_PER_RAY).
     No counterpart in the reference: it is what an autograd function keeps between forward and
     backward."""
     spec = _pack_tree(tree, rays.origins.dtype if isinstance(rays.origins, torch.Tensor) else None)
@@ -538,7 +552,7 @@ def volume_render_noted(tree, rays, opt):
     od = _render_out_dim(spec, opt)
     out = torch.empty((rspec.n_rays, od), dtype=rays.origins.dtype, device=rays.origins.device)
     copt = opt._pack()
-    ws, ws_bytes = _backward_workspace(tree, rspec.n_rays)
+    ws, ws_bytes = _backward_workspace(tree, rspec.n_rays, records_per_ray)
     marks = _attach_marks(spec, tree, opt, rspec.n_rays)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_noted", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),

@@ -897,6 +897,18 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
                                           stream);
 }
 
+int svox_notes_pool_info(int64_t n_rays, int64_t workspace_bytes, int64_t* counter_offset, int64_t* pool_stocks) {
+    if (!counter_offset || !pool_stocks) return fail(SVOX_ERR_NULL_POINTER, "svox_notes_pool_info: NULL output");
+    ReplaySpace ws;
+    // (any 16-byte aligned address does for the arithmetic)
+    char* const base = (char*)(uintptr_t)4096;
+    if (!carve_workspace(base, workspace_bytes, n_rays, &ws))
+        return fail(SVOX_ERR_BAD_SHAPE, "svox_notes_pool_info: the workspace does not hold a chunk per ray");
+    *counter_offset = (int64_t)((char*)ws.stocks_taken - base);
+    *pool_stocks = (ws.n_chunks - ws.first_shared + kChunkStock - 1) / kChunkStock;
+    return SVOX_OK;
+}
+
 int64_t svox_volume_render_backward_workspace_bytes(int64_t n_rays, int32_t records_per_ray) {
     if (n_rays <= 0 || records_per_ray <= 0) return 0;
     const int64_t chunks_per_ray = (records_per_ray + kChunkRecords - 1) / kChunkRecords;

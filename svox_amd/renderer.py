@@ -44,6 +44,56 @@ def _wants_notes(data):
     return KEEP_NOTES and torch.is_grad_enabled() and data.requires_grad
 
 
+class NotesBudget:
+    """How much room per ray the notes of a renderer's forward passes get.  It starts at
+    csrc.BACKWARD_RECORDS_PER_RAY leaves per ray; a pass whose notes ran out of room (its rays are then
+    marched by the backward pass: correct, but the noting was for nothing) doubles the room of the
+    passes after it, up to MAX_FACTOR times the start (and to the memory limits of
+    csrc._backward_workspace); passes that use less than a quarter of their room halve it again.
+
+    Nothing here waits for the GPU: the counter a pass leaves is copied to pinned memory behind the
+    pass, and looked at by a later pass only once the copy has arrived."""
+
+    MAX_FACTOR = 16
+
+    def __init__(self):
+        self.factor = 1
+        self._pending = None      # (pinned int64[1], event, pool stocks) of the last pass looked after
+        self._landing = None      # the pinned buffer, allocated on first use
+
+    def records_per_ray(self):
+        self._settle()
+        return int(_C.BACKWARD_RECORDS_PER_RAY) * self.factor
+
+    def _settle(self):
+        if self._pending is None:
+            return
+        landing, event, pool = self._pending
+        if not event.query():
+            return
+        self._pending = None
+        self.adjust(int(landing[0]), pool)
+
+    def adjust(self, asked, pool):
+        """One observation: `asked` stocks of chunks were asked for, the workspace had `pool`."""
+        if asked > 0 and asked >= pool:
+            self.factor = min(self.factor * 2, self.MAX_FACTOR)
+        elif asked * 4 < pool and self.factor > 1:
+            self.factor //= 2
+
+    def observe(self, notes, n_rays):
+        """Called right after the launch of a noted forward pass (on the current stream)."""
+        if notes is None or self._pending is not None:
+            return
+        counter, pool = _C.notes_pool_use(notes, n_rays)
+        if self._landing is None:
+            self._landing = torch.empty(1, dtype=torch.int64, pin_memory=True)
+        self._landing.copy_(counter, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        self._pending = (self._landing, event, pool)
+
+
 class _VolumeRenderFunction(torch.autograd.Function):
     """svox/renderer.py:57-72.  The specs are kept on ctx as plain attributes, so the backward
     pass sees the tree as it is when backward runs.
@@ -54,19 +104,21 @@ class _VolumeRenderFunction(torch.autograd.Function):
     the two passes (their version counters tell), the backward pass marches as the reference does."""
 
     @staticmethod
-    def forward(ctx, data, tree, rays, opt, keep_notes=False):
+    def forward(ctx, data, tree, rays, opt, keep_notes=False, budget=None):
         ctx.tree, ctx.rays, ctx.opt = tree, rays, opt
         ctx.notes = None
         ctx.versions = _versions(tree, rays)
         if keep_notes:
-            out, ctx.notes = _C.volume_render_noted(tree, rays, opt)
+            out, ctx.notes = _C.volume_render_noted(tree, rays, opt, budget.records_per_ray() if budget else None)
+            if budget:
+                budget.observe(ctx.notes, int(rays.origins.shape[0]))
             return out
         return _C.volume_render(tree, rays, opt)
 
     @staticmethod
     def backward(ctx, grad_out):
         if not ctx.needs_input_grad[0]:
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         notes, ctx.notes = ctx.notes, None
         if ctx.versions != _versions(ctx.tree, ctx.rays):
             # the tree or the rays were written to since the forward pass: its notes and the marks of
@@ -76,7 +128,7 @@ class _VolumeRenderFunction(torch.autograd.Function):
             grad = _C.volume_render_backward_noted(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous(), notes)
         else:
             grad = _C.volume_render_backward(ctx.tree, ctx.rays, ctx.opt, grad_out.contiguous())
-        return grad, None, None, None, None
+        return grad, None, None, None, None, None
 
 
 def _tree_versions(tree):
@@ -97,24 +149,28 @@ class _VolumeRenderImageFunction(torch.autograd.Function):
     rendered in one launch.  Notes are kept between the passes as in _VolumeRenderFunction."""
 
     @staticmethod
-    def forward(ctx, data, tree, cam, opt, keep_notes=False):
+    def forward(ctx, data, tree, cam, opt, keep_notes=False, budget=None):
         ctx.tree, ctx.cam, ctx.opt = tree, cam, opt
         ctx.notes = None
         ctx.versions = _image_versions(tree, cam)
         if keep_notes:
-            out, ctx.notes = _C.volume_render_images_noted(tree, cam, opt)
+            out, ctx.notes = _C.volume_render_images_noted(tree, cam, opt,
+                                                           budget.records_per_ray() if budget else None)
+            if budget:
+                n_images = 1 if cam.c2w.dim() == 2 else int(cam.c2w.shape[0])
+                budget.observe(ctx.notes, n_images * cam.height * cam.width)
             return out
         return _C.volume_render_image(tree, cam, opt) if cam.c2w.dim() == 2 else _C.volume_render_images(tree, cam, opt)
 
     @staticmethod
     def backward(ctx, grad_out):
         if not ctx.needs_input_grad[0]:
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         notes, ctx.notes = ctx.notes, None
         if ctx.versions != _image_versions(ctx.tree, ctx.cam):
             notes, ctx.tree.child_marks = None, None     # as in _VolumeRenderFunction.backward
         grad = _C.volume_render_images_backward_noted(ctx.tree, ctx.cam, ctx.opt, grad_out.contiguous(), notes)
-        return grad, None, None, None, None
+        return grad, None, None, None, None, None
 
 
 _VolumeRenderImagesFunction = _VolumeRenderImageFunction
@@ -153,9 +209,12 @@ class VolumeRenderer(nn.Module):
     Memory and state beyond the reference's renderer (which holds nothing between calls):
 
     * A forward pass that will be differentiated (gradient mode on, `tree.data.requires_grad`) keeps
-      notes of the leaves its rays met until `backward()` has run: 768 bytes per ray (30 leaves per ray
-      on average; 3.9 GB for eight 800x800 images), at most `csrc.BACKWARD_WORKSPACE_LIMIT` (4 GiB) and
-      at most a quarter of the device memory that is free at the time.  Where that leaves no room, or
+      notes of the leaves its rays met until `backward()` has run: 768 bytes per ray to begin with (30
+      leaves per ray on average; 3.9 GB for eight 800x800 images); a pass whose notes ran out of room
+      doubles the room of the next passes, up to 16 times, and passes that leave most of it unused
+      halve it again (`renderer.notes_budget`, a `NotesBudget`).  At most
+      `csrc.BACKWARD_WORKSPACE_LIMIT` (4 GiB) and at most a quarter of the device memory that is free
+      at the time.  Where that leaves no room, or
       the allocation fails, the pass runs without notes and the backward pass marches through the tree
       twice, as the reference does: same results, slower.  The noted forward pass follows every ray to
       its end (no early stop), so it is slower than a forward pass under `torch.no_grad()`.  The notes
@@ -190,6 +249,7 @@ class VolumeRenderer(nn.Module):
             ddim = tree.data_dim
             self._data_format = DataFormat("" if ddim == 4 else f"SH{(ddim - 1) // 3}")
         self.tree._weight_accum = None
+        self.notes_budget = NotesBudget()
 
     @property
     def data_format(self):
@@ -206,7 +266,7 @@ class VolumeRenderer(nn.Module):
         self._require_gpu(cuda, "VolumeRenderer.forward")
         return _VolumeRenderFunction.apply(self.tree.data, self.tree._spec(),
                                            _rays_spec_from_rays(rays), self._get_options(fast),
-                                           _wants_notes(self.tree.data))
+                                           _wants_notes(self.tree.data), self.notes_budget)
 
     def render_persp(self, c2w, width=800, height=800, fx=1111.111, fy=None, cuda=True, fast=False):
         """Render a pinhole image -> (height, width, rgb_dim).  c2w is (3, 4) or (4, 4), OpenGL
@@ -221,7 +281,7 @@ class VolumeRenderer(nn.Module):
                                 width, height, fx, fy)
         fn = _VolumeRenderImagesFunction if c2w.dim() == 3 else _VolumeRenderImageFunction
         return fn.apply(self.tree.data, self.tree._spec(), cam, self._get_options(fast),
-                        _wants_notes(self.tree.data))
+                        _wants_notes(self.tree.data), self.notes_budget)
 
     def se_grad(self, rays, colors):
         """Rendered colour plus gradient and Hessian diagonal (Gauss-Newton: squared Jacobian rows) of

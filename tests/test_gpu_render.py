@@ -459,6 +459,45 @@ def test_noted_forward_and_backward_from_notes(gpu, oracle_mod, fmt, fast, persi
         C.set_debug_flags(0)
 
 
+def test_notes_budget_follows_the_scene(gpu, oracle_mod):
+    """Rays through a dense tree meet more leaves with density than the starting room for notes holds:
+    the first training step loses notes (those rays are marched: same gradient), the renderer gives
+    the next steps more room until nothing is lost, and takes it back for rays that need none."""
+    tree = synth.dense_tree(5, "SH4", seed=3, sigma="lognormal", coeff_std=0.5, zero_fraction=0.0)
+    rays = synth.sphere_rays(3000, seed=5)
+    opt = options(tree, step_size=1e-3)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    go = torch.randn(3000, 3, generator=torch.Generator().manual_seed(2)) * 1e-2
+    want, slack = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go,
+                                                    n_threads=8, want_slack=True)
+    dev = on_gpu(tree, gpu)
+    dev.data.requires_grad_(True)
+    r = svox.VolumeRenderer(dev, step_size=1e-3)
+    dev_rays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu))
+    factors, asked = [], []
+    for _ in range(5):
+        dev.data.grad = None
+        factors.append(r.notes_budget.factor)
+        r(dev_rays).backward(go.to(gpu))
+        torch.cuda.synchronize()
+        err, ok = grad_close(dev.data.grad.cpu().numpy(), want, slack=slack)
+        assert ok, (factors, err)
+    factors.append(r.notes_budget.records_per_ray() // C.BACKWARD_RECORDS_PER_RAY)
+    assert factors[0] == 1 and factors[-1] > 1, factors
+    assert factors[-1] == factors[-2], factors            # it settles
+    # with the room it settled on nothing is lost any more
+    out, notes = C.volume_render_noted(dev._spec(), rays_spec(rays, gpu), opt, r.notes_budget.records_per_ray())
+    counter, pool = C.notes_pool_use(notes, 3000)
+    assert 0 < int(counter.cpu()[0]) < pool
+    # rays that miss the tree need no room: the budget goes back to where it started
+    away = svox.Rays(dev_rays.origins + 5.0, dev_rays.dirs, dev_rays.viewdirs)
+    for _ in range(6):
+        dev.data.grad = None
+        r(away).backward(go.to(gpu))
+        torch.cuda.synchronize()
+    assert r.notes_budget.records_per_ray() == C.BACKWARD_RECORDS_PER_RAY
+
+
 def test_autograd_uses_notes_and_marches_again_after_a_write(gpu, oracle_mod):
     """renderer(rays).backward(): the gradient from the forward pass's notes equals the oracle's; if
     tree.data is written to between the two passes, the backward pass sees the tree as it then is

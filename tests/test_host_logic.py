@@ -345,3 +345,42 @@ def test_tree_keeps_marks_only_while_it_is_unchanged():
     assert C._marks_for_this_call(spec, opt, 10) is None
     spec.child_marks = torch.zeros_like(tree.child)
     assert C._marks_for_this_call(spec, opt, 10 ** 9) is None       # the caller brought marks
+
+
+def test_notes_budget_grows_when_the_notes_ran_out_and_shrinks_when_they_are_not_used():
+    from svox_amd.renderer import NotesBudget
+    from svox_amd import csrc as C
+    b = NotesBudget()
+    base = int(C.BACKWARD_RECORDS_PER_RAY)
+    assert b.records_per_ray() == base
+    b.adjust(asked=10, pool=10)          # every stock handed out: the notes ran out (or just fitted)
+    assert b.factor == 2 and b.records_per_ray() == 2 * base
+    b.adjust(asked=40, pool=30)
+    assert b.factor == 4
+    b.adjust(asked=20, pool=30)          # fits, and more than a quarter is used: stay
+    assert b.factor == 4
+    b.adjust(asked=7, pool=30)           # under a quarter: halve
+    assert b.factor == 2
+    b.adjust(asked=0, pool=30)
+    b.adjust(asked=0, pool=30)
+    assert b.factor == 1                 # never below the start
+    for _ in range(10):
+        b.adjust(asked=99, pool=1)
+    assert b.factor == NotesBudget.MAX_FACTOR
+
+
+def test_notes_pool_info_matches_the_documented_workspace_layout():
+    import ctypes
+    from svox_amd.csrc import _abi
+    lib = _abi.load_library()
+    n = 1000
+    nbytes = int(lib.svox_volume_render_backward_workspace_bytes(n, 30))
+    offset, pool = ctypes.c_int64(), ctypes.c_int64()
+    assert lib.svox_notes_pool_info(n, nbytes, ctypes.byref(offset), ctypes.byref(pool)) == 0
+    # chunks, then one bit per ray (rounded to 16 bytes), then 256 bytes whose second half starts with the counter
+    chunks = (nbytes - 256 - 16 * ((n + 127) // 128)) // 384
+    assert chunks == 2 * n
+    assert offset.value == chunks * 384 + 16 * ((n + 127) // 128) + 128 and offset.value % 8 == 0
+    assert pool.value == (chunks - n + 63) // 64
+    assert lib.svox_notes_pool_info(n, 384 * (n - 1), ctypes.byref(offset), ctypes.byref(pool)) == -2
+    assert lib.svox_notes_pool_info(n, nbytes, None, ctypes.byref(pool)) == -1
