@@ -61,6 +61,15 @@ class NotesBudget:
         self._pending = None      # (pinned int64[1], event, pool stocks) of the last pass looked after
         self._landing = None      # the pinned buffer, allocated on first use
 
+    def __getstate__(self):
+        # (a copy or a pickle of the renderer takes the figure along, not the buffer and the event)
+        return {"factor": self.factor}
+
+    def __setstate__(self, state):
+        self.factor = state["factor"]
+        self._pending = None
+        self._landing = None
+
     def records_per_ray(self):
         self._settle()
         return int(_C.BACKWARD_RECORDS_PER_RAY) * self.factor

@@ -367,6 +367,9 @@ def test_notes_budget_grows_when_the_notes_ran_out_and_shrinks_when_they_are_not
     for _ in range(10):
         b.adjust(asked=99, pool=1)
     assert b.factor == NotesBudget.MAX_FACTOR
+    import copy
+    import pickle
+    assert copy.deepcopy(b).factor == b.factor and pickle.loads(pickle.dumps(b)).factor == b.factor
 
 
 def test_notes_pool_info_matches_the_documented_workspace_layout():
