@@ -388,14 +388,17 @@ def main():
             torch.cuda.synchronize()
             return (time.perf_counter() - t0) * 1e3 / n
 
+        itarget = torch.rand(H, W, 3, generator=g).to(dev)
         fwd_bwd["image_pose"] = {
             "forward_backward_ms": round(timed(image_step), 3),
+            "se_grad_persp_ms": round(timed(lambda: renderer.se_grad_persp(poses[0], itarget, width=W, height=H,
+                                                                           fx=fx)), 3),
             "backward_marching_ms": round(timed(lambda: C.volume_render_image_backward(spec, icam, opt, igo,
                                                                                         workspace=False)), 3),
             "note": f"render_persp of pose 0 ({W}x{H}) and its gradient through autograd; then the stateless "
                     "backward operator without a workspace (zero-fill of the gradient included in both)"}
         tree.data.grad = None
-        del igo
+        del igo, itarget
         log(f"[bench] fwd+bwd {fwd_bwd}")
 
     # ---------------------------------------------------------------- point queries (dense 128^3 SH9 tree)

@@ -2370,25 +2370,30 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
                                                                        float* __restrict__ color_out,
                                                                        float* __restrict__ grad_data,
                                                                        float* __restrict__ hess_data,
-                                                                       ReplaySpace ws) {
+                                                                       ReplaySpace ws, int ray_shift) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     constexpr bool kRgba = P::kFormat == SVOX_FORMAT_RGBA;
     __shared__ float basis_rows[kMarchThreads * D];
     __shared__ float resid_rows[kMarchThreads * 3];
     __shared__ int32_t l_leaf[kSeRecordCap];
-    __shared__ float l_gs[kSeRecordCap], l_hs[kSeRecordCap], l_gci[kSeRecordCap * 3];
+    // per record four gradient factors (the three colour factors, then the density term) and the
+    // density term of the Hessian
+    __shared__ float l_factor[kSeRecordCap * 4], l_hs[kSeRecordCap];
     __shared__ uint8_t l_owner[kSeRecordCap];
     __shared__ GroupScratch group;
     const int lane = threadIdx.x;
-    const int64_t ray = blockIdx.x * (int64_t)kMarchThreads + lane;
+    // 2^ray_shift consecutive rays per wavefront (64, or 16 for the pixels of images), as in
+    // replay_backward_kernel
+    const int64_t ray = ((int64_t)blockIdx.x << ray_shift) + lane;
+    const bool seated = lane < (1 << ray_shift);
     const bool stamped = stamp_matches(ws);
     const float2* first = ws.base + ray * kChunkFloat2;
     int count = 0;
     int32_t first_link = 0;
     float dscale = 0.0f;
     bool missed = true;
-    if (ray < src.n_slots()) {
+    if (seated && ray < src.n_slots()) {
         const float2 head = first[kHeadFloat2], tail = first[kHeadFloat2 + 1];
         first_link = __float_as_int(head.x);
         count = stamped ? __float_as_int(head.y) : -1;
@@ -2396,7 +2401,12 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
         missed = tail.y != 0.0f;
     }
     const unsigned long long undone = __ballot(count < 0);
-    if (lane == 0) ws.undone[blockIdx.x] = undone;
+    if (lane == 0) {
+        if (ray_shift == 6)
+            ws.undone[blockIdx.x] = undone;
+        else
+            ((uint16_t*)ws.undone)[blockIdx.x] = (uint16_t)undone;
+    }
     const bool hit = count >= 0 && !missed;   // the rays this launch answers
     const bool work = hit && count > 0;
     if (!__any(hit)) return;
@@ -2428,28 +2438,78 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
         wave_lds_sync();
         // where enough records share a leaf, the records of a leaf are brought together first
         const bool grouped = group_by_leaf(group, merge, l_leaf, n, lane);
-        add_records_by_leaf<K, 2>(
-            n, lane, grouped ? group.leaf : l_leaf,
-            // element e of a record: colour coefficient (c, i) or, last, the density
-            [&](int at, int e, float* t) {
-                const int rec = grouped ? group.order[at] : at;
+        auto emit = [&](int32_t leaf, int e, const float* sum) {
+            const int64_t at = (int64_t)leaf * K + e;
+            atomicAdd(grad_data + at, sum[0]);
+            atomicAdd(hess_data + at, sum[1]);
+        };
+        if constexpr (K > kMarchThreads / 2) {
+            // One record at a time, lane e on element e; place, leaf and owner of the records are held
+            // in registers, record r by lane r, and handed round by readlane, so that the LDS reads of a
+            // record have their addresses from scalars and those of four records are in flight together
+            // (RecordList::add_held).
+            const bool mine = lane < n;
+            int my_rec = mine ? (grouped ? group.order[lane] : lane) : 0;
+            int my_leaf = l_leaf[my_rec];
+            int my_owner = l_owner[my_rec];
+            asm volatile("" : "+v"(my_rec), "+v"(my_leaf), "+v"(my_owner));   // (set in every lane before any readlane)
+            constexpr int kBlock = 4;
+            for (int e = lane; e < K; e += kMarchThreads) {
                 const int c = kRgba ? e : e / D;
-                if (c < 3) {
-                    const int owner = l_owner[rec];
-                    const float v = l_gci[rec * 3 + c];
-                    const float gw = kRgba ? v : basis_rows[owner * D + (e - c * D)] * v;
-                    t[0] = gw * resid_rows[owner * 3 + c];
-                    t[1] = gw * gw;
-                } else {
-                    t[0] = l_gs[rec];
-                    t[1] = l_hs[rec];
+                const int i = kRgba ? 0 : e - c * D;
+                const int cc = c < 3 ? c : 0;
+                int32_t cur = -1;
+                float acc[2] = {0.0f, 0.0f};
+                for (int at = 0; at < n; at += kBlock) {
+                    int32_t leaf[kBlock];
+                    float f[kBlock], b[kBlock], rs[kBlock], hs[kBlock];
+#pragma unroll
+                    for (int u = 0; u < kBlock; ++u) {
+                        const int a = at + u < n ? at + u : n - 1;   // (past the end: the last record again, unused)
+                        const int rec = __builtin_amdgcn_readlane(my_rec, a);
+                        const int owner = __builtin_amdgcn_readlane(my_owner, a);
+                        leaf[u] = __builtin_amdgcn_readlane(my_leaf, a);
+                        f[u] = l_factor[rec * 4 + c];
+                        b[u] = kRgba ? 1.0f : basis_rows[owner * D + i];
+                        rs[u] = resid_rows[owner * 3 + cc];
+                        hs[u] = l_hs[rec];
+                    }
+#pragma unroll
+                    for (int u = 0; u < kBlock; ++u) {
+                        if (at + u < n) {
+                            if (leaf[u] != cur) {
+                                if (cur >= 0) emit(cur, e, acc);
+                                cur = leaf[u];
+                                acc[0] = acc[1] = 0.0f;
+                            }
+                            const float gw = kRgba ? f[u] : b[u] * f[u];
+                            acc[0] += c < 3 ? gw * rs[u] : f[u];
+                            acc[1] += c < 3 ? gw * gw : hs[u];
+                        }
+                    }
                 }
-            },
-            [&](int32_t leaf, int e, const float* sum) {
-                const int64_t at = (int64_t)leaf * K + e;
-                atomicAdd(grad_data + at, sum[0]);
-                atomicAdd(hess_data + at, sum[1]);
-            });
+                if (cur >= 0) emit(cur, e, acc);
+            }
+        } else {
+            add_records_by_leaf<K, 2>(
+                n, lane, grouped ? group.leaf : l_leaf,
+                // element e of a record: colour coefficient (c, i) or, last, the density
+                [&](int at, int e, float* t) {
+                    const int rec = grouped ? group.order[at] : at;
+                    const int c = kRgba ? e : e / D;
+                    if (c < 3) {
+                        const int owner = l_owner[rec];
+                        const float v = l_factor[rec * 4 + c];
+                        const float gw = kRgba ? v : basis_rows[owner * D + (e - c * D)] * v;
+                        t[0] = gw * resid_rows[owner * 3 + c];
+                        t[1] = gw * gw;
+                    } else {
+                        t[0] = l_factor[rec * 4 + 3];
+                        t[1] = l_hs[rec];
+                    }
+                },
+                emit);
+        }
         wave_lds_sync();
         n = 0;
     };
@@ -2464,11 +2524,11 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
             if (take) {
                 l_leaf[at] = leaf;
                 l_owner[at] = (uint8_t)lane;
-                l_gs[at] = g_sigma;
                 l_hs[at] = h_sigma;
-                l_gci[at * 3] = gci[0];
-                l_gci[at * 3 + 1] = gci[1];
-                l_gci[at * 3 + 2] = gci[2];
+                l_factor[at * 4] = gci[0];
+                l_factor[at * 4 + 1] = gci[1];
+                l_factor[at * 4 + 2] = gci[2];
+                l_factor[at * 4 + 3] = g_sigma;
             }
             const unsigned long long taken = __ballot(take);
             n += __popcll(taken);

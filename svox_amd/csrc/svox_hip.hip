@@ -579,6 +579,16 @@ NoteStamp stamp_of_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, in
     return stamp_of(tree, &as_rays, opt);
 }
 
+// log2 of the rays a wavefront of the replay kernels takes: 16 rays for the pixels of images (neighbours,
+// long together), 64 for ray batches (SVOX_REPLAY_SHIFT = 4 or 6 overrides)
+int replay_ray_shift(bool image) {
+    static const int forced_shift = [] {
+        const char* e = getenv("SVOX_REPLAY_SHIFT");
+        return e ? atoi(e) : -1;
+    }();
+    return forced_shift == 4 || forced_shift == 6 ? forced_shift : (image ? 4 : 6);
+}
+
 // The backward pass of `all` from the notes in the workspace: the rays with complete notes by
 // replay_backward_kernel, the others, which it marks in the bitmap, by two marches.
 template <class Source>
@@ -586,13 +596,7 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
                                const void* grad_output, void* grad_data_out, void* workspace, int64_t workspace_bytes,
                                int64_t n_slots, const NoteStamp& stamp, hipStream_t stream) {
     const int D = fast_basis(tree, opt);
-    // rays per wavefront of the replay: 16 for the pixels of images (neighbours, long together), 64 for ray
-    // batches (SVOX_REPLAY_SHIFT = 4 or 6 overrides)
-    static const int forced_shift = [] {
-        const char* e = getenv("SVOX_REPLAY_SHIFT");
-        return e ? atoi(e) : -1;
-    }();
-    const int ray_shift = forced_shift == 4 || forced_shift == 6 ? forced_shift : (is_image_source(all) ? 4 : 6);
+    const int ray_shift = replay_ray_shift(is_image_source(all));
     const unsigned waves = blocks_for(n_slots, 1 << ray_shift);
     ReplaySpace ws;
     carve_workspace(workspace, workspace_bytes, n_slots, &ws);
@@ -632,9 +636,10 @@ int se_grad_from_notes(const SvoxTreeSpec* tree, const Source& all, const Source
     ReplaySpace ws;
     carve_workspace(workspace, workspace_bytes, n_slots, &ws);
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
-    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_se_grad_kernel<P, Source>), dim3(blocks_for(n_slots, kMarchThreads)),
+    const int ray_shift = replay_ray_shift(is_image_source(all));
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_se_grad_kernel<P, Source>), dim3(blocks_for(n_slots, 1 << ray_shift)),
                                                dim3(kMarchThreads), 0, stream, all, *opt, (const float*)color_ref,
-                                               (float*)color_out, (float*)grad, (float*)hess, ws));
+                                               (float*)color_out, (float*)grad, (float*)hess, ws, ray_shift));
     rc = check_launch("se_grad");
     if (rc) return rc;
     launch_se_grad<Source, float>(tree, rest, opt, 3, color_ref, color_out, grad, hess, stream, ws.undone);
