@@ -1275,6 +1275,15 @@ struct RecordList {
         if (n == 0) return;
         wave_lds_sync();
         if (flush_grouped()) return;
+        if constexpr (kHeld) {
+            // long records: one at a time with its values handed round by readlane (measured on the
+            // marching backward of an 800x800 image: 2.55 -> 2.38 ms, with a workspace 2.07 -> 1.80 ms;
+            // for records of up to 32 scalars the flat form below is as fast)
+            add_held(nullptr);
+            wave_lds_sync();
+            n = 0;
+            return;
+        }
         const int total = n * K;
         for (int f = lane; f < total; f += kMarchThreads) {
             const int rec = f / K, e = f - rec * K;
