@@ -1067,6 +1067,9 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
 //               price is idle lanes where K does not divide 64.  Consecutive records of the same leaf
 //               are summed in registers and added once.  term(rec, e, t) gives the NV values of
 //               element e of record rec, emit(leaf, e, sum) adds them.
+// Records longer than half a wavefront (K > 32: one record at a time either way) are added by
+// RecordList::add_held in both forms: the by-record scheme with the values of a record handed round by
+// readlane instead of read through LDS one after the other.
 // Before either, group_by_leaf looks for leaves that several records of the list share; if enough do,
 // the list is put in an order that brings the records of a leaf together and added by record.
 
