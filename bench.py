@@ -202,7 +202,7 @@ def main():
         l2_misses = int(m.group(1)) if m else None
 
     roofline = {
-        "bound": "hbm", "kernel": "render_forward_kernel<OctreePolicy<SH,16>, ImageSource>",
+        "bound": "hbm", "kernel": "render_forward_split_kernel<OctreePolicy<SH,16>, ImageSource>",
         "launch": f"{args.poses} poses x {W}x{H} in one launch",
         "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
         "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": traffic,

@@ -308,11 +308,14 @@ unsigned blocks_for(int64_t items, int per_block) { return (unsigned)((items + p
 // Whether a forward launch of `blocks` 64-ray wavefronts takes render_forward_split_kernel (two
 // wavefronts per 64 rays: one walks, one shades).  It shortens the chain of a tile's longest ray, which
 // is what a launch that does not fill the GPU with heavy tiles waits for: measured on 800x800 images,
-// sparse 512^3 tree 0.42 -> 0.35 ms (one pose), 0.45 -> 0.41 (two), dense 128^3 tree 0.55 -> 0.38; where
-// every tile is heavy and the GPU full (four 1008x756 NDC poses, 48 384 tiles) it costs 5 %, and a
-// batch of 256 Ki unrelated rays 36 %.  SVOX_SPLIT_FORWARD=1 / 0 forces / forbids it;
+// sparse 512^3 tree 0.43 -> 0.34 ms (one pose), 0.62 -> 0.56 (four), 0.92 -> 0.87 (eight; with the
+// empty leaves marked 0.81 -> 0.77), sixteen poses equal; dense 128^3 tree 0.54 -> 0.37 (one), 0.84 ->
+// 0.75 (four).  Where every tile is heavy and the GPU full it costs: four 1008x756 NDC poses (47 628
+// tiles) 3 %, two of them 1 % (one gains 2 %), a batch of 256 Ki unrelated rays 33 %.  Hence: images of
+// up to 98 304 tiles (eight 800x800 poses are 80 000) -- but 16 384 under NDC, where every ray passes
+// through the tree --, ray batches of up to 128 Ki rays.  SVOX_SPLIT_FORWARD=1 / 0 forces / forbids it;
 // SVOX_SPLIT_BLOCKS sets the largest launch that takes it (experiments).
-bool use_split_forward(unsigned blocks, bool image) {
+bool use_split_forward(unsigned blocks, bool image, const SvoxRenderOptions* opt) {
     static const int forced = [] {
         const char* e = getenv("SVOX_SPLIT_FORWARD");
         return e ? atoi(e) : -1;
@@ -324,7 +327,8 @@ bool use_split_forward(unsigned blocks, bool image) {
     if (g_debug_flags & 12) return (g_debug_flags & 8) != 0;
     if (forced >= 0) return forced > 0;
     if (limit >= 0) return (long)blocks <= limit;
-    return blocks <= (image ? 24576u : 2048u);
+    if (!image) return blocks <= 2048u;
+    return blocks <= (opt->ndc_width > 0 ? 16384u : 98304u);
 }
 template <typename T>
 constexpr bool is_image_source(const ImageSource<T>&) { return true; }
@@ -345,7 +349,7 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
                                                dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt,    \
                                                *opt, (float*)out, ReplaySpace{}))
             const bool refill = src.per_wave > kMarchThreads;
-            if (!refill && !tree->weight_accum && use_split_forward(blocks, is_image_source(src))) {
+            if (!refill && !tree->weight_accum && use_split_forward(blocks, is_image_source(src), opt)) {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false>), dim3(blocks),
                                                            dim3(kSplitThreads), 0, stream, march_tree(tree, opt), dealt,
                                                            *opt, (float*)out, ReplaySpace{}));
@@ -469,7 +473,7 @@ int launch_noted(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOp
     if (rc) return rc;
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
     const bool refill = src.per_wave > kMarchThreads;
-    if (!refill && use_split_forward(blocks, is_image_source(src))) {
+    if (!refill && use_split_forward(blocks, is_image_source(src), opt)) {
         SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, true>), dim3(blocks),
                                                    dim3(kSplitThreads), 0, stream, march_tree(tree, opt), dealt, *opt,
                                                    (float*)out, ws));
