@@ -341,7 +341,7 @@ def main():
             "separate_calls": {
                 "value": round(B / (sep_ms * 1e-3) / 1e6, 3), "ms_per_step": round(sep_ms, 3),
                 "note": "volume_render + volume_render_backward + SGD update as independent calls (the backward "
-                        "marches, and replays its second march from a workspace of its own)"},
+                        "walks every ray once, taking notes in a workspace of its own, and forms the gradient from the notes)"},
             "samples_per_ray": round(train_stats["samples_bwd"] / B, 2),
             "positive_per_ray": round(train_stats["samples_bwd_pos"] / B, 2),
         }

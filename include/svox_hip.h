@@ -186,10 +186,10 @@ int svox_volume_render_backward(const SvoxTreeSpec* tree, const SvoxRaysSpec* ra
                                 void* grad_data_out, int32_t accumulate, void* stream);
 
 /* No counterpart in the reference.  svox_volume_render_backward with a workspace in device memory
- * (16-byte aligned, any contents, overwritten): while the first of the two marches of a ray passes
- * the leaves with sigma > 0, the kernel notes in the workspace what the second march needs of them
- * (24 bytes per leaf, in chunks of 384 bytes = 15 leaves and a link); a ray whose notes fit is not
- * marched a second time, the others are.  The first n_rays chunks are the rays' own; the rest of
+ * (16-byte aligned, any contents, overwritten): the first of the two marches of a ray notes in the
+ * workspace what the second march needs of the leaves with sigma > 0 (24 bytes per leaf, in chunks
+ * of 384 bytes = 15 leaves and a link), and a second launch forms the gradient of every ray whose
+ * notes fit from those notes, without the tree; the other rays are marched a second time.  The first n_rays chunks are the rays' own; the rest of
  * the workspace is shared out among the wavefronts for rays with more than 15 such leaves.  After
  * the chunks come one bit per ray and 256 bytes of bookkeeping (used by the two calls below), so
  * the workspace holds (workspace_bytes - 256 - 16 * ceil(n_rays / 128)) / 384 chunks and is useful

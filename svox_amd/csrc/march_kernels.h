@@ -660,14 +660,16 @@ __device__ __forceinline__ int64_t skip_clear_words(const unsigned long long* __
 
 // What a launch of render_backward_kernel does:
 //   kBackwardPlain   both marches walk the tree;
-//   kBackwardReplay  march 1 leaves notes in the workspace, march 2 replays them.
-// (The notes a forward pass leaves for a later backward pass are taken by render_forward_kernel and
-// render_forward_split_kernel with kNoted, and used by replay_backward_kernel.)
-enum BackwardMode { kBackwardPlain = 0, kBackwardReplay = 1 };
+//   kBackwardSecond  only the second march: the first was made by a noting forward kernel.
+// (Notes are taken by render_forward_kernel and render_forward_split_kernel with kNoted and used by
+// replay_backward_kernel; render_backward_kernel serves the rays that have none.)
+enum BackwardMode { kBackwardPlain = 0, kBackwardSecond = 1 };
 
 // Head of a ray's notes, kept in the spare floats of its first chunk (after the 15 records): the
 // link to the next chunk, the number of notes (-1: they did not fit; 0 also for a ray that misses
-// the tree), the ray's delta_scale (rt_kernel.cu:228) and 1.0f if the ray misses the tree, else 0.0f.
+// the tree), the ray's delta_scale (rt_kernel.cu:228), a flag (1.0f: the ray misses the tree, 2.0f:
+// its walk broke off in a malformed tree, else 0.0f) and the sum of the backward pass's first march
+// where the noting pass could form it (NoteTaker::finish).
 constexpr int kChunkRecords = 15;
 constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
 constexpr int kHeadFloat2 = kChunkRecords * 3;          // float2 index of {link, count}, then {delta_scale, -}
@@ -736,10 +738,42 @@ struct NoteTaker {
         }
     }
     // The head of the notes: the count beside the link (written when the first chunk filled up), -1 if
-    // the notes are incomplete; then the ray's delta_scale.
-    __device__ __forceinline__ void finish(bool broken, float dscale) {
+    // the notes are incomplete; then the ray's delta_scale and 2.0f if the walk broke off in a
+    // malformed tree; then, from a noting pass that had the gradient of the picture at hand, the sum
+    // the backward pass forms in its first march (render_backward_kernel<kBackwardSecond> starts from it).
+    __device__ __forceinline__ void finish(bool broken, float dscale, float march1_sum = 0.0f) {
         ((float*)(first + kHeadFloat2))[1] = __int_as_float(lost || broken ? -1 : count);
-        first[kHeadFloat2 + 1] = make_float2(dscale, 0.0f);
+        first[kHeadFloat2 + 1] = make_float2(dscale, broken ? 2.0f : 0.0f);
+        first[kHeadFloat2 + 2] = make_float2(march1_sum, 0.0f);
+    }
+};
+
+// What a noting pass that has the gradient of the picture at hand accumulates per ray beside its notes:
+// the sum the backward pass forms in its first march (rt_kernel.cu:358-419; the same expressions, in
+// the same order, as march 1 of render_backward_kernel), so that a ray whose notes do not fit needs
+// only the second march afterwards.
+struct March1Sum {
+    float go[3], light, accum;
+    __device__ __forceinline__ void begin(const float* __restrict__ grad_out, int64_t slot) {
+        go[0] = grad_out[slot * 3];
+        go[1] = grad_out[slot * 3 + 1];
+        go[2] = grad_out[slot * 3 + 2];
+        light = 1.0f;
+        accum = 0.0f;
+    }
+    // a leaf with sigma > 0 and the sigmoids s of its colour
+    __device__ __forceinline__ void leaf(float dt, float sigma, float dscale, const float* s, float d_rgb_pad, float pad) {
+        const float att = expf_fixed(-dt * sigma * dscale);
+        const float weight = light * (1.0f - att);
+        float total_color = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 3; ++c) total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
+        light *= att;
+        accum = fma_(weight, total_color, accum);
+    }
+    __device__ __forceinline__ float end(float bg) const {
+        const float total_grad = (go[0] + go[1]) + go[2];
+        return fma_(light * bg, total_grad, accum);
     }
 };
 
@@ -767,11 +801,14 @@ struct NoteTaker {
 // kNoted: the forward pass of a training step.  The picture is composed as without it; beside it the
 // launch leaves in the workspace the notes the backward pass works from (NoteTaker): every leaf with
 // sigma > 0 of the whole ray, so a ray is walked to its end also after its picture stopped early, and
-// the colours of the leaves at or below sigma_thresh are evaluated too.
-template <class P, class Source, bool kAccum, bool kRefill, bool kNoted = false>
+// the colours of the leaves at or below sigma_thresh are evaluated too.  With out == nullptr only the
+// notes are taken (the backward pass without a forward pass before it); kGrad: that backward pass's
+// grad_out is given, and the sum of its first march is formed on the way (March1Sum).
+template <class P, class Source, bool kAccum, bool kRefill, bool kNoted = false, bool kGrad = false>
 __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<float> tr, Source src,
                                                                        SvoxRenderOptions opt,
-                                                                       float* __restrict__ out, ReplaySpace ws) {
+                                                                       float* __restrict__ out, ReplaySpace ws,
+                                                                       const float* __restrict__ grad_out = nullptr) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
@@ -799,6 +836,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     bool active = false;
     bool painted = false;   // kNoted: the ray's picture is finished (early stop), its notes go on
     NoteTaker notes;
+    March1Sum sum1;
     int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of chunks for notes (uniform)
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
@@ -819,13 +857,16 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
             cur.restart();
             active = true;
             if constexpr (kNoted) {
-                painted = false;
+                painted = out == nullptr;   // no picture asked for: nothing to compose
                 notes.begin(ws, slot);
+                if constexpr (kGrad) sum1.begin(grad_out, slot);
             }
         } else {
-            out[slot * 3] = bg;
-            out[slot * 3 + 1] = bg;
-            out[slot * 3 + 2] = bg;
+            if (!kNoted || out) {
+                out[slot * 3] = bg;
+                out[slot * 3 + 1] = bg;
+                out[slot * 3 + 2] = bg;
+            }
             if constexpr (kNoted) NoteTaker::missed(ws, slot);
         }
     };
@@ -892,8 +933,11 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                 }
                 stopped = stopped || (take && light <= stop_thresh);
                 if constexpr (kNoted) {
-                    notes.take(ws, shared_next, shared_end, lane, active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f,
-                               q_leaf[q], q_dt[q], q_sigma[q], q_s[q]);
+                    const bool note = active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
+                    notes.take(ws, shared_next, shared_end, lane, note, q_leaf[q], q_dt[q], q_sigma[q], q_s[q]);
+                    if constexpr (kGrad) {
+                        if (note) sum1.leaf(q_dt[q], q_sigma[q], r.dscale, q_s[q], d_rgb_pad, pad);
+                    }
                 }
             }
         }
@@ -916,7 +960,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                     out[slot * 3 + 1] = fma_(light, bg, acc[1]);
                     out[slot * 3 + 2] = fma_(light, bg, acc[2]);
                 }
-                if constexpr (kNoted) notes.finish(broken, r.dscale);
+                if constexpr (kNoted) notes.finish(broken, r.dscale, kGrad ? sum1.end(bg) : 0.0f);
                 active = false;
             }
         }
@@ -1399,10 +1443,11 @@ __device__ __forceinline__ void box_write(int32_t* at, int32_t value) {
     __hip_atomic_store(at, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-template <class P, class Source, bool kNoted = false>
+template <class P, class Source, bool kNoted = false, bool kGrad = false>
 __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(TreeDev<float> tr, Source src,
                                                                              SvoxRenderOptions opt,
-                                                                             float* __restrict__ out, ReplaySpace ws) {
+                                                                             float* __restrict__ out, ReplaySpace ws,
+                                                                             const float* __restrict__ grad_out = nullptr) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
@@ -1430,9 +1475,11 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         if (slot >= 0) active = setup_ray(r, origin, dir, scaling);
         if (!walks) {
             if (slot >= 0 && !active) {
-                out[slot * 3] = bg;
-                out[slot * 3 + 1] = bg;
-                out[slot * 3 + 2] = bg;
+                if (!kNoted || out) {
+                    out[slot * 3] = bg;
+                    out[slot * 3 + 1] = bg;
+                    out[slot * 3 + 2] = bg;
+                }
                 if constexpr (kNoted) NoteTaker::missed(ws, slot);
             }
             if constexpr (P::kFormat == SVOX_FORMAT_SH) {
@@ -1501,11 +1548,14 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
     float light = 1.0f;
     int32_t taken = 0;
     int spins = 0;
-    // kNoted: the picture of a ray may be finished (early stop) while its notes go on
-    bool painted = false;
+    // kNoted: the picture of a ray may be finished (early stop) while its notes go on; without `out`
+    // there is no picture to compose
+    bool painted = kNoted && out == nullptr;
     NoteTaker notes;
+    March1Sum sum1;
     int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of chunks for notes (uniform)
     if constexpr (kNoted) notes.begin(ws, active ? slot : 0);
+    if constexpr (kNoted && kGrad) sum1.begin(grad_out, active ? slot : 0);
     while (true) {
         const int32_t w = box_read(&box.written[lane]);
         asm volatile("" ::: "memory");   // the ring is read after the count, not before
@@ -1517,7 +1567,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
                 out[slot * 3 + 1] = fma_(light, bg, acc[1]);
                 out[slot * 3 + 2] = fma_(light, bg, acc[2]);
             }
-            if constexpr (kNoted) notes.finish((w & kBrokenBit) != 0, r.dscale);
+            if constexpr (kNoted) notes.finish((w & kBrokenBit) != 0, r.dscale, kGrad ? sum1.end(bg) : 0.0f);
             active = false;
         }
         if (!__any(active)) break;
@@ -1527,7 +1577,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         if (!__any(n_take > 0)) {   // the walk has found nothing new yet
             if (++spins > kSpinLimit) {
                 // cannot happen while the walk runs; a picture with NaN in it says so if it ever does
-                if (active) out[slot * 3] = out[slot * 3 + 1] = out[slot * 3 + 2] = __int_as_float(0x7fc00000);
+                if (active && out) out[slot * 3] = out[slot * 3 + 1] = out[slot * 3 + 2] = __int_as_float(0x7fc00000);
                 break;
             }
             __builtin_amdgcn_s_sleep(1);
@@ -1577,8 +1627,11 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
                 light = take ? light * q_att[q] : light;
                 stopped = stopped || (take && light <= stop_thresh);
                 if constexpr (kNoted) {
-                    notes.take(ws, shared_next, shared_end, lane, active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f,
-                               q_leaf[q], q_dt[q], q_sigma[q], q_s[q]);
+                    const bool note = active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
+                    notes.take(ws, shared_next, shared_end, lane, note, q_leaf[q], q_dt[q], q_sigma[q], q_s[q]);
+                    if constexpr (kGrad) {
+                        if (note) sum1.leaf(q_dt[q], q_sigma[q], r.dscale, q_s[q], d_rgb_pad, pad);
+                    }
                 }
             }
             wave_lds_sync();   // the colours are read before the next list overwrites them
@@ -1599,17 +1652,15 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
     }
 }
 
-// kReplay: during march 1 a lane notes, for every leaf with sigma > 0, what march 2 needs of it; if
-// the notes fit into the workspace, march 2 does not walk the tree again but replays them (a ray
-// with no such leaf is finished on the spot), otherwise it marches as without a workspace.  The
-// duration of a launch is set by its longest rays: halving their second march is what this buys.
+// kMode: kBackwardPlain runs both marches; kBackwardSecond runs only the second, for rays whose first
+// march a noting forward kernel has already made (with grad_out at hand: NoteTaker keeps the sum of
+// march 1 in the head of the ray's notes) but whose notes did not fit the workspace.
 template <class P, class Source, bool kRefill, int kMode>
 __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<float> tr, Source src,
                                                                         SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
                                                                         float* __restrict__ grad_data,
                                                                         ReplaySpace ws) {
-    constexpr bool kReplay = kMode != kBackwardPlain;
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
@@ -1626,19 +1677,12 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
     const int64_t total = src.total();
     const int64_t end = next + src.per_wave < total ? next + src.per_wave : total;
 
-    enum { kMarch1 = 0, kMarch2 = 1, kReplaying = 2 };
+    enum { kMarch1 = 0, kMarch2 = 1 };
     RayState<float> r;
     float go[3] = {0.f, 0.f, 0.f};
     float light = 1.0f, accum = 0.0f, tmin = 0.0f;
     bool active = false;
     int phase = kMarch1;
-    // notes of march 1: total count, the chunk being written / read and the position in it
-    int rec_count = 0, rec_next = 0, rec_pos = 0;
-    int32_t rec_link = 0;              // replay: index of the chunk after rec_chunk
-    bool rec_lost = false;             // the workspace ran out: this ray marches twice
-    float2* rec_first = ws.base;
-    float2* rec_chunk = ws.base;
-    int64_t shared_next = 0, shared_end = 0;   // the wavefront's stock of further chunks (uniform)
     MergeState merge;
     OctreeCursor cur;
     cur.reset(path + lane, kMarchThreads);
@@ -1651,6 +1695,13 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
         if (!Source::kItemsAreSlots && ws.only && slot >= 0 && !((ws.only[slot >> 6] >> (slot & 63)) & 1ull)) return;
         if (slot >= 0 && setup_ray(r, origin, dir, scaling)) {
+            float march1_sum = 0.0f;
+            if constexpr (kMode == kBackwardSecond) {
+                const float2* head = ws.base + slot * kChunkFloat2 + kHeadFloat2;
+                // (a walk that broke off in a malformed tree: the reference adds nothing for such a ray)
+                if (head[1].y != 0.0f) return;
+                march1_sum = head[2].x;
+            }
             if constexpr (P::kFormat == SVOX_FORMAT_SH) {
                 float basis[D];
                 sh_basis<float>(P::kBasis, vdir, basis);
@@ -1661,18 +1712,11 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             go[1] = grad_out[slot * 3 + 1];
             go[2] = grad_out[slot * 3 + 2];
             light = 1.0f;
-            accum = 0.0f;
+            accum = march1_sum;
             tmin = r.t;
             cur.restart();
-            phase = kMarch1;
+            phase = kMode == kBackwardSecond ? kMarch2 : kMarch1;
             active = true;
-            if constexpr (kReplay) {
-                rec_count = 0;
-                rec_pos = 0;
-                rec_lost = false;
-                rec_first = ws.base + slot * kChunkFloat2;
-                rec_chunk = rec_first;
-            }
         }
     };
     if constexpr (!kRefill) {
@@ -1689,178 +1733,76 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             if (!__any(active)) break;
         }
 
-        // ---- walk (lanes that replay their notes do not walk)
-        const bool replaying = kReplay && phase == kReplaying;
+        // ---- walk
         int32_t q_leaf[kQueue];
         float q_dt[kQueue];
         bool broken;
         float q_sigma[kQueue];
-        const bool any_walk = !kReplay || __any(active && !replaying);
-        if (any_walk) {
-            walk_turns(tr, r, cur, step, active && !replaying, broken, q_leaf, q_dt);
-            // ---- sigma
-            fetch_sigma<K>(tr.data, q_leaf, q_sigma);
-        } else {
-            // every lane left replays: a round without the tree
-            broken = false;
+        walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt);
+        // ---- sigma
+        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+        // ---- shade list: every leaf with density
+        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane);
+        wave_lds_sync();
+        if (n_entries > 0) shade_entries<P, true>(tr.data, sh, n_entries, lane);
+        wave_lds_sync();
+        // ---- composite slot by slot; the gradient records of the round are added together
+        RecordList<P, D> records{sh, grad_data, lane, merge};
+        // what does not depend on the transmittance is evaluated for the four slots side by side
+        float q_att[kQueue], q_total[kQueue], q_s[kQueue][3];
 #pragma unroll
-            for (int q = 0; q < kQueue; ++q) {
-                q_leaf[q] = -1;
-                q_dt[q] = 0.0f;
-                q_sigma[q] = 0.0f;
+        for (int q = 0; q < kQueue; ++q) {
+            q_att[q] = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
+            const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
+            float total_color = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                q_s[q][c] = s[c];
+                total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
             }
+            q_total[q] = total_color;
         }
-        // ---- replayed leaves: the next kQueue notes take the slots.
-        // Their loads are in flight together with the density loads of the walking lanes.
-        if constexpr (kReplay) {
-            if (active && replaying) {
 #pragma unroll
-                for (int q = 0; q < kQueue; ++q) {
-                    if (rec_next + q < rec_count) {
-                        if (rec_pos == kChunkRecords) {
-                            // the link was read when this chunk was entered: no load to wait for here
-                            rec_chunk = ws.base + (int64_t)rec_link * kChunkFloat2;
-                            rec_link = __float_as_int(rec_chunk[kHeadFloat2].x);
-                            rec_pos = 0;
-                        }
-                        const float2* e = rec_chunk + rec_pos * 3;
-                        const float2 a = e[0], b = e[1], c = e[2];
-                        rec_pos += 1;
-                        q_leaf[q] = __float_as_int(a.x);
-                        q_dt[q] = a.y;
-                        q_sigma[q] = b.x;
-                        float* s = sh.colour + (q * kMarchThreads + lane) * 3;
-                        s[0] = b.y;
-                        s[1] = c.x;
-                        s[2] = c.y;
-                    }
-                }
-            }
-        }
-        // ---- shade list (walking lanes only)
-        const int n_entries = any_walk ? build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane, replaying) : 0;
-        {
-            wave_lds_sync();
-            if (n_entries > 0) shade_entries<P, true>(tr.data, sh, n_entries, lane);
-            wave_lds_sync();
-            // ---- composite slot by slot; the gradient records of the round are added together
-            RecordList<P, D> records{sh, grad_data, lane, merge};
-            // what does not depend on the transmittance is evaluated for the four slots side by side
-            float q_att[kQueue], q_total[kQueue], q_s[kQueue][3];
-#pragma unroll
-            for (int q = 0; q < kQueue; ++q) {
-                q_att[q] = expf_fixed(-q_dt[q] * q_sigma[q] * r.dscale);
-                const float* s = sh.colour + (q * kMarchThreads + lane) * 3;
-                float total_color = 0.0f;
-#pragma unroll
-                for (int c = 0; c < 3; ++c) {
-                    q_s[q][c] = s[c];
-                    total_color = fma_(fma_(s[c], d_rgb_pad, -pad), go[c], total_color);
-                }
-                q_total[q] = total_color;
-            }
-#pragma unroll
-            for (int q = 0; q < kQueue; ++q) {
-                bool emit = false, note = false;
-                float tmp2[3] = {0.f, 0.f, 0.f};
-                float g_sigma = 0.f;
-                float note_s[3] = {0.f, 0.f, 0.f};
-                if (active && q_leaf[q] >= 0 && (replaying || q_sigma[q] > 0.0f)) {
-                    const float att = q_att[q];
-                    const float weight = light * (1.0f - att);
-                    const float* s = q_s[q];
-                    const float total_color = q_total[q];
-                    light *= att;
-                    if (phase == kMarch1) {
-                        accum = fma_(weight, total_color, accum);
-                        if constexpr (kReplay) {
-                            note = true;
-                            note_s[0] = s[0];
-                            note_s[1] = s[1];
-                            note_s[2] = s[2];
-                        }
-                    } else {
-#pragma unroll
-                        for (int c = 0; c < 3; ++c) {
-                            if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-                                tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
-                            } else {
-                                tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)go[c] *
-                                                  (double)d_rgb_pad);
-                            }
-                        }
-                        accum = fma_(-weight, total_color, accum);
-                        g_sigma = q_dt[q] * r.dscale * fma_(total_color, light, -accum);
-                        emit = true;
-                    }
-                }
-                if constexpr (kReplay) {
-                    // lanes whose chunk is full take the next chunks of the wavefront's stock, in lane order
-                    const bool need = note && !rec_lost && rec_pos == kChunkRecords;
-                    const unsigned long long m = __ballot(need);
-                    if (m) {
-                        if (shared_next + __popcll(m) > shared_end) {
-                            // a new stock (what is left of the old one is given up): one atomic per 64 chunks
-                            unsigned long long t = 0;
-                            if (lane == 0) t = atomicAdd(ws.stocks_taken, 1ull);
-                            const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)t);
-                            const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(t >> 32));
-                            const int64_t stock = (int64_t)(((unsigned long long)hi << 32) | lo);
-                            shared_next = ws.first_shared + stock * kChunkStock;
-                            shared_end = shared_next + kChunkStock < ws.n_chunks ? shared_next + kChunkStock : ws.n_chunks;
-                            if (shared_next > shared_end) shared_next = shared_end;
-                        }
-                        const int64_t mine = shared_next + rank_in(m);
-                        if (need) {
-                            if (mine < shared_end) {
-                                rec_chunk[kHeadFloat2] = make_float2(__int_as_float((int32_t)mine), 0.0f);
-                                rec_chunk = ws.base + mine * kChunkFloat2;
-                                rec_pos = 0;
-                            } else {
-                                rec_lost = true;
-                            }
-                        }
-                        shared_next += __popcll(m);
-                    }
-                    if (note) {
-                        if (!rec_lost) {
-                            float2* e = rec_chunk + rec_pos * 3;
-                            e[0] = make_float2(__int_as_float(q_leaf[q]), q_dt[q]);
-                            e[1] = make_float2(q_sigma[q], note_s[0]);
-                            e[2] = make_float2(note_s[1], note_s[2]);
-                            rec_pos += 1;
-                        }
-                        rec_count += 1;
-                    }
-                }
-                records.append(emit, q_leaf[q], tmp2, g_sigma);
-            }
-            records.flush();
-        }
-        // ---- end of a march
-        if (active) {
-            if (replaying) {
-                rec_next += kQueue;
-                if (rec_next >= rec_count) active = false;
-            } else if (broken || !(r.t < r.tmax)) {
-                if (phase == kMarch1 && !broken) {
-                    const float total_grad = (go[0] + go[1]) + go[2];
-                    accum = fma_(light * bg, total_grad, accum);
-                    light = 1.0f;
-                    if (kReplay && !rec_lost) {
-                        phase = kReplaying;
-                        rec_next = 0;
-                        rec_pos = 0;
-                        rec_chunk = rec_first;
-                        rec_link = __float_as_int(rec_first[kHeadFloat2].x);   // garbage if there is none
-                        if (rec_count == 0) active = false;   // no leaf with sigma > 0: nothing to add
-                    } else {
-                        phase = kMarch2;
-                        r.t = tmin;
-                    }
+        for (int q = 0; q < kQueue; ++q) {
+            bool emit = false;
+            float tmp2[3] = {0.f, 0.f, 0.f};
+            float g_sigma = 0.f;
+            if (active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f) {
+                const float att = q_att[q];
+                const float weight = light * (1.0f - att);
+                const float* s = q_s[q];
+                const float total_color = q_total[q];
+                light *= att;
+                if (phase == kMarch1) {
+                    accum = fma_(weight, total_color, accum);
                 } else {
-                    active = false;
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) {
+                        if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
+                            tmp2[c] = weight * s[c] * (1.0f - s[c]) * go[c] * d_rgb_pad;
+                        } else {
+                            tmp2[c] = (float)((double)(weight * s[c]) * (1.0 - (double)s[c]) * (double)go[c] *
+                                              (double)d_rgb_pad);
+                        }
+                    }
+                    accum = fma_(-weight, total_color, accum);
+                    g_sigma = q_dt[q] * r.dscale * fma_(total_color, light, -accum);
+                    emit = true;
                 }
+            }
+            records.append(emit, q_leaf[q], tmp2, g_sigma);
+        }
+        records.flush();
+        // ---- end of a march
+        if (active && (broken || !(r.t < r.tmax))) {
+            if (phase == kMarch1 && !broken) {
+                const float total_grad = (go[0] + go[1]) + go[2];
+                accum = fma_(light * bg, total_grad, accum);
+                light = 1.0f;
+                phase = kMarch2;
+                r.t = tmin;
+            } else {
+                active = false;
             }
         }
     }

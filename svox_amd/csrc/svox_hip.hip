@@ -411,33 +411,28 @@ bool carve_workspace(void* workspace, int64_t workspace_bytes, int64_t n_slots, 
     return true;
 }
 
-// The backward pass, with whatever the workspace allows: march 2 replayed from notes of march 1 if it
-// is large enough, else two marches.
+// The backward pass by two marches per ray (no workspace, or one that cannot serve: see backward_by_noting).
 template <class Source, typename T>
 void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, int out_dim,
-                     const void* grad_out, void* grad_data, void* workspace, int64_t workspace_bytes,
-                     int64_t n_slots, hipStream_t stream) {
+                     const void* grad_out, void* grad_data, hipStream_t stream) {
     const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
         const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
             const Source dealt = dealt_out(src, blocks);
-            // every ray owns one chunk; the wavefronts draw on what is left of the workspace
-            ReplaySpace ws;
-            const bool replay = carve_workspace(workspace, workspace_bytes, n_slots, &ws) &&
-                                zero_fill(ws.stocks_taken, 16, stream) == SVOX_OK;
-#define SVOX_LAUNCH_BACKWARD(REFILL, MODE)                                                                      \
-    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, REFILL, MODE>), dim3(blocks),  \
-                                               dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt,     \
-                                               *opt, (const float*)grad_out, (float*)grad_data, ws))
-            const bool refill = src.per_wave > kMarchThreads;
-            if (replay) {
-                if (refill) { SVOX_LAUNCH_BACKWARD(true, kBackwardReplay); } else { SVOX_LAUNCH_BACKWARD(false, kBackwardReplay); }
+            const ReplaySpace none{};
+            if (src.per_wave > kMarchThreads) {
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, true, kBackwardPlain>),
+                                                           dim3(blocks), dim3(kMarchThreads), 0, stream,
+                                                           march_tree(tree, opt), dealt, *opt, (const float*)grad_out,
+                                                           (float*)grad_data, none));
             } else {
-                if (refill) { SVOX_LAUNCH_BACKWARD(true, kBackwardPlain); } else { SVOX_LAUNCH_BACKWARD(false, kBackwardPlain); }
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, false, kBackwardPlain>),
+                                                           dim3(blocks), dim3(kMarchThreads), 0, stream,
+                                                           march_tree(tree, opt), dealt, *opt, (const float*)grad_out,
+                                                           (float*)grad_data, none));
             }
-#undef SVOX_LAUNCH_BACKWARD
             return;
         }
     }
@@ -458,11 +453,13 @@ ImageSource<T> noting_shape(const ImageSource<T>& s) { return s; }
 
 // The forward pass of a training step: the picture into `out` and, in the workspace, the notes of
 // every ray under `stamp`.  Needs a usable workspace and the octree kernels, which noted_ok() tells
-// beforehand.  A launch that does not fill the GPU runs on two wavefronts per 64 rays.
+// beforehand.  A launch that does not fill the GPU runs on two wavefronts per 64 rays.  out may be
+// nullptr (notes only); grad_out, if given, is the gradient of the picture the backward pass will be
+// called with: the notes' heads then also carry the sum of that pass's first march.
 template <class Source>
 int launch_noted(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOptions* opt, void* out,
                  void* workspace, int64_t workspace_bytes, int64_t n_slots, const NoteStamp& stamp,
-                 hipStream_t stream) {
+                 hipStream_t stream, const void* grad_out = nullptr) {
     const int D = fast_basis(tree, opt);
     const unsigned blocks = blocks_for(total_items_of(src), src.per_wave);
     const Source dealt = dealt_out(src, blocks);
@@ -473,19 +470,29 @@ int launch_noted(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOp
     if (rc) return rc;
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
     const bool refill = src.per_wave > kMarchThreads;
-    if (!refill && use_split_forward(blocks, is_image_source(src), opt)) {
-        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, true>), dim3(blocks),
-                                                   dim3(kSplitThreads), 0, stream, march_tree(tree, opt), dealt, *opt,
-                                                   (float*)out, ws));
-    } else if (refill) {
-        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, false, true, true>), dim3(blocks),
-                                                   dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt, *opt,
-                                                   (float*)out, ws));
+    const bool split = !refill && use_split_forward(blocks, is_image_source(src), opt);
+    const dim3 threads(split ? kSplitThreads : kMarchThreads);
+#define SVOX_LAUNCH_NOTING(KERNEL)                                                                                   \
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL(KERNEL, dim3(blocks), threads, 0, stream, march_tree(tree, opt), dealt, \
+                                               *opt, (float*)out, ws, (const float*)grad_out))
+    if (grad_out) {
+        if (split) {
+            SVOX_LAUNCH_NOTING((render_forward_split_kernel<P, Source, true, true>));
+        } else if (refill) {
+            SVOX_LAUNCH_NOTING((render_forward_kernel<P, Source, false, true, true, true>));
+        } else {
+            SVOX_LAUNCH_NOTING((render_forward_kernel<P, Source, false, false, true, true>));
+        }
     } else {
-        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, false, false, true>), dim3(blocks),
-                                                   dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt, *opt,
-                                                   (float*)out, ws));
+        if (split) {
+            SVOX_LAUNCH_NOTING((render_forward_split_kernel<P, Source, true, false>));
+        } else if (refill) {
+            SVOX_LAUNCH_NOTING((render_forward_kernel<P, Source, false, true, true, false>));
+        } else {
+            SVOX_LAUNCH_NOTING((render_forward_kernel<P, Source, false, false, true, false>));
+        }
     }
+#undef SVOX_LAUNCH_NOTING
     return SVOX_OK;
 }
 
@@ -560,9 +567,6 @@ int se_grad_prepare(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, void
     return zero_fill(hess, data_bytes(tree), stream);
 }
 
-// wavefronts that look after the rays of a batch that replay_backward_kernel leaves undone (normally none)
-constexpr int kUndoneWaves = 256;
-
 // Can notes be taken (launch_noted) and used (replay_backward_kernel)?  The octree kernels, a forward
 // pass whose threshold does not admit leaves the backward pass ignores, no weight accumulator, and a
 // workspace with a chunk for every ray.
@@ -594,11 +598,13 @@ int replay_ray_shift(bool image) {
 }
 
 // The backward pass of `all` from the notes in the workspace: the rays with complete notes by
-// replay_backward_kernel, the others, which it marks in the bitmap, by two marches.
+// replay_backward_kernel, the others, which it marks in the bitmap, by marching (`rest`: the launch
+// shape for those): twice, or -- march1_known: the noting pass had grad_output and left the sum of
+// the first march in the heads of the notes -- once.
 template <class Source>
 int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest, const SvoxRenderOptions* opt,
                                const void* grad_output, void* grad_data_out, void* workspace, int64_t workspace_bytes,
-                               int64_t n_slots, const NoteStamp& stamp, hipStream_t stream) {
+                               int64_t n_slots, const NoteStamp& stamp, hipStream_t stream, bool march1_known = false) {
     const int D = fast_basis(tree, opt);
     const int ray_shift = replay_ray_shift(is_image_source(all));
     const unsigned waves = blocks_for(n_slots, 1 << ray_shift);
@@ -610,18 +616,53 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
                                                ray_shift));
     int rc = check_launch("volume_render_backward_noted");
     if (rc) return rc;
-    ReplaySpace only = ReplaySpace{nullptr, 0, 0, nullptr, nullptr, {0, 0, 0, 0, 0, 0}, nullptr, ws.undone};
+    ReplaySpace only{};
+    only.base = ws.base;
+    only.only = ws.undone;
     const unsigned blocks = blocks_for(total_items_of(rest), rest.per_wave);
+#define SVOX_LAUNCH_REST(REFILL, MODE)                                                                              \
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, REFILL, MODE>), dim3(blocks),      \
+                                               dim3(kMarchThreads), 0, stream, march_tree(tree, opt), rest, *opt,    \
+                                               (const float*)grad_output, (float*)grad_data_out, only))
     if (rest.per_wave > kMarchThreads) {
-        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, true, kBackwardPlain>), dim3(blocks),
-                                                   dim3(kMarchThreads), 0, stream, march_tree(tree, opt), rest, *opt,
-                                                   (const float*)grad_output, (float*)grad_data_out, only));
+        if (march1_known) { SVOX_LAUNCH_REST(true, kBackwardSecond); } else { SVOX_LAUNCH_REST(true, kBackwardPlain); }
     } else {
-        SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_backward_kernel<P, Source, false, kBackwardPlain>), dim3(blocks),
-                                                   dim3(kMarchThreads), 0, stream, march_tree(tree, opt), rest, *opt,
-                                                   (const float*)grad_output, (float*)grad_data_out, only));
+        if (march1_known) { SVOX_LAUNCH_REST(false, kBackwardSecond); } else { SVOX_LAUNCH_REST(false, kBackwardPlain); }
     }
+#undef SVOX_LAUNCH_REST
     return check_launch("volume_render_backward_noted");
+}
+
+// the options under which notes are taken where no picture hangs on them (se_grad, the backward pass alone): every leaf with sigma > 0, no early stop
+SvoxRenderOptions without_thresholds(const SvoxRenderOptions* opt) {
+    SvoxRenderOptions o = *opt;
+    o.sigma_thresh = 0.0f;
+    o.stop_thresh = 0.0f;
+    return o;
+}
+
+// The backward pass of a call that brings a workspace but no notes: one noting march without a picture
+// (thresholds play no part in the backward pass, rt_kernel.cu:377, 441), then backward_from_notes.  The
+// reference's two marches per ray become one walk of the tree and one pass over 24 bytes per leaf with
+// density.  `all`, `rest` as in backward_from_notes; returns 1 if notes cannot be taken here (the
+// caller then marches twice), else a status.
+template <class Source>
+int backward_by_noting(const SvoxTreeSpec* tree, const Source& all, const Source& rest, const SvoxRenderOptions* opt,
+                       const void* grad_output, void* grad_data_out, void* workspace, int64_t workspace_bytes,
+                       int64_t n_slots, NoteStamp stamp, hipStream_t stream) {
+    SvoxTreeSpec quiet = *tree;
+    quiet.weight_accum = nullptr;   // (the backward pass accumulates no weights)
+    const SvoxRenderOptions plain = without_thresholds(opt);
+    if (!noted_ok(&quiet, &plain, n_slots, workspace, workspace_bytes)) return 1;
+    // (the notes belong to this call alone: the stamp carries its gradient buffer too)
+    stamp.word[0] ^= (unsigned long long)(uintptr_t)grad_output;
+    int rc = launch_noted(&quiet, noting_shape(all), &plain, nullptr, workspace, workspace_bytes, n_slots, stamp, stream,
+                          grad_output);
+    if (rc) return rc;
+    rc = check_launch("volume_render_backward");
+    if (rc) return rc;
+    return backward_from_notes(&quiet, all, rest, &plain, grad_output, grad_data_out, workspace, workspace_bytes,
+                               n_slots, stamp, stream, true);
 }
 
 // se_grad of the rays of `all` with their notes kept in the workspace between its two halves: one
@@ -650,13 +691,6 @@ int se_grad_from_notes(const SvoxTreeSpec* tree, const Source& all, const Source
     return check_launch("se_grad");
 }
 
-// the options under which se_grad's notes are taken: every leaf with sigma > 0, no early stop
-SvoxRenderOptions without_thresholds(const SvoxRenderOptions* opt) {
-    SvoxRenderOptions o = *opt;
-    o.sigma_thresh = 0.0f;
-    o.stop_thresh = 0.0f;
-    return o;
-}
 
 }  // namespace
 
@@ -804,10 +838,7 @@ int svox_volume_render_backward_noted(const SvoxTreeSpec* tree, const SvoxRaysSp
     if (rays->n_rays == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
     const BatchSource<float> all = batch_source<float>(rays, true);
-    BatchSource<float> rest = all;
-    const int64_t words = (rays->n_rays + kMarchThreads - 1) / kMarchThreads;
-    rest.per_wave = (int)((words + kUndoneWaves - 1) / kUndoneWaves) * kMarchThreads;
-    return backward_from_notes(tree, all, rest, opt, grad_output, grad_data_out, workspace, workspace_bytes,
+    return backward_from_notes(tree, all, all, opt, grad_output, grad_data_out, workspace, workspace_bytes,
                                rays->n_rays, stamp_of(tree, rays, opt), (hipStream_t)stream);
 }
 
@@ -940,19 +971,24 @@ int svox_volume_render_backward_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec*
     if (rays->n_rays == 0) return SVOX_OK;
     if (!grad_output) return fail(SVOX_ERR_NULL_POINTER, "grad_output is NULL");
     if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
+    if (tree->dtype == SVOX_F32 && workspace) {
+        const BatchSource<float> all = batch_source<float>(rays, true);
+        rc = backward_by_noting(tree, all, all, opt, grad_output, grad_data_out, workspace, workspace_bytes,
+                                rays->n_rays, stamp_of(tree, rays, opt), (hipStream_t)stream);
+        if (rc <= 0) return rc;
+    }
     if (tree->dtype == SVOX_F32)
         launch_backward<BatchSource<float>, float>(tree, batch_source<float>(rays, true), opt, od, grad_output,
-                                                   grad_data_out, workspace, workspace_bytes, rays->n_rays,
-                                                   (hipStream_t)stream);
+                                                   grad_data_out, (hipStream_t)stream);
     else
         launch_backward<BatchSource<double>, double>(tree, batch_source<double>(rays, true), opt, od, grad_output,
-                                                     grad_data_out, nullptr, 0, 0, (hipStream_t)stream);
+                                                     grad_data_out, (hipStream_t)stream);
     return check_launch("volume_render_backward");
 }
 
 // svox_volume_render_backward_ws on the library's own array: no allocation anywhere on the way (the
-// stock counter in the array's tail is cleared by the fill kernel of launch_backward before every
-// launch; everything else in the array is written before it is read within the launch).
+// stock counter in the array's tail is cleared by the fill kernel of launch_noted before the noting
+// launch; everything else in the array is written by that launch before the launches after it read it).
 int svox_volume_render_backward_static(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
                                        const SvoxRenderOptions* opt, const void* grad_output, void* grad_data_out,
                                        int32_t accumulate, void* stream) {
@@ -998,13 +1034,16 @@ int svox_volume_render_images_backward_ws(const SvoxTreeSpec* tree, const SvoxCa
     if (workspace_bytes < 0) return fail(SVOX_ERR_BAD_SHAPE, "negative workspace size");
     if (tree->dtype == SVOX_F32) {
         const auto src = image_source<float>(cam, n_images, pose_stride);
-        launch_backward<ImageSource<float>, float>(tree, src, opt, od, grad_output, grad_data_out, workspace,
-                                                   workspace_bytes, (int64_t)n_images * cam->width * cam->height,
-                                                   (hipStream_t)stream);
+        if (workspace) {
+            rc = backward_by_noting(tree, src, src, opt, grad_output, grad_data_out, workspace, workspace_bytes,
+                                    (int64_t)n_images * cam->width * cam->height,
+                                    stamp_of_image(tree, cam, n_images, opt), (hipStream_t)stream);
+            if (rc <= 0) return rc;
+        }
+        launch_backward<ImageSource<float>, float>(tree, src, opt, od, grad_output, grad_data_out, (hipStream_t)stream);
     } else {
         const auto src = image_source<double>(cam, n_images, pose_stride);
-        launch_backward<ImageSource<double>, double>(tree, src, opt, od, grad_output, grad_data_out, nullptr, 0, 0,
-                                                     (hipStream_t)stream);
+        launch_backward<ImageSource<double>, double>(tree, src, opt, od, grad_output, grad_data_out, (hipStream_t)stream);
     }
     return check_launch("volume_render_image_backward");
 }
@@ -1070,10 +1109,7 @@ int svox_se_grad_ws(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const Sv
     rc = se_grad_prepare(tree, opt, grad_out, hessdiag_out, &od, (hipStream_t)stream);
     if (rc) return rc;
     const BatchSource<float> all = batch_source<float>(rays, true);
-    BatchSource<float> rest = all;
-    const int64_t words = (rays->n_rays + kMarchThreads - 1) / kMarchThreads;
-    rest.per_wave = (int)((words + kUndoneWaves - 1) / kUndoneWaves) * kMarchThreads;
-    return se_grad_from_notes(tree, all, rest, &plain, color_ref, color_out, grad_out, hessdiag_out, workspace,
+    return se_grad_from_notes(tree, all, all, &plain, color_ref, color_out, grad_out, hessdiag_out, workspace,
                               workspace_bytes, rays->n_rays, stamp_of(tree, rays, &plain), (hipStream_t)stream);
 }
 
