@@ -107,7 +107,11 @@ __device__ __forceinline__ void maybe_world2ndc(const SvoxRenderOptions& opt, T*
 //          consecutive items one 16x16 block (four tiles), image after image: the rays a wavefront
 //          holds at any time stay close in the tree, and the dispatcher starts the next image's
 //          blocks as the previous image's last ones drain.  Items that fall outside the image
-//          (sizes that are not multiples of 16) have no ray.
+//          (sizes that are not multiples of 16) have no ray.  The blocks of an image are counted
+//          row by row or (inside_out) ring by ring from the middle of the image: a launch lasts as
+//          long as its longest rays, a camera that looks at an object has them in the middle of
+//          the picture, and counted from there they start first instead of after the dispatcher
+//          has gone through the upper half of the image.
 // fetch_item returns the output slot of the item (ray index / pixel index) or -1, and the ray in
 // tree coordinates.
 template <typename T>
@@ -168,6 +172,29 @@ __device__ __forceinline__ int64_t chunk_of_block(unsigned b, unsigned n_blocks,
     return (int64_t)((j / group) * kXcds + xcd) * group + j % group;
 }
 
+// Block `rank` of an nbx x nby grid of blocks counted from the middle outwards: the innermost
+// rectangle first, then ring after ring (each ring clockwise from its top left corner).
+__device__ __forceinline__ void block_inside_out(int rank, int nbx, int nby, int& bx, int& by) {
+    int p = (min(nbx, nby) - 1) / 2;
+    while (p > 0 && rank >= (nbx - 2 * p) * (nby - 2 * p)) --p;
+    const int w = nbx - 2 * p, h = nby - 2 * p;
+    const int inner = (w > 2 && h > 2) ? (w - 2) * (h - 2) : 0;
+    const int k = rank - inner;
+    if (h == 1) {
+        bx = p + k; by = p;
+    } else if (w == 1) {
+        bx = p; by = p + k;
+    } else if (k < w) {
+        bx = p + k; by = p;
+    } else if (k < w + h - 1) {
+        bx = p + w - 1; by = p + (k - w + 1);
+    } else if (k < 2 * w + h - 2) {
+        bx = p + w - 1 - (k - (w + h - 2)); by = p + h - 1;
+    } else {
+        bx = p; by = p + h - 1 - (k - (2 * w + h - 3));
+    }
+}
+
 template <typename T>
 struct ImageSource {
     Camera<T> cam;          // cam.c2w: pose of image 0
@@ -177,6 +204,7 @@ struct ImageSource {
     int refill_at;          // idle lanes that trigger taking new rays
     int xcd_group;          // see chunk_of_block
     int run;                // > 0: the images advance together, `run` 16x16 blocks at a time
+    int inside_out;         // != 0: the blocks of an image are counted from its middle outwards
     // pixels are numbered image by image, row by row; the items run through the tiles instead
     static constexpr bool kItemsAreSlots = false;
     __device__ __forceinline__ int64_t n_slots() const { return (int64_t)n_images * cam.height * cam.width; }
@@ -213,7 +241,8 @@ struct ImageSource {
             if (image >= n_images) return -1;
             b = (int)(block - (int64_t)image * (nbx * nby));
         }
-        const int by = b / nbx, bx = b - by * nbx;
+        int by = b / nbx, bx = b - by * nbx;
+        if (inside_out) block_inside_out(b, nbx, nby, bx, by);
         const int sub = within >> 6, pos = within & 63;
         const int ix = bx * 16 + (sub & 1) * 8 + (pos & 7);
         const int iy = by * 16 + (sub >> 1) * 8 + (pos >> 3);
