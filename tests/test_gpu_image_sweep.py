@@ -108,3 +108,33 @@ def test_every_image_path_against_the_oracle(gpu, oracle_mod, case):
             finally:
                 C.set_debug_flags(0)
     assert not failures, f"case {case} {p}: " + "; ".join(failures)
+
+
+# Picture shapes whose grid of 16x16 blocks is a single block, a row, a column, or has an odd number
+# of rings: the blocks of an image are counted ring by ring from the middle, and every pixel must be
+# rendered exactly once whatever the shape.
+SHAPES = [(1, 1), (16, 16), (17, 16), (200, 5), (5, 200), (33, 17), (48, 80), (81, 49), (130, 100)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=[f"{w}x{h}" for w, h in SHAPES])
+def test_every_pixel_of_odd_shaped_pictures(gpu, oracle_mod, shape):
+    W, H = shape
+    tree = synth.shell_tree(depth=5, n_spheres=5, data_format="SH4", seed=11, sigma_range=(5.0, 60.0))
+    fx = 0.9 * max(W, H)
+    poses = synth.orbit_poses(2, seed=5, radius=2.5)
+    opt = options(tree, step_size=2e-3, fast=True, background_brightness=0.25)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    want = np.stack([oracle_mod.volume_render_image(ot, c2w, fx, fx, W, H, opt, n_threads=8) for c2w in poses])
+    go = torch.randn(2, H, W, 3, generator=torch.Generator().manual_seed(3)) * 1e-2
+    want_g = sum(oracle_mod.volume_render_image_backward(ot, c2w, fx, fx, W, H, opt, go[i])
+                 for i, c2w in enumerate(poses))
+    dev = on_gpu(tree, gpu)
+    spec = dev._spec()
+    cam = cam_spec(torch.stack(poses).to(gpu), W, H, fx)
+    assert np.array_equal(C.volume_render_images(spec, cam, opt).cpu().numpy(), want)
+    one = C.volume_render_image(spec, cam_spec(poses[1].to(gpu), W, H, fx), opt)
+    assert np.array_equal(one.cpu().numpy(), want[1])
+    for workspace in (True, False):
+        got = C.volume_render_images_backward(spec, cam, opt, go.to(gpu), workspace=workspace)
+        err, ok = grad_close(got.cpu().numpy(), want_g)
+        assert ok, f"{W}x{H} workspace {workspace}: {err:.3e}"
