@@ -187,6 +187,23 @@ def main():
     gather_lines_per_us = 3 * idx.numel() / (a.elapsed_time(b) * 1e3)
     del table, idx
 
+    # what the memory system serves when nothing else is in the way: the library's gather probe (every lane
+    # reads 16 bytes of random 64-byte pieces, four reads in flight) on the tree's records, 1.13 GiB (every
+    # read misses L2), and on 2 MiB of them (every read hits L2 once warm)
+    def probe_rate(buffer):
+        C.gather_probe(buffer, unit_bytes=64, iters=16)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        reads = C.gather_probe(buffer, unit_bytes=64, iters=64)
+        b.record()
+        torch.cuda.synchronize()
+        return reads / (a.elapsed_time(b) * 1e3)
+
+    flat_data = tree.data.detach().view(-1)
+    probe_miss_per_us = probe_rate(flat_data)
+    probe_hit_per_us = probe_rate(flat_data[: (2 << 20) // 4])
+
     # HBM bytes and L2 requests per launch of the dominant kernel come from rocprofv3 counters (separate
     # --pmc runs), not from this process: the committed summary carries the figures for the default workload
     traffic = l2_requests = l2_misses = None
@@ -224,6 +241,15 @@ def main():
             "l2_requests_per_us": round(l2_requests / (durs.mean() * 1e3), 1) if l2_requests else None,
             "l2_misses_per_us": round(l2_misses / (durs.mean() * 1e3), 1) if l2_misses else None,
             "torch_index_select_lines_per_us": round(gather_lines_per_us, 1),
+            # the gather probe: 64-byte requests per microsecond that miss / hit L2, and the time the launch's
+            # requests alone would take at those rates (misses at the one, the other requests at the other)
+            "probe_l2_miss_requests_per_us": round(probe_miss_per_us, 1),
+            "probe_l2_hit_requests_per_us": round(probe_hit_per_us, 1),
+            "launch_ms_at_probe_rates": round((l2_misses / probe_miss_per_us
+                                               + (l2_requests - l2_misses) / probe_hit_per_us) / 1e3, 4)
+            if l2_requests and l2_misses else None,
+            "frac_of_probe_rates": round((l2_misses / probe_miss_per_us + (l2_requests - l2_misses) / probe_hit_per_us)
+                                         / 1e3 / float(durs.mean()), 4) if l2_requests and l2_misses else None,
             # filled in by the query leg: what this library's own gather kernel reaches on random records
             "gather_ceiling_lines_per_us": None, "misses_over_gather_ceiling": None,
         },

@@ -342,6 +342,17 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
                              const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
                              SvoxMarchStats* stats_out, void* stream);
 
+/* No counterpart in the reference; a measurement aid.  The march kernels read scattered 64-byte
+ * pieces of the tree, and how many such requests per microsecond the memory system serves is the
+ * ceiling their launches run against.  This launch measures it: `blocks` blocks of 256 lanes, every
+ * lane reading 16 bytes at the start of 4 * iters pseudo-random `unit_bytes`-sized units (64, 128
+ * or 256) of buffer[0, bytes), four reads in flight per lane; nothing is written unless a checksum
+ * that cannot occur does (`sink`: 16 bytes per lane of the launch, may be left uninitialised).
+ * The caller times the call: blocks * 256 * 4 * iters reads.  A buffer that fits one L2 (4 MiB)
+ * gives the rate of L2 hits, a large one the rate of L2 misses. */
+int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t iters, int32_t blocks,
+                      void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -706,6 +706,19 @@ def volume_render_stats(tree, rays_or_cam, opt):
     return {n: int(v) for n, v in zip(names, vals) if n != "reserved"}
 
 
+def gather_probe(buffer, unit_bytes=64, iters=64, blocks=2048):
+    """Queues the library's gather probe on `buffer` (a contiguous CUDA tensor): blocks * 256 lanes, each
+    reading 16 bytes of 4 * iters pseudo-random `unit_bytes`-sized units.  Returns the number of reads;
+    the caller times the call (a measurement aid for the scattered-read ceiling of the march kernels)."""
+    if not buffer.is_contiguous():
+        raise ValueError("gather_probe: buffer must be contiguous")
+    sink = torch.empty((int(blocks) * 256, 4), dtype=torch.int32, device=buffer.device)
+    with torch.cuda.device(buffer.device):
+        _call("svox_gather_probe", buffer.data_ptr(), buffer.numel() * buffer.element_size(), int(unit_bytes),
+              int(iters), int(blocks), sink.data_ptr(), _stream(buffer.device))
+    return int(blocks) * 256 * 4 * int(iters)
+
+
 def set_debug_flags(flags):
     """bit 0: route every call to the generic kernels; bit 1: small ray batches run like large ones;
     bit 2 / bit 3: forward renders never / always take the two-wavefront kernel"""

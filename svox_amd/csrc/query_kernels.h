@@ -174,6 +174,40 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(TreeDev<T> tr, con
     }
 }
 
+// Measurement aid (svox_gather_probe): every lane reads 16 bytes at the start of 4 * iters
+// pseudo-random units of the buffer, four reads in flight.  The checksum keeps the reads alive; the
+// store never happens for data a caller can have (it would need one exact 32-bit value).
+__device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
+    x ^= x >> 16;
+    x *= 0x7feb352dU;
+    x ^= x >> 15;
+    x *= 0x846ca68bU;
+    x ^= x >> 16;
+    return x;
+}
+__global__ __launch_bounds__(256) void gather_probe_kernel(const uint4* __restrict__ buffer, uint64_t n_units,
+                                                           int unit16, int iters, uint4* __restrict__ sink) {
+    uint4 acc = make_uint4(0u, 0u, 0u, 0u);
+    uint32_t seed = blockIdx.x * 256u + threadIdx.x;
+    for (int it = 0; it < iters; ++it) {
+        uint4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            seed = probe_hash(seed + 0x9e3779b9u * (uint32_t)(k + 1));
+            const uint64_t unit = ((uint64_t)seed * n_units) >> 32;
+            v[k] = buffer[unit * (uint64_t)unit16];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            acc.x ^= v[k].x;
+            acc.y += v[k].y;
+            acc.z ^= v[k].z;
+            acc.w += v[k].w;
+        }
+    }
+    if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) sink[blockIdx.x * 256u + threadIdx.x] = acc;
+}
+
 // calc_corner_kernel, svox_kernel.cu:91-115: climb parent links from the leaf's node to the
 // root; per level result = (result + cell index) / N.
 template <typename T>

@@ -1235,5 +1235,18 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
     return check_launch("volume_render_stats");
 }
 
+int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t iters, int32_t blocks,
+                      void* sink, void* stream) {
+    if (!buffer || !sink) return fail(SVOX_ERR_NULL_POINTER, "svox_gather_probe: NULL buffer or sink");
+    if (unit_bytes != 64 && unit_bytes != 128 && unit_bytes != 256)
+        return fail(SVOX_ERR_BAD_SHAPE, "svox_gather_probe: unit_bytes must be 64, 128 or 256");
+    if (((uintptr_t)buffer & 15u) || bytes < unit_bytes || bytes / unit_bytes > 0xffffffffll || iters < 1 ||
+        blocks < 1 || blocks > (1 << 20))
+        return fail(SVOX_ERR_BAD_SHAPE, "svox_gather_probe: buffer, iters or blocks out of range");
+    hipLaunchKernelGGL(gather_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4*)buffer, (uint64_t)(bytes / unit_bytes), unit_bytes / 16, iters, (uint4*)sink);
+    return check_launch("gather_probe");
+}
+
 }  // extern "C"
 #pragma GCC visibility pop

@@ -870,3 +870,17 @@ def test_density_softplus_on_the_octree_forward_kernel(gpu, oracle_mod, fmt):
     want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go.cpu())
     err, ok = grad_close(dev.data.grad.cpu().numpy(), want_g, rel=2e-4)   # (logf and its derivative from two libraries)
     assert ok, err
+
+
+def test_gather_probe_runs_and_checks_its_arguments(gpu):
+    """The measurement aid reads and writes nothing a caller can see; bad arguments are refused."""
+    buf = torch.arange(1 << 18, dtype=torch.int32, device=gpu)
+    before = buf.clone()
+    assert C.gather_probe(buf, unit_bytes=64, iters=3, blocks=8) == 8 * 256 * 4 * 3
+    assert C.gather_probe(buf, unit_bytes=256, iters=1, blocks=1) == 1024
+    torch.cuda.synchronize()
+    assert torch.equal(buf, before)
+    with pytest.raises(RuntimeError):
+        C.gather_probe(buf, unit_bytes=48)
+    with pytest.raises(RuntimeError):
+        C.gather_probe(buf[:8], unit_bytes=64)
