@@ -1851,7 +1851,8 @@ template <class P, class Source>
 __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3))) void replay_backward_kernel(Source src, SvoxRenderOptions opt,
                                                                         const float* __restrict__ grad_out,
                                                                         float* __restrict__ grad_data,
-                                                                        ReplaySpace ws, int ray_shift) {
+                                                                        ReplaySpace ws, int ray_shift,
+                                                                        int march1_known) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     __shared__ ShadeShared<D, true> sh;
     const int lane = threadIdx.x;
@@ -1903,13 +1904,16 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
     wave_lds_sync();   // the basis rows are read by other lanes when the records are added
 
     float light = 1.0f, accum = 0.0f;
+    // march1_known: the pass that took the notes had grad_out and left the sum of the first march in
+    // the head of the ray's notes (March1Sum: the same expressions in the same order as pass 0 below)
+    if (march1_known && work) accum = first[kHeadFloat2 + 2].x;
     MergeState merge{2};   // (a wavefront of 64 unrelated rays flushes about twice: it never looks)
     RecordList<P, D, true> records{sh, grad_data, lane, merge};
     struct Group {
         float2 note[kReplayGroup][3];
     };
 #pragma unroll 1
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int pass = march1_known ? 1 : 0; pass < 2; ++pass) {
         const float2* chunk = first;
         int32_t link = first_link;
         int pos = 0;

@@ -627,7 +627,7 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P, Source>), dim3(waves), dim3(kMarchThreads), 0,
                                                stream, all, *opt, (const float*)grad_output, (float*)grad_data_out, ws,
-                                               ray_shift));
+                                               ray_shift, march1_known ? 1 : 0));
     int rc = check_launch("volume_render_backward_noted");
     if (rc) return rc;
     ReplaySpace only{};
