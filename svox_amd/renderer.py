@@ -234,7 +234,8 @@ class VolumeRenderer(nn.Module):
       marches through the tree as it then is, which is what the reference's backward pass sees.
       Only a write through `tree.data.data[...]` that is not followed by `tree.touch()` goes unseen.
     * A call of `render_persp` on a stack of poses with at least `csrc.AUTO_MARK_RAYS_PER_CELL` (0.7)
-      rays per cell of the tree first marks the empty leaves (one int32 per cell, freed after the
+      rays per cell of the tree, and at least `csrc.AUTO_MARK_MIN_RAYS` (262 144) rays, first marks the
+      empty leaves (one int32 per cell, freed after the
       call; 25 MB and 0.125 ms for a 512^3 tree of 774 k nodes) so that the march passes through them
       without reading their density.  Smaller calls do not; `N3Tree.mark_empty_leaves()` keeps marks
       on the tree for all of them.  Pictures are bit-identical either way.

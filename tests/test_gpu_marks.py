@@ -204,6 +204,7 @@ def test_large_multi_pose_launch_marks_the_leaves_for_itself(gpu, monkeypatch):
     cam = cam_spec(torch.stack(synth.orbit_poses(3, seed=4, radius=2.5)).to(gpu), 160, 120, 130.0)
     opt = options(tree, step_size=1e-3, fast=True)
     assert 3 * 160 * 120 > C.AUTO_MARK_RAYS_PER_CELL * tree.child.numel()
+    monkeypatch.setattr(C, "AUTO_MARK_MIN_RAYS", 3 * 160 * 120)   # (the floor on the number of rays: just met)
     made = []
     real = C.mark_empty_leaves
     monkeypatch.setattr(C, "mark_empty_leaves", lambda t: made.append(1) or real(t))

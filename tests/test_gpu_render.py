@@ -788,8 +788,13 @@ def test_workspace_and_marking_thresholds_from_both_sides(gpu, monkeypatch):
     cells = tree.child.numel()
     opt = options(tree, step_size=1e-3, fast=True)
     monkeypatch.setattr(C, "AUTO_MARK_RAYS_PER_CELL", 1000 / cells)
+    assert C._marks_for_this_call(tree._spec(), opt, 1000) is None        # (below the floor on the rays)
+    monkeypatch.setattr(C, "AUTO_MARK_MIN_RAYS", 0)
     assert C._marks_for_this_call(tree._spec(), opt, 1000) is not None
     assert C._marks_for_this_call(tree._spec(), opt, 999) is None
+    monkeypatch.setattr(C, "AUTO_MARK_MIN_RAYS", 2000)
+    assert C._marks_for_this_call(tree._spec(), opt, 1999) is None
+    assert C._marks_for_this_call(tree._spec(), opt, 2000) is not None
 
 
 def test_render_of_a_saved_and_loaded_tree(gpu, oracle_mod, tmp_path):
