@@ -537,6 +537,8 @@ class N3Tree(nn.Module):
         self[:] /= val
         return self
 
+    __idiv__ = __itruediv__   # the name the reference defines (svox/svox.py:968)
+
     @property
     def ndim(self):
         return 2

@@ -202,6 +202,9 @@ def _delegate_to_values():
         setattr(N3TreeView, name, make(name, False))
     for name in with_grad:
         setattr(N3TreeView, name, make(name, True))
+    # the reference also lists the Python 2 spellings of division
+    N3TreeView.__div__ = N3TreeView.__truediv__
+    N3TreeView.__rdiv__ = N3TreeView.__rtruediv__
     N3TreeView.__hash__ = object.__hash__
 
 

@@ -387,3 +387,34 @@ def test_notes_pool_info_matches_the_documented_workspace_layout():
     assert pool.value == (chunks - n + 63) // 64
     assert lib.svox_notes_pool_info(n, 384 * (n - 1), ctypes.byref(offset), ctypes.byref(pool)) == -2
     assert lib.svox_notes_pool_info(n, nbytes, None, ctypes.byref(pool)) == -1
+
+
+def test_the_public_names_of_the_reference_are_all_there():
+    """Every public method and property of the reference's N3Tree (svox/svox.py:57-1113), N3TreeView
+    (svox/helpers.py:27-358, with the operators it forwards to `.values`) and VolumeRenderer
+    (svox/renderer.py:114-469), plus the names svox/__init__.py exports."""
+    from svox_amd.view import N3TreeView
+    tree_names = """__call__ __getitem__ __setitem__ __iadd__ __isub__ __imul__ __idiv__ __len__ __repr__
+        accumulate_weights capacity check_integrity clone diam_frontier expand forward from_grid frontier_depth
+        load max_depth max_frontier merge n_frontier n_internal n_leaves ndim numel partial reduce_frontier refine
+        save set set_grid shape shrink shrink_to_fit size snap tree2world world2tree
+        depths lengths lengths_local corners corners_local values values_local sample sample_local aux
+        normal_ clamp_ uniform_ relu_ sigmoid_ nan_to_num_""".split()
+    view_names = """__repr__ __setitem__ __torch_function__ aux clamp_ corners corners_local depths lengths
+        lengths_local nan_to_num_ ndim normal_ refine relu_ sample sample_local set shape sigmoid_ uniform_
+        values values_nograd
+        __floordiv__ __mod__ __div__ __eq__ __ne__ __ge__ __gt__ __le__ __lt__ __floor__ __ceil__ __round__
+        __len__ item size dim numel __add__ __mul__ __sub__ __truediv__ __radd__ __rsub__ __rmul__ __rdiv__
+        __abs__ __pos__ __neg__ clamp clamp_max clamp_min relu sigmoid max min mean sum __getitem__""".split()
+    renderer_names = "forward render_persp se_grad se_grad_persp persp_rays data_format _get_options".split()
+    assert [n for n in tree_names if not hasattr(svox.N3Tree, n)] == []
+    assert [n for n in view_names if not hasattr(N3TreeView, n)] == []
+    assert [n for n in renderer_names if not hasattr(svox.VolumeRenderer, n)] == []
+    for name in ("N3Tree", "VolumeRenderer", "NDCConfig", "Rays", "DataFormat", "LocalIndex"):
+        assert hasattr(svox, name), name
+    # the in-place division the reference spells __idiv__ works as `/=`
+    tree = svox.N3Tree(data_dim=4, init_refine=1)
+    tree.data.data.fill_(3.0)
+    tree /= 2.0
+    assert torch.all(tree[:].values == 1.5)            # (the leaves; cells of inner nodes are no part of tree[:])
+    assert torch.equal((tree[0] / 3.0), tree[0].values / 3.0)
