@@ -52,7 +52,9 @@ class NotesBudget:
     csrc._backward_workspace); passes that use less than a quarter of their room halve it again.
 
     Nothing here waits for the GPU: the counter a pass leaves is copied to pinned memory behind the
-    pass, and looked at by a later pass only once the copy has arrived."""
+    pass, and looked at by a later pass only once the copy has arrived.  While the stream is being
+    captured into a graph (torch.cuda.graph) nothing is observed: a replay cannot change the size of
+    the buffers it was captured with, so the room stays what it was when the capture began."""
 
     MAX_FACTOR = 16
 
@@ -75,7 +77,7 @@ class NotesBudget:
         return int(_C.BACKWARD_RECORDS_PER_RAY) * self.factor
 
     def _settle(self):
-        if self._pending is None:
+        if self._pending is None or torch.cuda.is_current_stream_capturing():
             return
         landing, event, pool = self._pending
         if not event.query():
@@ -92,7 +94,7 @@ class NotesBudget:
 
     def observe(self, notes, n_rays):
         """Called right after the launch of a noted forward pass (on the current stream)."""
-        if notes is None or self._pending is not None:
+        if notes is None or self._pending is not None or torch.cuda.is_current_stream_capturing():
             return
         counter, pool = _C.notes_pool_use(notes, n_rays)
         if self._landing is None:

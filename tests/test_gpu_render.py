@@ -889,3 +889,50 @@ def test_gather_probe_runs_and_checks_its_arguments(gpu):
         C.gather_probe(buf, unit_bytes=48)
     with pytest.raises(RuntimeError):
         C.gather_probe(buf[:8], unit_bytes=64)
+
+
+def test_a_training_step_replays_from_a_hip_graph(gpu):
+    """forward + backward + SGD update captured with torch.cuda.graph: every launch of the library goes
+    to torch's current stream, its zero-fills are kernels and all its buffers come from torch's allocator,
+    so the step can be captured.  Every replay -- with unrelated eager work and a synchronisation between
+    them -- must give what the eager step gives (up to the order of the atomic additions)."""
+    tree = on_gpu(synth.dense_tree(3, "SH4", seed=0, sigma="lognormal", coeff_std=0.5), gpu)
+    r = svox.VolumeRenderer(tree, step_size=1e-3)
+    n = 4096
+    rays = synth.sphere_rays(n, seed=1)
+    rays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.dirs.clone().to(gpu))
+    target = torch.rand(n, 3, device=gpu, generator=torch.Generator(device=gpu).manual_seed(3))
+    start = tree.data.detach().clone()
+
+    def step():
+        out = r(rays)
+        loss = ((out - target) ** 2).sum()
+        loss.backward()
+        with torch.no_grad():
+            tree.data.data -= 0.1 * tree.data.grad
+        tree.data.grad = None
+        return loss.detach()
+
+    eager_losses, eager_data = [], []
+    for _ in range(4):
+        eager_losses.append(float(step()))
+        eager_data.append(tree.data.detach().clone())
+    assert eager_losses[3] < eager_losses[0]
+
+    tree.data.data.copy_(start)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # (torch asks for a warm-up on a side stream)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured_loss = step()
+    tree.data.data.copy_(start)
+    for i in range(4):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert abs(float(captured_loss) - eager_losses[i]) <= 1e-5 * abs(eager_losses[i]), (i, float(captured_loss))
+        err, ok = grad_close(tree.data.detach().cpu().numpy(), eager_data[i].cpu().numpy(), rel=1e-5)
+        assert ok, (i, err)
+        assert float((torch.rand(1000, device=gpu) * 2).sum()) > 0          # eager work between the replays
