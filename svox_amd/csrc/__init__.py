@@ -460,6 +460,11 @@ def _check_grad(grad_output, shape, dtype):
 # BACKWARD_WORKSPACE_LIMIT bytes, and of what is free on the device at the time (memory torch holds
 # in its cache counted as free) no more than BACKWARD_WORKSPACE_FREE_FRACTION.
 BACKWARD_RECORDS_PER_RAY = 30
+# Batches of fewer than 2^20 rays get up to four times that room per ray (the workspace stays below what
+# 2^20 rays take, 768 MiB): a launch lasts as long as its longest ray, so the few rays of a small batch whose
+# notes do not fit cost their backward pass a whole march (4 096 rays through a dense 16^3 tree, 26 of them
+# without room: 213 us instead of 55).
+SMALL_BATCH_ROOM = 4
 BACKWARD_WORKSPACE_LIMIT = 4 << 30
 BACKWARD_WORKSPACE_FREE_FRACTION = 0.25
 _ASK_DEVICE_ABOVE = 64 << 20   # smaller workspaces are taken without asking the device what is free
@@ -475,6 +480,7 @@ def _backward_workspace(tree, n_rays, records_per_ray=None):
         return None, 0
     size_of = _abi.load_library().svox_volume_render_backward_workspace_bytes
     per_ray = int(BACKWARD_RECORDS_PER_RAY if records_per_ray is None else records_per_ray)
+    per_ray *= max(1, min(int(SMALL_BATCH_ROOM), (1 << 20) // int(n_rays)))
     limit = BACKWARD_WORKSPACE_LIMIT
     if size_of(n_rays, per_ray) > _ASK_DEVICE_ABOVE:
         device = tree.data.device

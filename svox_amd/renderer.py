@@ -221,7 +221,8 @@ class VolumeRenderer(nn.Module):
 
     * A forward pass that will be differentiated (gradient mode on, `tree.data.requires_grad`) keeps
       notes of the leaves its rays met until `backward()` has run: 768 bytes per ray to begin with (30
-      leaves per ray on average; 3.9 GB for eight 800x800 images); a pass whose notes ran out of room
+      leaves per ray on average; 3.9 GB for eight 800x800 images; batches below 2^20 rays get up to four
+      times the room per ray, `csrc.SMALL_BATCH_ROOM`); a pass whose notes ran out of room
       doubles the room of the next passes, up to 16 times, and passes that leave most of it unused
       halve it again (`renderer.notes_budget`, a `NotesBudget`).  At most
       `csrc.BACKWARD_WORKSPACE_LIMIT` (4 GiB) and at most a quarter of the device memory that is free

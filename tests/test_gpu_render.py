@@ -338,6 +338,7 @@ def test_backward_workspace_sizes(gpu, oracle_mod, fmt, monkeypatch):
     assert stats["samples_bwd_pos"] > 8 * 6000          # many rays have more than 4 and 8 such leaves
     dev = on_gpu(tree, gpu)
     rs = rays_spec(rays, gpu)
+    monkeypatch.setattr(C, "SMALL_BATCH_ROOM", 1)     # (the sizes below are meant as they stand)
     for per_ray in (0, 15, 30, 90):      # no workspace; first chunks only; some / plenty of shared chunks
         monkeypatch.setattr(C, "BACKWARD_RECORDS_PER_RAY", per_ray)
         got = C.volume_render_backward(dev._spec(), rs, opt, go.to(gpu), workspace=per_ray > 0).cpu().numpy()
@@ -442,6 +443,7 @@ def test_noted_forward_and_backward_from_notes(gpu, oracle_mod, fmt, fast, persi
     rs = rays_spec(rays, gpu)
     C.set_debug_flags(2 if persistent else 0)
     try:
+        monkeypatch.setattr(C, "SMALL_BATCH_ROOM", 1)     # (the sizes below are meant as they stand)
         for per_ray in (30, 15):
             monkeypatch.setattr(C, "BACKWARD_RECORDS_PER_RAY", per_ray)
             out, notes = C.volume_render_noted(dev._spec(), rs, opt)
@@ -459,10 +461,11 @@ def test_noted_forward_and_backward_from_notes(gpu, oracle_mod, fmt, fast, persi
         C.set_debug_flags(0)
 
 
-def test_notes_budget_follows_the_scene(gpu, oracle_mod):
+def test_notes_budget_follows_the_scene(gpu, oracle_mod, monkeypatch):
     """Rays through a dense tree meet more leaves with density than the starting room for notes holds:
     the first training step loses notes (those rays are marched: same gradient), the renderer gives
     the next steps more room until nothing is lost, and takes it back for rays that need none."""
+    monkeypatch.setattr(C, "SMALL_BATCH_ROOM", 1)     # (without the extra room a batch this small starts with)
     tree = synth.dense_tree(5, "SH4", seed=3, sigma="lognormal", coeff_std=0.5, zero_fraction=0.0)
     rays = synth.sphere_rays(3000, seed=5)
     opt = options(tree, step_size=1e-3)
@@ -759,6 +762,10 @@ def test_workspace_and_marking_thresholds_from_both_sides(gpu, monkeypatch):
     tree = on_gpu(synth.shell_tree(depth=5, n_spheres=4, data_format="SH4", seed=5, sigma_range=(20.0, 200.0)), gpu)
     n = 4096
     size_of = C._abi.load_library().svox_volume_render_backward_workspace_bytes
+    assert C._backward_workspace(tree, n)[1] == size_of(n, 120)        # (a small batch: four times the room)
+    assert C._backward_workspace(tree, 1 << 19)[1] == size_of(1 << 19, 60)
+    assert C._backward_workspace(tree, (1 << 19) + 1)[1] == size_of((1 << 19) + 1, 30)
+    monkeypatch.setattr(C, "SMALL_BATCH_ROOM", 1)
     assert C._backward_workspace(tree, n)[1] == size_of(n, 30)
     monkeypatch.setattr(C, "BACKWARD_WORKSPACE_LIMIT", size_of(n, 30) - 1)
     assert C._backward_workspace(tree, n)[1] == size_of(n, 15)
