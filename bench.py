@@ -405,14 +405,18 @@ def main():
             tree.data.grad = None
             renderer.render_persp(poses[0], width=W, height=H, fx=fx, fast=True).backward(igo)
 
-        def timed(fn, n=3):
+        def timed(fn, n=5):
+            # median of n steps queued back to back, an event between every two (a process now and then
+            # stalls for tens of milliseconds once, early on: a mean over a few steps would carry that)
             fn()
             torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(n):
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+            marks[0].record()
+            for i in range(n):
                 fn()
+                marks[i + 1].record()
             torch.cuda.synchronize()
-            return (time.perf_counter() - t0) * 1e3 / n
+            return float(np.median([marks[i].elapsed_time(marks[i + 1]) for i in range(n)]))
 
         itarget = torch.rand(H, W, 3, generator=g).to(dev)
         fwd_bwd["image_pose"] = {
