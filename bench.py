@@ -371,6 +371,38 @@ def main():
             "samples_per_ray": round(train_stats["samples_bwd"] / B, 2),
             "positive_per_ray": round(train_stats["samples_bwd_pos"] / B, 2),
         }
+        # The gradient records reach memory as fp32 atomic adds, K scalars per leaf with density: what the
+        # memory system takes of those is measured by the library's atomic probe (wavefronts adding to runs
+        # of 16 consecutive floats, one 64-byte request each, at random places of a scratch the size of the
+        # gradient).  A record of K floats at a K-float stride lies in (4 K + 60) / 64 such pieces on average.
+        scratch = torch.zeros_like(tree.data).view(-1)
+        C.atomic_probe(scratch, run_floats=16, iters=8)
+        torch.cuda.synchronize()
+        pa, pb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        pa.record()
+        _, probe_requests = C.atomic_probe(scratch, run_floats=16, iters=512)
+        pb.record()
+        torch.cuda.synchronize()
+        atomic_requests_per_us = probe_requests / (pa.elapsed_time(pb) * 1e3)
+        za, zb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        za.record()
+        scratch.zero_()
+        zb.record()
+        torch.cuda.synchronize()
+        zero_ms = za.elapsed_time(zb)
+        del scratch
+        records = int(train_stats["samples_bwd_pos"])
+        record_requests = records * (4 * K + 60) / 64
+        fwd_bwd["atomics"] = {
+            "probe_requests_per_us": round(atomic_requests_per_us, 1),
+            "records": records, "requests_per_record": round((4 * K + 60) / 64, 2),
+            "ms_at_probe_rate": round(record_requests / atomic_requests_per_us / 1e3, 4),
+            "backward_ms_without_zero_fill": round(bwd_ms - zero_ms, 4),
+            "frac_of_probe_rate": round(record_requests / atomic_requests_per_us / 1e3 / max(bwd_ms - zero_ms, 1e-9), 4),
+            "note": "64-byte atomic-add requests per microsecond the memory system takes (the same for 1, 4 or 16 "
+                    "floats per request and for a scratch of 2 MiB or 2 GiB), and the time the records of this "
+                    "step's backward pass would take at that rate",
+        }
         tree.data.grad = None
         # the squared-error step on the same rays: colour, gradient and Hessian diagonal in one call
         target = torch.rand(B, 3, generator=g).to(dev)

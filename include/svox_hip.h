@@ -353,6 +353,15 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
 int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t iters, int32_t blocks,
                       void* sink, void* stream);
 
+/* No counterpart in the reference; the measurement aid for the backward kernels, whose gradient records
+ * reach memory as fp32 atomic adds.  `blocks` blocks of 256 lanes; in each of `iters` rounds the 64 lanes
+ * of a wavefront add 1.0f to 64 / run_floats runs of `run_floats` consecutive floats (1, 4, 16 or 64; a run
+ * of 16 floats that starts on a 64-byte boundary is one 64-byte request) at pseudo-random run-aligned
+ * places of scratch[0, bytes), which the caller gives up to the probe (float contents are changed).
+ * The caller times the call: blocks * 256 * iters adds in blocks * 256 * iters / min(run_floats, 16)
+ * requests. */
+int svox_atomic_probe(void* scratch, int64_t bytes, int32_t run_floats, int32_t iters, int32_t blocks, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -729,6 +729,20 @@ def gather_probe(buffer, unit_bytes=64, iters=64, blocks=2048):
     return int(blocks) * 256 * 4 * int(iters)
 
 
+def atomic_probe(scratch, run_floats=16, iters=64, blocks=4096):
+    """Queues the library's atomic-add probe on `scratch` (a contiguous float32 CUDA tensor whose contents are
+    given up): blocks * 256 lanes, each adding 1.0f `iters` times, the lanes of a wavefront to runs of
+    `run_floats` consecutive floats at pseudo-random places.  Returns (adds, 64-byte requests); the caller
+    times the call (a measurement aid for the ceiling of the backward kernels' atomics)."""
+    if not scratch.is_contiguous() or scratch.dtype != torch.float32:
+        raise ValueError("atomic_probe: scratch must be a contiguous float32 tensor")
+    with torch.cuda.device(scratch.device):
+        _call("svox_atomic_probe", scratch.data_ptr(), scratch.numel() * 4, int(run_floats), int(iters), int(blocks),
+              _stream(scratch.device))
+    adds = int(blocks) * 256 * int(iters)
+    return adds, adds // min(int(run_floats), 16)
+
+
 def set_debug_flags(flags):
     """bit 0: route every call to the generic kernels; bit 1: small ray batches run like large ones;
     bit 2 / bit 3: forward renders never / always take the two-wavefront kernel"""

@@ -208,6 +208,20 @@ __global__ __launch_bounds__(256) void gather_probe_kernel(const uint4* __restri
     if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) sink[blockIdx.x * 256u + threadIdx.x] = acc;
 }
 
+// Measurement aid (svox_atomic_probe): per round the wavefront adds 1.0f to 64 / run consecutive-float runs
+// at pseudo-random run-aligned places.
+__global__ __launch_bounds__(256) void atomic_probe_kernel(float* __restrict__ scratch, uint64_t n_runs, int run,
+                                                           int iters) {
+    const int lane = threadIdx.x & 63;
+    uint32_t seed = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 977u;
+    for (int it = 0; it < iters; ++it) {
+        seed = probe_hash(seed + 0x9e3779b9u);
+        const uint32_t s = probe_hash(seed + (uint32_t)(lane / run));
+        const uint64_t at = ((uint64_t)s * n_runs) >> 32;
+        atomicAdd(scratch + at * (uint64_t)run + (lane % run), 1.0f);
+    }
+}
+
 // calc_corner_kernel, svox_kernel.cu:91-115: climb parent links from the leaf's node to the
 // root; per level result = (result + cell index) / N.
 template <typename T>

@@ -1250,5 +1250,18 @@ int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int
     return check_launch("gather_probe");
 }
 
+int svox_atomic_probe(void* scratch, int64_t bytes, int32_t run_floats, int32_t iters, int32_t blocks, void* stream) {
+    if (!scratch) return fail(SVOX_ERR_NULL_POINTER, "svox_atomic_probe: NULL scratch");
+    if (run_floats != 1 && run_floats != 4 && run_floats != 16 && run_floats != 64)
+        return fail(SVOX_ERR_BAD_SHAPE, "svox_atomic_probe: run_floats must be 1, 4, 16 or 64");
+    const int64_t n_runs = bytes / (4 * (int64_t)run_floats);
+    if (((uintptr_t)scratch & 63u) || n_runs < 1 || n_runs > 0xffffffffll || iters < 1 || blocks < 1 ||
+        blocks > (1 << 20))
+        return fail(SVOX_ERR_BAD_SHAPE, "svox_atomic_probe: scratch (64-byte aligned), iters or blocks out of range");
+    hipLaunchKernelGGL(atomic_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (float*)scratch, (uint64_t)n_runs, run_floats, iters);
+    return check_launch("atomic_probe");
+}
+
 }  // extern "C"
 #pragma GCC visibility pop

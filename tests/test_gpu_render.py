@@ -943,3 +943,17 @@ def test_a_training_step_replays_from_a_hip_graph(gpu):
         err, ok = grad_close(tree.data.detach().cpu().numpy(), eager_data[i].cpu().numpy(), rel=1e-5)
         assert ok, (i, err)
         assert float((torch.rand(1000, device=gpu) * 2).sum()) > 0          # eager work between the replays
+
+
+def test_atomic_probe_adds_what_it_says(gpu):
+    """The measurement aid for atomics: every add is 1.0f, so the scratch sums to the number of adds."""
+    scratch = torch.zeros(1 << 16, dtype=torch.float32, device=gpu)
+    adds, requests = C.atomic_probe(scratch, run_floats=16, iters=5, blocks=3)
+    assert adds == 3 * 256 * 5 and requests == adds // 16
+    assert float(scratch.double().sum()) == adds
+    adds, requests = C.atomic_probe(scratch, run_floats=1, iters=2, blocks=2)
+    assert requests == adds
+    with pytest.raises(RuntimeError):
+        C.atomic_probe(scratch, run_floats=3)
+    with pytest.raises(RuntimeError):
+        C.atomic_probe(scratch[1:17], run_floats=16)       # not 64-byte aligned
