@@ -342,6 +342,13 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
                              const SvoxCameraSpec* cam, const SvoxRenderOptions* opt,
                              SvoxMarchStats* stats_out, void* stream);
 
+/* No counterpart in the reference.  Which family of kernels serves the render calls of this tree under
+ * these options: 1 the wavefront-per-tile octree kernels (fp32, N = 2, RGBA / SH / SG records with basis_dim
+ * 1, 4, 9, 16 or 25 and the full component range), 0 the one-ray-per-lane kernels that cover everything
+ * else the reference accepts (fp64, ASG, other N, other basis sizes, partial component ranges), or a
+ * negative SvoxStatus for a tree or options no kernel accepts.  Results do not depend on the family. */
+int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt);
+
 /* No counterpart in the reference; a measurement aid.  The march kernels read scattered 64-byte
  * pieces of the tree, and how many such requests per microsecond the memory system serves is the
  * ceiling their launches run against.  This launch measures it: `blocks` blocks of 256 lanes, every

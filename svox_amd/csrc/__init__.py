@@ -716,6 +716,18 @@ def volume_render_stats(tree, rays_or_cam, opt):
     return {n: int(v) for n, v in zip(names, vals) if n != "reserved"}
 
 
+def octree_kernels_serve(tree, opt):
+    """True where the wavefront-per-tile octree kernels serve the render calls of `tree` under `opt`, False
+    where the one-ray-per-lane kernels do (fp64, ASG, N != 2, other basis sizes, partial component ranges)."""
+    spec = _pack_tree(tree)
+    copt = opt._pack()
+    rc = _abi.load_library().svox_octree_kernels_serve(ctypes.byref(spec), ctypes.byref(copt))
+    if rc < 0:
+        lib = _abi.load_library()
+        raise RuntimeError(f"svox.octree_kernels_serve: {lib.svox_last_error().decode('utf-8', 'replace')}")
+    return bool(rc)
+
+
 def gather_probe(buffer, unit_bytes=64, iters=64, blocks=2048):
     """Queues the library's gather probe on `buffer` (a contiguous CUDA tensor): blocks * 256 lanes, each
     reading 16 bytes of 4 * iters pseudo-random `unit_bytes`-sized units.  Returns the number of reads;

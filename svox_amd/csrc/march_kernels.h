@@ -378,10 +378,28 @@ template <int FMT, int D>
 struct OctreePolicy {
     using scalar = float;
     static constexpr bool kOctree = true;
-    static constexpr int kFormat = FMT;
+    static constexpr int kFormat = FMT;                                // RGBA, SH or SG
     static constexpr int kBasis = D;                                   // 0 for RGBA
     static constexpr int kRecord = (FMT == SVOX_FORMAT_RGBA) ? 4 : 3 * D + 1;
+    // SH: the basis is a closed form of the view direction, cheap enough to evaluate again wherever a
+    // colour is formed; SG: D exponentials, evaluated once per ray and kept as a row in LDS
+    static constexpr bool kForwardRows = FMT == SVOX_FORMAT_SG;
 };
+
+// The table of lobes of a spherical-gaussian tree (TreeSpec.extra_data: basis_dim rows [lambda, mu]).
+struct Lobes {
+    const float* table;
+    int cols;
+};
+// The basis of one ray (maybe_precalc_basis, rt_kernel.cu:111-187) for the policy's format.
+template <class P>
+__device__ __forceinline__ void policy_basis(const Lobes& lobes, const float* vdir, float* out) {
+    if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+        sh_basis<float>(P::kBasis, vdir, out);
+    } else {
+        precalc_basis<float>(P::kFormat, P::kBasis, lobes.table, lobes.cols, vdir, out);
+    }
+}
 
 // atomicMax of the reference (common.cuh:152-172): compare-and-swap loop around fmaxf
 __device__ __forceinline__ void atomic_max_float(float* addr, float value) {
@@ -841,7 +859,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
-    __shared__ ShadeShared<D, false> sh;
+    __shared__ ShadeShared<D, P::kForwardRows> sh;
     const int lane = threadIdx.x;
     float offset[3], scaling[3];
     load_transform(tr, offset, scaling);
@@ -880,6 +898,11 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                 sh.vdir[lane * 3] = vdir[0];
                 sh.vdir[lane * 3 + 1] = vdir[1];
                 sh.vdir[lane * 3 + 2] = vdir[2];
+            } else if constexpr (P::kForwardRows) {
+                float basis[D];
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols}, vdir, basis);
+#pragma unroll
+                for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
             acc[0] = acc[1] = acc[2] = 0.0f;
             light = 1.0f;
@@ -929,7 +952,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         bool stopped = false;
         if (n_entries > 0) {   // most rounds of a ray pass through empty space: nothing to shade
             wave_lds_sync();   // list and view directions are visible to every lane
-            shade_entries<P, false>(tr.data, sh, n_entries, lane);
+            shade_entries<P, P::kForwardRows>(tr.data, sh, n_entries, lane);
             wave_lds_sync();
             // ---- composite
             // the attenuations and padded colours of the four slots do not depend on one another: they
@@ -1480,7 +1503,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
-    __shared__ ShadeShared<D, false> sh;
+    __shared__ ShadeShared<D, P::kForwardRows> sh;
     __shared__ SplitBox box;
     if constexpr (kNoted) {
         if (blockIdx.x == 0 && threadIdx.x < kStampWords) ws.stamp_at[threadIdx.x] = ws.stamp[threadIdx.x];
@@ -1516,6 +1539,13 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
                     sh.vdir[lane * 3] = vdir[0];
                     sh.vdir[lane * 3 + 1] = vdir[1];
                     sh.vdir[lane * 3 + 2] = vdir[2];
+                }
+            } else if constexpr (P::kForwardRows) {
+                if (active) {
+                    float basis[D];
+                    policy_basis<P>(Lobes{tr.extra, tr.extra_cols}, vdir, basis);
+#pragma unroll
+                    for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
                 }
             }
         }
@@ -1634,7 +1664,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         bool stopped = false;
         if (n_entries > 0) {
             wave_lds_sync();
-            shade_entries<P, false>(tr.data, sh, n_entries, lane);
+            shade_entries<P, P::kForwardRows>(tr.data, sh, n_entries, lane);
             wave_lds_sync();
             float q_att[kQueue], q_rgb[kQueue][3], q_s[kQueue][3];
 #pragma unroll
@@ -1731,9 +1761,9 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                 if (head[1].y != 0.0f) return;
                 march1_sum = head[2].x;
             }
-            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+            if constexpr (P::kFormat != SVOX_FORMAT_RGBA) {
                 float basis[D];
-                sh_basis<float>(P::kBasis, vdir, basis);
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols}, vdir, basis);
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
@@ -1852,7 +1882,7 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
                                                                         const float* __restrict__ grad_out,
                                                                         float* __restrict__ grad_data,
                                                                         ReplaySpace ws, int ray_shift,
-                                                                        int march1_known) {
+                                                                        int march1_known, Lobes lobes) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     __shared__ ShadeShared<D, true> sh;
     const int lane = threadIdx.x;
@@ -1889,11 +1919,11 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     float go[3] = {0.f, 0.f, 0.f};
     if (work) {
-        if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+        if constexpr (P::kFormat != SVOX_FORMAT_RGBA) {
             float vdir[3];
             src.view_dir(ray, vdir);
             float basis[D];
-            sh_basis<float>(P::kBasis, vdir, basis);
+            policy_basis<P>(lobes, vdir, basis);
 #pragma unroll
             for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
         }
@@ -2187,9 +2217,9 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         if (slot < 0) return;
         if (!Source::kItemsAreSlots && only && !((only[slot >> 6] >> (slot & 63)) & 1ull)) return;
         if (setup_ray(r, origin, dir, scaling)) {
-            if constexpr (P::kFormat == SVOX_FORMAT_SH) {
+            if constexpr (P::kFormat != SVOX_FORMAT_RGBA) {
                 float basis[D];
-                sh_basis<float>(P::kBasis, vdir, basis);
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols}, vdir, basis);
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
@@ -2357,7 +2387,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
                                                                        float* __restrict__ color_out,
                                                                        float* __restrict__ grad_data,
                                                                        float* __restrict__ hess_data,
-                                                                       ReplaySpace ws, int ray_shift) {
+                                                                       ReplaySpace ws, int ray_shift, Lobes lobes) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     constexpr bool kRgba = P::kFormat == SVOX_FORMAT_RGBA;
@@ -2412,7 +2442,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
             float vdir[3];
             src.view_dir(ray, vdir);
             float basis[D];
-            sh_basis<float>(P::kBasis, vdir, basis);
+            policy_basis<P>(lobes, vdir, basis);
 #pragma unroll
             for (int i = 0; i < D; ++i) basis_rows[lane * D + i] = basis[i];
         }

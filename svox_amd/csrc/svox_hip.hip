@@ -178,16 +178,26 @@ int check_rays(const SvoxRaysSpec* rays) {
 }
 
 // default options on an fp32 octree whose record matches the format: the specialised kernels
-// (density_softplus only in the forward kernel: `softplus_ok`)
+// (density_softplus only in the forward kernel: `softplus_ok`).  Returns what SVOX_DISPATCH_OCTREE
+// switches on: 0 for RGBA, basis_dim for spherical harmonics, kLobeKernels + basis_dim for spherical
+// gaussians, -1 for everything the generic kernels serve.
+constexpr int kLobeKernels = 100;
 int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, bool softplus_ok = false) {
     if (!octree_fast_ok(tree) || (opt->density_softplus && !softplus_ok)) return -1;
     if (opt->format == SVOX_FORMAT_RGBA) return tree->data_dim == 4 ? 0 : -1;
-    if (opt->format != SVOX_FORMAT_SH) return -1;
+    if (opt->format != SVOX_FORMAT_SH && opt->format != SVOX_FORMAT_SG) return -1;
     const int D = opt->basis_dim;
     if (D != 1 && D != 4 && D != 9 && D != 16 && D != 25) return -1;
     if (tree->data_dim != 3 * D + 1 || opt->min_comp != 0 || opt->max_comp != D - 1) return -1;
+    if (opt->format == SVOX_FORMAT_SG) {
+        // spherical gaussians: the table of lobes must be there, [lambda, mu, ...] per lobe (rt_kernel.cu:133-139)
+        if (!tree->extra_data || tree->extra_rows < D || tree->extra_cols < 4) return -1;
+        return kLobeKernels + D;
+    }
     return D;
 }
+
+Lobes lobes_of(const SvoxTreeSpec* tree) { return Lobes{(const float*)tree->extra_data, tree->extra_cols}; }
 
 // The tree as the octree march kernels see it: with the caller's marks of the empty leaves in place
 // of the child table where they apply (no leaf with sigma <= 0 may contribute: sigma_thresh >= 0).
@@ -316,7 +326,12 @@ unsigned blocks_for(int64_t items, int per_block) { return (unsigned)((items + p
         case 4: { using P = OctreePolicy<SVOX_FORMAT_SH, 4>; __VA_ARGS__; } break;   \
         case 9: { using P = OctreePolicy<SVOX_FORMAT_SH, 9>; __VA_ARGS__; } break;   \
         case 16: { using P = OctreePolicy<SVOX_FORMAT_SH, 16>; __VA_ARGS__; } break; \
-        default: { using P = OctreePolicy<SVOX_FORMAT_SH, 25>; __VA_ARGS__; } break; \
+        case 25: { using P = OctreePolicy<SVOX_FORMAT_SH, 25>; __VA_ARGS__; } break; \
+        case kLobeKernels + 1: { using P = OctreePolicy<SVOX_FORMAT_SG, 1>; __VA_ARGS__; } break;   \
+        case kLobeKernels + 4: { using P = OctreePolicy<SVOX_FORMAT_SG, 4>; __VA_ARGS__; } break;   \
+        case kLobeKernels + 9: { using P = OctreePolicy<SVOX_FORMAT_SG, 9>; __VA_ARGS__; } break;   \
+        case kLobeKernels + 16: { using P = OctreePolicy<SVOX_FORMAT_SG, 16>; __VA_ARGS__; } break; \
+        default: { using P = OctreePolicy<SVOX_FORMAT_SG, 25>; __VA_ARGS__; } break; \
     }
 
 // Whether a forward launch of `blocks` 64-ray wavefronts takes render_forward_split_kernel (two
@@ -629,7 +644,7 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P, Source>), dim3(waves), dim3(kMarchThreads), 0,
                                                stream, all, *opt, (const float*)grad_output, (float*)grad_data_out, ws,
-                                               ray_shift, march1_known ? 1 : 0));
+                                               ray_shift, march1_known ? 1 : 0, lobes_of(tree)));
     int rc = check_launch("volume_render_backward_noted");
     if (rc) return rc;
     ReplaySpace only{};
@@ -700,7 +715,8 @@ int se_grad_from_notes(const SvoxTreeSpec* tree, const Source& all, const Source
     const int ray_shift = replay_ray_shift(is_image_source(all), n_slots);
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_se_grad_kernel<P, Source>), dim3(blocks_for(n_slots, 1 << ray_shift)),
                                                dim3(kMarchThreads), 0, stream, all, *opt, (const float*)color_ref,
-                                               (float*)color_out, (float*)grad, (float*)hess, ws, ray_shift));
+                                               (float*)color_out, (float*)grad, (float*)hess, ws, ray_shift,
+                                               lobes_of(tree)));
     rc = check_launch("se_grad");
     if (rc) return rc;
     launch_se_grad<Source, float>(tree, rest, opt, 3, color_ref, color_out, grad, hess, stream, ws.undone);
@@ -1235,6 +1251,13 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
         }
     }
     return check_launch("volume_render_stats");
+}
+
+int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
+    int od;
+    const int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    return fast_basis(tree, opt, true) >= 0 ? 1 : 0;
 }
 
 int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t iters, int32_t blocks,

@@ -1,0 +1,98 @@
+"""Spherical-gaussian trees (data_format SGn, svox/helpers.py:384-437; basis rt_kernel.cu:133-139) on the
+wavefront-per-tile octree kernels: every render path against the oracle, for the basis sizes those kernels
+are built for, and the hand-over to the one-ray-per-lane kernels for the sizes they are not.
+
+Bars: pictures bit for bit, gradients within 1e-4 relative (util.grad_close)."""
+import numpy as np
+import pytest
+import torch
+
+import svox_amd as svox
+from svox_amd import csrc as C
+from svox_amd import synth
+from util import cam_spec, grad_close, on_gpu, options, rays_spec
+
+pytestmark = pytest.mark.gpu
+
+
+def lobe_tree(n_lobes, seed, depth=6):
+    """A sparse shell tree whose records are read as n_lobes spherical gaussians."""
+    tree = synth.shell_tree(depth=depth, n_spheres=5, data_format=f"SG{n_lobes}", seed=seed, sigma_range=(5.0, 80.0))
+    g = torch.Generator().manual_seed(seed + 17)
+    lobes = torch.cat([torch.rand(n_lobes, 1, generator=g) * 4, synth.unit_vectors(n_lobes, g)], dim=1)
+    del tree.extra_data
+    tree.register_buffer("extra_data", lobes)
+    return tree
+
+
+@pytest.mark.parametrize("n_lobes", [1, 4, 9, 16, 25])
+def test_spherical_gaussians_on_the_octree_kernels(gpu, oracle_mod, n_lobes):
+    tree = lobe_tree(n_lobes, seed=3 + n_lobes)
+    n = 3000
+    rays = synth.sphere_rays(n, seed=4)
+    W, H, fx = 70, 50, 60.0
+    poses = synth.orbit_poses(2, seed=6, radius=2.5)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    go = torch.randn(n, 3, generator=torch.Generator().manual_seed(5)) * 1e-2
+    gi = torch.randn(2, H, W, 3, generator=torch.Generator().manual_seed(6)) * 1e-2
+    ref = torch.rand(n, 3, generator=torch.Generator().manual_seed(7))
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    cam = cam_spec(torch.stack(poses).to(gpu), W, H, fx)
+    for fast in (True, False):
+        opt = options(tree, step_size=2e-3, fast=fast)
+        assert C.octree_kernels_serve(dev._spec(), opt)
+        want = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+        want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+        want_img = np.stack([oracle_mod.volume_render_image(ot, c2w, fx, fx, W, H, opt, n_threads=8) for c2w in poses])
+        want_gi = sum(oracle_mod.volume_render_image_backward(ot, c2w, fx, fx, W, H, opt, gi[i])
+                      for i, c2w in enumerate(poses))
+        want_se = oracle_mod.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, opt, n_threads=8)
+        plain = dev._spec()
+        marked = dev._spec()
+        marked.child_marks = C.mark_empty_leaves(plain)
+        for flags in (0, 2, 4, 8, 1):     # the library's choice; batches run like large ones; one / two wavefronts per tile; generic
+            for spec in (plain, marked):
+                C.set_debug_flags(flags)
+                try:
+                    tag = (n_lobes, fast, flags, spec is marked)
+                    assert np.array_equal(C.volume_render(spec, rs, opt).cpu().numpy(), want), tag
+                    assert np.array_equal(C.volume_render_images(spec, cam, opt).cpu().numpy(), want_img), tag
+                    out, notes = C.volume_render_noted(spec, rs, opt)
+                    assert np.array_equal(out.cpu().numpy(), want), tag
+                    for got in (C.volume_render_backward_noted(spec, rs, opt, go.to(gpu), notes),
+                                C.volume_render_backward(spec, rs, opt, go.to(gpu), workspace=True),
+                                C.volume_render_backward(spec, rs, opt, go.to(gpu), workspace=False)):
+                        err, ok = grad_close(got.cpu().numpy(), want_g)
+                        assert ok, (tag, err)
+                    for workspace in (True, False):
+                        got = C.volume_render_images_backward(spec, cam, opt, gi.to(gpu), workspace=workspace)
+                        err, ok = grad_close(got.cpu().numpy(), want_gi)
+                        assert ok, (tag, "image", workspace, err)
+                        se = C.se_grad(spec, rs, ref.to(gpu), opt, workspace=workspace)
+                        assert np.array_equal(se[0].cpu().numpy(), want_se[0]), (tag, "se colour", workspace)
+                        for k in (1, 2):
+                            err, ok = grad_close(se[k].cpu().numpy(), want_se[k])
+                            assert ok, (tag, "se", k, workspace, err)
+                finally:
+                    C.set_debug_flags(0)
+
+
+def test_which_kernels_serve_which_trees(gpu):
+    """The octree kernels take fp32 octrees with RGBA, SH or SG records of 1, 4, 9, 16 or 25 basis functions
+    and the full component range; everything else goes to the one-ray-per-lane kernels."""
+    def serve(tree, **kw):
+        dev = on_gpu(tree, gpu)
+        return C.octree_kernels_serve(dev._spec(), options(tree, **kw))
+    assert serve(synth.dense_tree(2, "RGBA", seed=1))
+    assert serve(synth.dense_tree(2, "SH9", seed=1))
+    assert serve(synth.dense_tree(2, "SH9", seed=1), density_softplus=True)
+    assert not serve(synth.dense_tree(2, "SH9", seed=1), min_comp=1, max_comp=3)
+    assert not serve(synth.dense_tree(2, "SH4", seed=1, dtype=torch.float64))
+    assert serve(lobe_tree(9, seed=2, depth=4))
+    assert not serve(lobe_tree(5, seed=2, depth=4))                       # no kernel built for five lobes
+    g = torch.Generator().manual_seed(1)
+    frames = torch.linalg.qr(torch.randn(4, 3, 3, generator=g))[0].reshape(4, 9)
+    asg = svox.N3Tree(data_format="ASG4", init_refine=1, extra_data=torch.cat([torch.rand(4, 2, generator=g) * 3, frames], 1))
+    assert not serve(asg)
+    assert not serve(svox.N3Tree(N=3, data_format="SH4", init_refine=1))
