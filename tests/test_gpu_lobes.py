@@ -96,3 +96,37 @@ def test_which_kernels_serve_which_trees(gpu):
     asg = svox.N3Tree(data_format="ASG4", init_refine=1, extra_data=torch.cat([torch.rand(4, 2, generator=g) * 3, frames], 1))
     assert not serve(asg)
     assert not serve(svox.N3Tree(N=3, data_format="SH4", init_refine=1))
+
+
+@pytest.mark.parametrize("op", ["sum", "max"])
+def test_weight_accumulation_on_a_spherical_gaussian_tree(gpu, oracle_mod, op):
+    """accumulate_weights (svox/svox.py:1136-1158, rt_kernel.cu:298-304) through the octree forward kernel
+    of the spherical-gaussian policy, and the Python renderer end to end (autograd included)."""
+    tree = lobe_tree(9, seed=21)
+    rays = synth.sphere_rays(2000, seed=8)
+    opt = options(tree, step_size=2e-3, fast=True)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    ot.weight_accum = np.zeros(tree.child.shape, dtype=np.float32)
+    ot.weight_accum_max = op == "max"
+    want = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    assert ot.weight_accum.max() > 0
+    dev = on_gpu(tree, gpu)
+    dev.data.requires_grad_(True)
+    renderer = svox.VolumeRenderer(dev, step_size=2e-3)
+    dev_rays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu))
+    with torch.no_grad():
+        with dev.accumulate_weights(op=op) as accum:
+            out = renderer(dev_rays, fast=True)
+            got = accum.value.cpu().numpy()
+    assert np.array_equal(out.cpu().numpy(), want)
+    if op == "max":
+        assert np.array_equal(got, ot.weight_accum)
+    else:
+        assert np.abs(got - ot.weight_accum).max() <= 1e-5 * max(1.0, np.abs(ot.weight_accum).max())
+    # the gradient through autograd (notes taken by the forward pass)
+    go = torch.randn(2000, 3, generator=torch.Generator().manual_seed(4)) * 1e-2
+    ot.weight_accum = None
+    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    renderer(dev_rays, fast=True).backward(go.to(gpu))
+    err, ok = grad_close(dev.data.grad.cpu().numpy(), want_g)
+    assert ok, err
