@@ -624,9 +624,9 @@ def main():
                     ev_time(lambda: C.volume_render_image(sgtree._spec(), gcam, sg_opt)), 4)
             finally:
                 C.set_debug_flags(0)
-        generic["note"] = ("fp32 SH and SG records of 1, 4, 9, 16 or 25 basis functions run on the octree kernels "
+        generic["note"] = ("fp32 SH, SG and ASG records of 1, 4, 9, 16 or 25 basis functions run on the octree kernels "
                            "(`..._generic_kernel_ms`: the same call forced onto the one-ray-per-lane kernels, which "
-                           "serve fp64, ASG and the other shapes)")
+                           "serve fp64 and the other shapes)")
         del sgtree
         gtree64 = gtree.double()
         g64cam = _make_camera_spec(poses[0].double().contiguous(), W, H, fx, fx)

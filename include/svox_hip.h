@@ -343,9 +343,9 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
                              SvoxMarchStats* stats_out, void* stream);
 
 /* No counterpart in the reference.  Which family of kernels serves the render calls of this tree under
- * these options: 1 the wavefront-per-tile octree kernels (fp32, N = 2, RGBA / SH / SG records with basis_dim
- * 1, 4, 9, 16 or 25 and the full component range), 0 the one-ray-per-lane kernels that cover everything
- * else the reference accepts (fp64, ASG, other N, other basis sizes, partial component ranges), or a
+ * these options: 1 the wavefront-per-tile octree kernels (fp32, N = 2, RGBA / SH / SG / ASG records with
+ * basis_dim 1, 4, 9, 16 or 25 and the full component range), 0 the one-ray-per-lane kernels that cover
+ * everything else the reference accepts (fp64, other N, other basis sizes, partial component ranges), or a
  * negative SvoxStatus for a tree or options no kernel accepts.  Results do not depend on the family. */
 int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt);
 

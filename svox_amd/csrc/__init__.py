@@ -718,7 +718,7 @@ def volume_render_stats(tree, rays_or_cam, opt):
 
 def octree_kernels_serve(tree, opt):
     """True where the wavefront-per-tile octree kernels serve the render calls of `tree` under `opt`, False
-    where the one-ray-per-lane kernels do (fp64, ASG, N != 2, other basis sizes, partial component ranges)."""
+    where the one-ray-per-lane kernels do (fp64, N != 2, other basis sizes, partial component ranges)."""
     spec = _pack_tree(tree)
     copt = opt._pack()
     rc = _abi.load_library().svox_octree_kernels_serve(ctypes.byref(spec), ctypes.byref(copt))

@@ -378,18 +378,22 @@ template <int FMT, int D>
 struct OctreePolicy {
     using scalar = float;
     static constexpr bool kOctree = true;
-    static constexpr int kFormat = FMT;                                // RGBA, SH or SG
+    static constexpr int kFormat = FMT;                                // RGBA, SH, or SG for both kinds of lobes
     static constexpr int kBasis = D;                                   // 0 for RGBA
     static constexpr int kRecord = (FMT == SVOX_FORMAT_RGBA) ? 4 : 3 * D + 1;
     // SH: the basis is a closed form of the view direction, cheap enough to evaluate again wherever a
-    // colour is formed; SG: D exponentials, evaluated once per ray and kept as a row in LDS
+    // colour is formed; lobes (SG, ASG): D exponentials, evaluated once per ray and kept as a row in LDS
     static constexpr bool kForwardRows = FMT == SVOX_FORMAT_SG;
 };
 
-// The table of lobes of a spherical-gaussian tree (TreeSpec.extra_data: basis_dim rows [lambda, mu]).
+// The table of lobes of a tree of spherical gaussians (TreeSpec.extra_data: basis_dim rows [lambda, mu])
+// or anisotropic ones ([lambda_x, lambda_y, x-axis, y-axis, z-axis]), and which of the two it is: the two
+// formats differ in nothing but the basis of a ray, which is evaluated once per ray, so one set of
+// kernels (OctreePolicy<SVOX_FORMAT_SG, D>) serves both and looks at `format` there.
 struct Lobes {
     const float* table;
     int cols;
+    int format;
 };
 // The basis of one ray (maybe_precalc_basis, rt_kernel.cu:111-187) for the policy's format.
 template <class P>
@@ -397,7 +401,7 @@ __device__ __forceinline__ void policy_basis(const Lobes& lobes, const float* vd
     if constexpr (P::kFormat == SVOX_FORMAT_SH) {
         sh_basis<float>(P::kBasis, vdir, out);
     } else {
-        precalc_basis<float>(P::kFormat, P::kBasis, lobes.table, lobes.cols, vdir, out);
+        precalc_basis<float>(lobes.format, P::kBasis, lobes.table, lobes.cols, vdir, out);
     }
 }
 
@@ -900,7 +904,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                 sh.vdir[lane * 3 + 2] = vdir[2];
             } else if constexpr (P::kForwardRows) {
                 float basis[D];
-                policy_basis<P>(Lobes{tr.extra, tr.extra_cols}, vdir, basis);
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, vdir, basis);
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
@@ -1543,7 +1547,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
             } else if constexpr (P::kForwardRows) {
                 if (active) {
                     float basis[D];
-                    policy_basis<P>(Lobes{tr.extra, tr.extra_cols}, vdir, basis);
+                    policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, vdir, basis);
 #pragma unroll
                     for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
                 }
@@ -1763,7 +1767,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             }
             if constexpr (P::kFormat != SVOX_FORMAT_RGBA) {
                 float basis[D];
-                policy_basis<P>(Lobes{tr.extra, tr.extra_cols}, vdir, basis);
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, vdir, basis);
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
@@ -2219,7 +2223,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         if (setup_ray(r, origin, dir, scaling)) {
             if constexpr (P::kFormat != SVOX_FORMAT_RGBA) {
                 float basis[D];
-                policy_basis<P>(Lobes{tr.extra, tr.extra_cols}, vdir, basis);
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, vdir, basis);
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }

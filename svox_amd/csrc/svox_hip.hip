@@ -179,25 +179,29 @@ int check_rays(const SvoxRaysSpec* rays) {
 
 // default options on an fp32 octree whose record matches the format: the specialised kernels
 // (density_softplus only in the forward kernel: `softplus_ok`).  Returns what SVOX_DISPATCH_OCTREE
-// switches on: 0 for RGBA, basis_dim for spherical harmonics, kLobeKernels + basis_dim for spherical
-// gaussians, -1 for everything the generic kernels serve.
+// switches on: 0 for RGBA, basis_dim for spherical harmonics, kLobeKernels + basis_dim for lobes (spherical
+// gaussians and anisotropic ones), -1 for everything the generic kernels serve.
 constexpr int kLobeKernels = 100;
 int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, bool softplus_ok = false) {
     if (!octree_fast_ok(tree) || (opt->density_softplus && !softplus_ok)) return -1;
     if (opt->format == SVOX_FORMAT_RGBA) return tree->data_dim == 4 ? 0 : -1;
-    if (opt->format != SVOX_FORMAT_SH && opt->format != SVOX_FORMAT_SG) return -1;
+    if (opt->format != SVOX_FORMAT_SH && opt->format != SVOX_FORMAT_SG && opt->format != SVOX_FORMAT_ASG) return -1;
     const int D = opt->basis_dim;
     if (D != 1 && D != 4 && D != 9 && D != 16 && D != 25) return -1;
     if (tree->data_dim != 3 * D + 1 || opt->min_comp != 0 || opt->max_comp != D - 1) return -1;
-    if (opt->format == SVOX_FORMAT_SG) {
-        // spherical gaussians: the table of lobes must be there, [lambda, mu, ...] per lobe (rt_kernel.cu:133-139)
-        if (!tree->extra_data || tree->extra_rows < D || tree->extra_cols < 4) return -1;
+    if (opt->format != SVOX_FORMAT_SH) {
+        // lobes: the table must be there, [lambda, mu] per spherical gaussian (rt_kernel.cu:133-139),
+        // [lambda_x, lambda_y, three axes] per anisotropic one (rt_kernel.cu:120-131)
+        const int need = opt->format == SVOX_FORMAT_SG ? 4 : 11;
+        if (!tree->extra_data || tree->extra_rows < D || tree->extra_cols < need) return -1;
         return kLobeKernels + D;
     }
     return D;
 }
 
-Lobes lobes_of(const SvoxTreeSpec* tree) { return Lobes{(const float*)tree->extra_data, tree->extra_cols}; }
+Lobes lobes_of(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
+    return Lobes{(const float*)tree->extra_data, tree->extra_cols, opt->format};
+}
 
 // The tree as the octree march kernels see it: with the caller's marks of the empty leaves in place
 // of the child table where they apply (no leaf with sigma <= 0 may contribute: sigma_thresh >= 0).
@@ -644,7 +648,7 @@ int backward_from_notes(const SvoxTreeSpec* tree, const Source& all, Source rest
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_backward_kernel<P, Source>), dim3(waves), dim3(kMarchThreads), 0,
                                                stream, all, *opt, (const float*)grad_output, (float*)grad_data_out, ws,
-                                               ray_shift, march1_known ? 1 : 0, lobes_of(tree)));
+                                               ray_shift, march1_known ? 1 : 0, lobes_of(tree, opt)));
     int rc = check_launch("volume_render_backward_noted");
     if (rc) return rc;
     ReplaySpace only{};
@@ -716,7 +720,7 @@ int se_grad_from_notes(const SvoxTreeSpec* tree, const Source& all, const Source
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((replay_se_grad_kernel<P, Source>), dim3(blocks_for(n_slots, 1 << ray_shift)),
                                                dim3(kMarchThreads), 0, stream, all, *opt, (const float*)color_ref,
                                                (float*)color_out, (float*)grad, (float*)hess, ws, ray_shift,
-                                               lobes_of(tree)));
+                                               lobes_of(tree, opt)));
     rc = check_launch("se_grad");
     if (rc) return rc;
     launch_se_grad<Source, float>(tree, rest, opt, 3, color_ref, color_out, grad, hess, stream, ws.undone);

@@ -1,6 +1,7 @@
-"""Spherical-gaussian trees (data_format SGn, svox/helpers.py:384-437; basis rt_kernel.cu:133-139) on the
-wavefront-per-tile octree kernels: every render path against the oracle, for the basis sizes those kernels
-are built for, and the hand-over to the one-ray-per-lane kernels for the sizes they are not.
+"""Trees of lobes -- spherical gaussians (data_format SGn) and anisotropic ones (ASGn), svox/helpers.py:384-437;
+bases rt_kernel.cu:120-139 -- on the wavefront-per-tile octree kernels: every render path against the oracle,
+for the basis sizes those kernels are built for, and the hand-over to the one-ray-per-lane kernels for the
+sizes they are not.
 
 Bars: pictures bit for bit, gradients within 1e-4 relative (util.grad_close)."""
 import numpy as np
@@ -15,19 +16,25 @@ from util import cam_spec, grad_close, on_gpu, options, rays_spec
 pytestmark = pytest.mark.gpu
 
 
-def lobe_tree(n_lobes, seed, depth=6):
-    """A sparse shell tree whose records are read as n_lobes spherical gaussians."""
-    tree = synth.shell_tree(depth=depth, n_spheres=5, data_format=f"SG{n_lobes}", seed=seed, sigma_range=(5.0, 80.0))
+def lobe_tree(n_lobes, seed, depth=6, kind="SG"):
+    """A sparse shell tree whose records are read as n_lobes spherical gaussians ([lambda, mu] each) or
+    anisotropic ones ([lambda_x, lambda_y, an orthonormal frame])."""
+    tree = synth.shell_tree(depth=depth, n_spheres=5, data_format=f"{kind}{n_lobes}", seed=seed, sigma_range=(5.0, 80.0))
     g = torch.Generator().manual_seed(seed + 17)
-    lobes = torch.cat([torch.rand(n_lobes, 1, generator=g) * 4, synth.unit_vectors(n_lobes, g)], dim=1)
+    if kind == "SG":
+        lobes = torch.cat([torch.rand(n_lobes, 1, generator=g) * 4, synth.unit_vectors(n_lobes, g)], dim=1)
+    else:
+        frames = torch.linalg.qr(torch.randn(n_lobes, 3, 3, generator=g))[0].reshape(n_lobes, 9)
+        lobes = torch.cat([torch.rand(n_lobes, 2, generator=g) * 3, frames], dim=1)
     del tree.extra_data
     tree.register_buffer("extra_data", lobes)
     return tree
 
 
-@pytest.mark.parametrize("n_lobes", [1, 4, 9, 16, 25])
-def test_spherical_gaussians_on_the_octree_kernels(gpu, oracle_mod, n_lobes):
-    tree = lobe_tree(n_lobes, seed=3 + n_lobes)
+@pytest.mark.parametrize("kind, n_lobes", [("SG", 1), ("SG", 4), ("SG", 9), ("SG", 16), ("SG", 25),
+                                           ("ASG", 4), ("ASG", 9), ("ASG", 25)])
+def test_lobes_on_the_octree_kernels(gpu, oracle_mod, kind, n_lobes):
+    tree = lobe_tree(n_lobes, seed=3 + n_lobes, kind=kind)
     n = 3000
     rays = synth.sphere_rays(n, seed=4)
     W, H, fx = 70, 50, 60.0
@@ -55,7 +62,7 @@ def test_spherical_gaussians_on_the_octree_kernels(gpu, oracle_mod, n_lobes):
             for spec in (plain, marked):
                 C.set_debug_flags(flags)
                 try:
-                    tag = (n_lobes, fast, flags, spec is marked)
+                    tag = (kind, n_lobes, fast, flags, spec is marked)
                     assert np.array_equal(C.volume_render(spec, rs, opt).cpu().numpy(), want), tag
                     assert np.array_equal(C.volume_render_images(spec, cam, opt).cpu().numpy(), want_img), tag
                     out, notes = C.volume_render_noted(spec, rs, opt)
@@ -79,8 +86,8 @@ def test_spherical_gaussians_on_the_octree_kernels(gpu, oracle_mod, n_lobes):
 
 
 def test_which_kernels_serve_which_trees(gpu):
-    """The octree kernels take fp32 octrees with RGBA, SH or SG records of 1, 4, 9, 16 or 25 basis functions
-    and the full component range; everything else goes to the one-ray-per-lane kernels."""
+    """The octree kernels take fp32 octrees with RGBA, SH, SG or ASG records of 1, 4, 9, 16 or 25 basis
+    functions and the full component range; everything else goes to the one-ray-per-lane kernels."""
     def serve(tree, **kw):
         dev = on_gpu(tree, gpu)
         return C.octree_kernels_serve(dev._spec(), options(tree, **kw))
@@ -91,10 +98,8 @@ def test_which_kernels_serve_which_trees(gpu):
     assert not serve(synth.dense_tree(2, "SH4", seed=1, dtype=torch.float64))
     assert serve(lobe_tree(9, seed=2, depth=4))
     assert not serve(lobe_tree(5, seed=2, depth=4))                       # no kernel built for five lobes
-    g = torch.Generator().manual_seed(1)
-    frames = torch.linalg.qr(torch.randn(4, 3, 3, generator=g))[0].reshape(4, 9)
-    asg = svox.N3Tree(data_format="ASG4", init_refine=1, extra_data=torch.cat([torch.rand(4, 2, generator=g) * 3, frames], 1))
-    assert not serve(asg)
+    assert serve(lobe_tree(4, seed=2, depth=4, kind="ASG"))
+    assert not serve(lobe_tree(6, seed=2, depth=4, kind="ASG"))
     assert not serve(svox.N3Tree(N=3, data_format="SH4", init_refine=1))
 
 
