@@ -46,8 +46,8 @@ def backward_bytes(stats, n_rays, K, ray_io_bytes, data_bytes):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--depth", type=int, default=9, help="finest grid is 2^depth per axis")
     ap.add_argument("--size", type=int, default=800, help="image width and height")
     ap.add_argument("--poses", type=int, default=8)
