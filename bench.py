@@ -190,22 +190,27 @@ def main():
     # what the memory system serves when nothing else is in the way: the library's gather probe (every lane
     # reads 16 bytes of random 64-byte pieces, four reads in flight) on the tree's records, 1.13 GiB (every
     # read misses L2), and on 2 MiB of them (every read hits L2 once warm)
-    def probe_rate(buffer):
-        C.gather_probe(buffer, unit_bytes=64, iters=16)
+    def probe_rate(buffer, unit_bytes=64, lanes=1):
+        C.gather_probe(buffer, unit_bytes=unit_bytes, iters=16, lanes_per_unit=lanes)
         torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
-        reads = C.gather_probe(buffer, unit_bytes=64, iters=64)
+        units = C.gather_probe(buffer, unit_bytes=unit_bytes, iters=64 * lanes, lanes_per_unit=lanes)
         b.record()
         torch.cuda.synchronize()
-        return reads / (a.elapsed_time(b) * 1e3)
+        return units / (a.elapsed_time(b) * 1e3)
 
     flat_data = tree.data.detach().view(-1)
     probe_miss_per_us = probe_rate(flat_data)
     probe_hit_per_us = probe_rate(flat_data[: (2 << 20) // 4])
+    # whole 128-byte lines (8 lanes x 16 bytes): the same lines per microsecond as one 16-byte read per line --
+    # the memory system moves lines, so this rate x 128 bytes is the bandwidth scattered reads can have
+    probe_lines_per_us = probe_rate(flat_data, unit_bytes=128, lanes=8)
 
     # HBM bytes and L2 requests per launch of the dominant kernel come from rocprofv3 counters (separate
     # --pmc runs), not from this process: the committed summary carries the figures for the default workload
+    # (traffic = 2.00 x FETCH_SIZE + WRITE_SIZE: the factor a plain copy gives, and the one the whole-line probe
+    # above gives for scattered reads -- the counter books 64 bytes for a request that moves a 128-byte line)
     traffic = l2_requests = l2_misses = None
     prof = os.path.join(ROOT, "profiles", "hbm_traffic_sparse512_sh16.txt")
     if args.depth == 9 and args.size == 800 and args.poses == 8 and os.path.exists(prof):
@@ -223,6 +228,9 @@ def main():
         "launch": f"{args.poses} poses x {W}x{H} in one launch",
         "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
         "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": traffic,
+        # the same launch on the bytes it makes the memory move (`traffic`: whole 128-byte lines per L2 miss)
+        "fetched_gbs": round(traffic / (float(durs.mean()) * 1e6), 1) if traffic else None,
+        "frac_on_fetched_bytes": round(traffic / (float(durs.mean()) * 1e6) / PEAK_HBM_GBS, 4) if traffic else None,
         "algorithmic_bytes_per_launch": int(launch_bytes.mean()),
         "avg_launch_ms": round(float(durs.mean()), 4),
         "empty_leaves_marked_per_call": bool(C.AUTO_MARK_RAYS_PER_CELL is not None
@@ -243,6 +251,8 @@ def main():
             "torch_index_select_lines_per_us": round(gather_lines_per_us, 1),
             # the gather probe: 64-byte requests per microsecond that miss / hit L2, and the time the launch's
             # requests alone would take at those rates (misses at the one, the other requests at the other)
+            "probe_whole_lines_per_us": round(probe_lines_per_us, 1),
+            "probe_line_bandwidth_gbs": round(probe_lines_per_us * 128 / 1e3, 1),
             "probe_l2_miss_requests_per_us": round(probe_miss_per_us, 1),
             "probe_l2_hit_requests_per_us": round(probe_hit_per_us, 1),
             "launch_ms_at_probe_rates": round((l2_misses / probe_miss_per_us

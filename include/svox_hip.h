@@ -349,16 +349,18 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
  * negative SvoxStatus for a tree or options no kernel accepts.  Results do not depend on the family. */
 int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt);
 
-/* No counterpart in the reference; a measurement aid.  The march kernels read scattered 64-byte
- * pieces of the tree, and how many such requests per microsecond the memory system serves is the
- * ceiling their launches run against.  This launch measures it: `blocks` blocks of 256 lanes, every
- * lane reading 16 bytes at the start of 4 * iters pseudo-random `unit_bytes`-sized units (64, 128
- * or 256) of buffer[0, bytes), four reads in flight per lane; nothing is written unless a checksum
- * that cannot occur does (`sink`: 16 bytes per lane of the launch, may be left uninitialised).
- * The caller times the call: blocks * 256 * 4 * iters reads.  A buffer that fits one L2 (4 MiB)
- * gives the rate of L2 hits, a large one the rate of L2 misses. */
-int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t iters, int32_t blocks,
-                      void* sink, void* stream);
+/* No counterpart in the reference; a measurement aid.  The march kernels read scattered pieces of the
+ * tree, and how many scattered cache lines per microsecond the memory system serves is the ceiling
+ * their launches run against.  This launch measures it: `blocks` blocks of 256 lanes; every group of
+ * `lanes_per_unit` consecutive lanes (1, 4, 8 or 16) reads, 16 bytes per lane, the first
+ * lanes_per_unit * 16 bytes of 4 * iters pseudo-random `unit_bytes`-sized units (64, 128 or 256; at
+ * least lanes_per_unit * 16) of buffer[0, bytes), four reads in flight per lane; nothing is written
+ * unless a checksum that cannot occur does (`sink`: 16 bytes per lane of the launch, may be left
+ * uninitialised).  The caller times the call: blocks * 256 * 4 * iters / lanes_per_unit units.  A buffer
+ * that fits one L2 (4 MiB) gives the rate of L2 hits, a large one the rate of L2 misses; units of 128
+ * bytes read whole (8 lanes) give the bytes a counter should report for a known number of lines. */
+int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t lanes_per_unit, int32_t iters,
+                      int32_t blocks, void* sink, void* stream);
 
 /* No counterpart in the reference; the measurement aid for the backward kernels, whose gradient records
  * reach memory as fp32 atomic adds.  `blocks` blocks of 256 lanes; in each of `iters` rounds the 64 lanes

@@ -728,17 +728,18 @@ def octree_kernels_serve(tree, opt):
     return bool(rc)
 
 
-def gather_probe(buffer, unit_bytes=64, iters=64, blocks=2048):
-    """Queues the library's gather probe on `buffer` (a contiguous CUDA tensor): blocks * 256 lanes, each
-    reading 16 bytes of 4 * iters pseudo-random `unit_bytes`-sized units.  Returns the number of reads;
-    the caller times the call (a measurement aid for the scattered-read ceiling of the march kernels)."""
+def gather_probe(buffer, unit_bytes=64, iters=64, blocks=2048, lanes_per_unit=1):
+    """Queues the library's gather probe on `buffer` (a contiguous CUDA tensor): blocks * 256 lanes, every
+    `lanes_per_unit` consecutive lanes reading the first lanes_per_unit * 16 bytes of 4 * iters pseudo-random
+    `unit_bytes`-sized units.  Returns the number of units read; the caller times the call (a measurement
+    aid for the scattered-read ceiling of the march kernels)."""
     if not buffer.is_contiguous():
         raise ValueError("gather_probe: buffer must be contiguous")
     sink = torch.empty((int(blocks) * 256, 4), dtype=torch.int32, device=buffer.device)
     with torch.cuda.device(buffer.device):
         _call("svox_gather_probe", buffer.data_ptr(), buffer.numel() * buffer.element_size(), int(unit_bytes),
-              int(iters), int(blocks), sink.data_ptr(), _stream(buffer.device))
-    return int(blocks) * 256 * 4 * int(iters)
+              int(lanes_per_unit), int(iters), int(blocks), sink.data_ptr(), _stream(buffer.device))
+    return int(blocks) * 256 * 4 * int(iters) // int(lanes_per_unit)
 
 
 def atomic_probe(scratch, run_floats=16, iters=64, blocks=4096):

@@ -130,7 +130,7 @@ SIGNATURES = {
     "svox_volume_render_backward_workspace_bytes": (c_int64, [c_int64, c_int32]),
     "svox_notes_pool_info": (ctypes.c_int, [c_int64, c_int64, P(c_int64), P(c_int64)]),
     "svox_octree_kernels_serve": (ctypes.c_int, [P(TreeSpecC), P(RenderOptionsC)]),
-    "svox_gather_probe": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "svox_gather_probe": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "svox_atomic_probe": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "svox_volume_render_noted": (
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int64, c_void_p]),

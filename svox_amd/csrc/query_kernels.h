@@ -174,9 +174,10 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(TreeDev<T> tr, con
     }
 }
 
-// Measurement aid (svox_gather_probe): every lane reads 16 bytes at the start of 4 * iters
-// pseudo-random units of the buffer, four reads in flight.  The checksum keeps the reads alive; the
-// store never happens for data a caller can have (it would need one exact 32-bit value).
+// Measurement aid (svox_gather_probe): every group of `lanes` consecutive lanes reads the first
+// lanes * 16 bytes of 4 * iters pseudo-random units of the buffer, 16 bytes per lane, four reads in
+// flight.  The checksum keeps the reads alive; the store never happens for data a caller can have (it
+// would need two exact 32-bit values).
 __device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
     x ^= x >> 16;
     x *= 0x7feb352dU;
@@ -186,16 +187,19 @@ __device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
     return x;
 }
 __global__ __launch_bounds__(256) void gather_probe_kernel(const uint4* __restrict__ buffer, uint64_t n_units,
-                                                           int unit16, int iters, uint4* __restrict__ sink) {
+                                                           int unit16, int lanes, int iters,
+                                                           uint4* __restrict__ sink) {
     uint4 acc = make_uint4(0u, 0u, 0u, 0u);
-    uint32_t seed = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t piece = tid % (uint32_t)lanes;
+    uint32_t seed = tid / (uint32_t)lanes;
     for (int it = 0; it < iters; ++it) {
         uint4 v[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             seed = probe_hash(seed + 0x9e3779b9u * (uint32_t)(k + 1));
             const uint64_t unit = ((uint64_t)seed * n_units) >> 32;
-            v[k] = buffer[unit * (uint64_t)unit16];
+            v[k] = buffer[unit * (uint64_t)unit16 + piece];
         }
 #pragma unroll
         for (int k = 0; k < 4; ++k) {

@@ -1264,16 +1264,20 @@ int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions*
     return fast_basis(tree, opt, true) >= 0 ? 1 : 0;
 }
 
-int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t iters, int32_t blocks,
-                      void* sink, void* stream) {
+int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t lanes_per_unit, int32_t iters,
+                      int32_t blocks, void* sink, void* stream) {
     if (!buffer || !sink) return fail(SVOX_ERR_NULL_POINTER, "svox_gather_probe: NULL buffer or sink");
     if (unit_bytes != 64 && unit_bytes != 128 && unit_bytes != 256)
         return fail(SVOX_ERR_BAD_SHAPE, "svox_gather_probe: unit_bytes must be 64, 128 or 256");
+    if ((lanes_per_unit != 1 && lanes_per_unit != 4 && lanes_per_unit != 8 && lanes_per_unit != 16) ||
+        lanes_per_unit * 16 > unit_bytes)
+        return fail(SVOX_ERR_BAD_SHAPE, "svox_gather_probe: lanes_per_unit must be 1, 4, 8 or 16 and fit the unit");
     if (((uintptr_t)buffer & 15u) || bytes < unit_bytes || bytes / unit_bytes > 0xffffffffll || iters < 1 ||
         blocks < 1 || blocks > (1 << 20))
         return fail(SVOX_ERR_BAD_SHAPE, "svox_gather_probe: buffer, iters or blocks out of range");
     hipLaunchKernelGGL(gather_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       (const uint4*)buffer, (uint64_t)(bytes / unit_bytes), unit_bytes / 16, iters, (uint4*)sink);
+                       (const uint4*)buffer, (uint64_t)(bytes / unit_bytes), unit_bytes / 16, lanes_per_unit, iters,
+                       (uint4*)sink);
     return check_launch("gather_probe");
 }
 

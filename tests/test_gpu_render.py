@@ -890,6 +890,9 @@ def test_gather_probe_runs_and_checks_its_arguments(gpu):
     before = buf.clone()
     assert C.gather_probe(buf, unit_bytes=64, iters=3, blocks=8) == 8 * 256 * 4 * 3
     assert C.gather_probe(buf, unit_bytes=256, iters=1, blocks=1) == 1024
+    assert C.gather_probe(buf, unit_bytes=128, iters=2, blocks=2, lanes_per_unit=8) == 2 * 256 * 4 * 2 // 8
+    with pytest.raises(RuntimeError):
+        C.gather_probe(buf, unit_bytes=64, lanes_per_unit=8)        # 8 lanes x 16 bytes do not fit 64
     torch.cuda.synchronize()
     assert torch.equal(buf, before)
     with pytest.raises(RuntimeError):
