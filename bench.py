@@ -246,6 +246,7 @@ def main():
         # committed profile) per microsecond against a plain gather of random 128-byte lines measured here
         "scattered_lines": {
             "l2_requests_per_launch": l2_requests, "l2_misses_per_launch": l2_misses,
+            "l2_hit_rate": round(1 - l2_misses / l2_requests, 4) if l2_requests and l2_misses else None,
             "l2_requests_per_us": round(l2_requests / (durs.mean() * 1e3), 1) if l2_requests else None,
             "l2_misses_per_us": round(l2_misses / (durs.mean() * 1e3), 1) if l2_misses else None,
             "torch_index_select_lines_per_us": round(gather_lines_per_us, 1),
