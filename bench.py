@@ -43,6 +43,19 @@ def backward_bytes(stats, n_rays, K, ray_io_bytes, data_bytes):
     return n_rays * ray_io_bytes + 2 * per_march + stats["samples_bwd_pos"] * 8 * K + data_bytes
 
 
+def kernel_source_stamp():
+    """sha256 over the sources the HIP library is built from: what a rocprofv3 summary under profiles/ is stamped with,
+    so that counters taken on other kernels are not mixed with this run's timings."""
+    import hashlib
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "svox_amd", "csrc")
+    for name in sorted(os.listdir(src)):
+        if name.endswith((".h", ".hip")):
+            h.update(name.encode())
+            h.update(open(os.path.join(src, name), "rb").read())
+    return h.hexdigest()[:16]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -57,7 +70,11 @@ def main():
     ap.add_argument("--no-query", action="store_true", help="skip the point-query leg")
     ap.add_argument("--no-large", action="store_true", help="skip the depth-10 SH25 NDC leg")
     ap.add_argument("--no-generic", action="store_true", help="skip the fp64 / SG / softplus leg (generic kernels)")
+    ap.add_argument("--print-stamp", action="store_true", help="print the stamp of the kernel sources and exit")
     args = ap.parse_args()
+    if args.print_stamp:
+        print(kernel_source_stamp())
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (rays would shard "
               "trivially across GPUs), run with --gpus 1", file=sys.stderr)
@@ -66,6 +83,7 @@ def main():
     import numpy as np
     import torch
 
+    import bench_probes
     import svox_amd as svox
     from svox_amd import csrc as C
     from svox_amd import synth
@@ -118,25 +136,41 @@ def main():
                 img = renderer.render_persp(p, width=W, height=H, fx=fx, fast=True)
         return img
 
-    def timed(fn):
+    step_spread = {}
+
+    def timed(fn, label=None):
+        """Mean wall-clock milliseconds per step over args.steps steps (synchronised on both sides); with a label,
+        the median and the minimum of the steps' own durations (an event between every two steps) are kept too."""
         for _ in range(args.warmup):
             fn()
+        marks_ = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        marks_[0].record()
+        for i in range(args.steps):
             fn()
+            marks_[i + 1].record()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / args.steps
+        mean_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        if label:
+            per = np.array([marks_[i].elapsed_time(marks_[i + 1]) for i in range(args.steps)])
+            step_spread[label] = {"median_ms": round(float(np.median(per)), 4), "min_ms": round(float(per.min()), 4),
+                                  "max_ms": round(float(per.max()), 4)}
+        return mean_ms
 
-    fwd_ms = timed(forward_step)
+    fwd_ms = timed(forward_step, "forward")
     fwd_mrays = n_rays_step / (fwd_ms * 1e-3) / 1e6
-    per_call_ms = timed(forward_step_per_call)
+    per_call_ms = timed(forward_step_per_call, "forward_per_call")
 
     # Launch duration of the dominant kernel with events on the launching stream.  A launch of this
     # size marks the empty leaves first (C._marks_for_this_call: a small kernel of its own, inside
     # `value`'s timed region); the render launch is timed here alone, with such marks already made.
     marked_spec = tree._spec()
-    marks = C._marks_for_this_call(marked_spec, opt, n_rays_step)
+    made = C._marks_for_this_call(marked_spec, opt, n_rays_step)
+    marks = None
+    if made is not None:
+        marks, marked_spec.child_marks_thresh = made
+        marked_spec.child_marks_softplus = bool(opt.density_softplus)
     marked_spec.child_marks = marks
     cam_all = _make_camera_spec(pose_stack, W, H, fx, fx)
     events = []
@@ -155,7 +189,22 @@ def main():
     else:
         launch_bytes = np.array([float(sum(fwd_bytes))])
     achieved = launch_bytes.mean() / (durs.mean() * 1e-3) / 1e9
+    marks_made_in_call = marks is not None
     del marked_spec, marks
+
+    # the launches of the reference's calling pattern (one pose per call, no marks), timed the same way
+    single = []
+    plain_spec = tree._spec()
+    for p in poses:
+        cam_p = _make_camera_spec(p.contiguous(), W, H, fx, fx)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        C.volume_render_image(plain_spec, cam_p, opt)
+        b.record()
+        single.append((a, b))
+    torch.cuda.synchronize()
+    single_ms = np.array([a.elapsed_time(b) for a, b in single])
+    single_bytes = float(sum(fwd_bytes))          # (no marks: the density of every visited leaf is read)
 
     # copy ceiling of this device (read + write of 1 GiB)
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev)
@@ -191,11 +240,11 @@ def main():
     # reads 16 bytes of random 64-byte pieces, four reads in flight) on the tree's records, 1.13 GiB (every
     # read misses L2), and on 2 MiB of them (every read hits L2 once warm)
     def probe_rate(buffer, unit_bytes=64, lanes=1):
-        C.gather_probe(buffer, unit_bytes=unit_bytes, iters=16, lanes_per_unit=lanes)
+        bench_probes.gather_probe(buffer, unit_bytes=unit_bytes, iters=16, lanes_per_unit=lanes)
         torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
-        units = C.gather_probe(buffer, unit_bytes=unit_bytes, iters=64 * lanes, lanes_per_unit=lanes)
+        units = bench_probes.gather_probe(buffer, unit_bytes=unit_bytes, iters=64 * lanes, lanes_per_unit=lanes)
         b.record()
         torch.cuda.synchronize()
         return units / (a.elapsed_time(b) * 1e3)
@@ -212,29 +261,48 @@ def main():
     # (traffic = 2.00 x FETCH_SIZE + WRITE_SIZE: the factor a plain copy gives, and the one the whole-line probe
     # above gives for scattered reads -- the counter books 64 bytes for a request that moves a 128-byte line)
     traffic = l2_requests = l2_misses = None
-    prof = os.path.join(ROOT, "profiles", "hbm_traffic_sparse512_sh16.txt")
+    traffic_source = None
+    prof_rel = os.path.join("profiles", "hbm_traffic_sparse512_sh16.txt")
+    prof = os.path.join(ROOT, prof_rel)
+    stamp = kernel_source_stamp()
     if args.depth == 9 and args.size == 800 and args.poses == 8 and os.path.exists(prof):
         import re
         text = open(prof).read()
-        m = re.search(r"traffic_bytes_per_launch:\s*(\d+)", text)
-        traffic = int(m.group(1)) if m else None
-        m = re.search(r"l2_requests_per_launch:\s*(\d+)", text)
-        l2_requests = int(m.group(1)) if m else None
-        m = re.search(r"l2_misses_per_launch:\s*(\d+)", text)
-        l2_misses = int(m.group(1)) if m else None
+        m = re.search(r"kernel_sources_stamp:\s*([0-9a-f]+)", text)
+        if m and m.group(1) == stamp:
+            traffic_source = f"{prof_rel} (rocprofv3 --pmc runs on these kernel sources, stamp {stamp})"
+            m = re.search(r"traffic_bytes_per_launch:\s*(\d+)", text)
+            traffic = int(m.group(1)) if m else None
+            m = re.search(r"l2_requests_per_launch:\s*(\d+)", text)
+            l2_requests = int(m.group(1)) if m else None
+            m = re.search(r"l2_misses_per_launch:\s*(\d+)", text)
+            l2_misses = int(m.group(1)) if m else None
+        else:
+            traffic_source = (f"none: {prof_rel} was taken on other kernel sources (its stamp "
+                              f"{m.group(1) if m else 'missing'}, these sources {stamp}); counters are not mixed with this run")
 
     roofline = {
         "bound": "hbm", "kernel": "render_forward_split_kernel<OctreePolicy<SH,16>, ImageSource>",
         "launch": f"{args.poses} poses x {W}x{H} in one launch",
         "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-        "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": traffic,
+        "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": traffic, "traffic_source": traffic_source,
         # the same launch on the bytes it makes the memory move (`traffic`: whole 128-byte lines per L2 miss)
         "fetched_gbs": round(traffic / (float(durs.mean()) * 1e6), 1) if traffic else None,
         "frac_on_fetched_bytes": round(traffic / (float(durs.mean()) * 1e6) / PEAK_HBM_GBS, 4) if traffic else None,
         "algorithmic_bytes_per_launch": int(launch_bytes.mean()),
         "avg_launch_ms": round(float(durs.mean()), 4),
-        "empty_leaves_marked_per_call": bool(C.AUTO_MARK_RAYS_PER_CELL is not None
-                                             and n_rays_step >= C.AUTO_MARK_RAYS_PER_CELL * tree.child.numel()),
+        "median_launch_ms": round(float(np.median(durs)), 4), "min_launch_ms": round(float(durs.min()), 4),
+        "empty_leaves_marked_per_call": marks_made_in_call,
+        # the reference's calling pattern beside it: one launch per pose (no marks), its own launch times and the
+        # fraction of the roofline those launches reach on their algorithmic bytes
+        "per_call": {
+            "launch": f"one pose {W}x{H} per launch, {args.poses} launches",
+            "avg_launch_ms": round(float(single_ms.mean()), 4), "median_launch_ms": round(float(np.median(single_ms)), 4),
+            "min_launch_ms": round(float(single_ms.min()), 4),
+            "algorithmic_bytes_per_launch": int(single_bytes / args.poses),
+            "achieved": round(single_bytes / (float(single_ms.sum()) * 1e-3) / 1e9, 2),
+            "frac": round(single_bytes / (float(single_ms.sum()) * 1e-3) / 1e9 / PEAK_HBM_GBS, 5),
+        },
         "copy_ceiling_gbs": round(copy_gbs, 1),
         "rays_hit": int(sum(s["rays_hit"] for s in pose_stats)),
         "samples": int(sum(s["samples"] for s in pose_stats)),
@@ -277,17 +345,17 @@ def main():
     auto_mark = C.AUTO_MARK_RAYS_PER_CELL
     C.AUTO_MARK_RAYS_PER_CELL = None          # no marks at all: the launch reads the density of every leaf it visits
     plain_imgs = forward_step()
-    plain_ms = timed(forward_step)
+    plain_ms = timed(forward_step, "forward_without_marks")
     C.AUTO_MARK_RAYS_PER_CELL = auto_mark
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    tree.mark_empty_leaves()
+    tree.mark_empty_leaves(sigma_thresh=opt.sigma_thresh)
     torch.cuda.synchronize()
     a.record()
-    tree.mark_empty_leaves()
+    tree.mark_empty_leaves(sigma_thresh=opt.sigma_thresh)
     b.record()
     torch.cuda.synchronize()
     mark_ms = a.elapsed_time(b)
-    marked_ms = timed(forward_step)
+    marked_ms = timed(forward_step, "forward_marks_kept")
     marked_equal = bool(torch.equal(forward_step(), plain_imgs))
     del plain_imgs
     tree.clear_leaf_marks()
@@ -334,14 +402,7 @@ def main():
             with torch.no_grad():
                 tree.data.data.add_(tree.data.grad, alpha=-lr)
 
-        for _ in range(args.warmup):
-            train_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            train_step()
-        torch.cuda.synchronize()
-        tb_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        tb_ms = timed(train_step, "fwd_bwd")
         for _ in range(2):
             train_step(record=True)
         torch.cuda.synchronize()
@@ -356,14 +417,7 @@ def main():
             with torch.no_grad():
                 tree.data.data.add_(grad, alpha=-lr)
 
-        for _ in range(args.warmup):
-            separate_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            separate_step()
-        torch.cuda.synchronize()
-        sep_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        sep_ms = timed(separate_step, "fwd_bwd_separate_calls")
         bbytes = backward_bytes(train_stats, B, K, 36 + 12, data_bytes)
         fbytes = forward_bytes(train_stats, B, K, 36 + 12)
         fwd_bwd = {
@@ -387,11 +441,11 @@ def main():
         # of 16 consecutive floats, one 64-byte request each, at random places of a scratch the size of the
         # gradient).  A record of K floats at a K-float stride lies in (4 K + 60) / 64 such pieces on average.
         scratch = torch.zeros_like(tree.data).view(-1)
-        C.atomic_probe(scratch, run_floats=16, iters=8)
+        bench_probes.atomic_probe(scratch, run_floats=16, iters=8)
         torch.cuda.synchronize()
         pa, pb = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         pa.record()
-        _, probe_requests = C.atomic_probe(scratch, run_floats=16, iters=512)
+        _, probe_requests = bench_probes.atomic_probe(scratch, run_floats=16, iters=512)
         pb.record()
         torch.cuda.synchronize()
         atomic_requests_per_us = probe_requests / (pa.elapsed_time(pb) * 1e3)
@@ -448,7 +502,7 @@ def main():
             tree.data.grad = None
             renderer.render_persp(poses[0], width=W, height=H, fx=fx, fast=True).backward(igo)
 
-        def timed(fn, n=5):
+        def timed_median(fn, n=5):
             # median of n steps queued back to back, an event between every two (a process now and then
             # stalls for tens of milliseconds once, early on: a mean over a few steps would carry that)
             fn()
@@ -463,10 +517,10 @@ def main():
 
         itarget = torch.rand(H, W, 3, generator=g).to(dev)
         fwd_bwd["image_pose"] = {
-            "forward_backward_ms": round(timed(image_step), 3),
-            "se_grad_persp_ms": round(timed(lambda: renderer.se_grad_persp(poses[0], itarget, width=W, height=H,
+            "forward_backward_ms": round(timed_median(image_step), 3),
+            "se_grad_persp_ms": round(timed_median(lambda: renderer.se_grad_persp(poses[0], itarget, width=W, height=H,
                                                                            fx=fx)), 3),
-            "backward_marching_ms": round(timed(lambda: C.volume_render_image_backward(spec, icam, opt, igo,
+            "backward_marching_ms": round(timed_median(lambda: C.volume_render_image_backward(spec, icam, opt, igo,
                                                                                         workspace=False)), 3),
             "note": f"render_persp of pose 0 ({W}x{H}) and its gradient through autograd; then the stateless "
                     "backward operator without a workspace (zero-fill of the gradient included in both)"}
@@ -684,7 +738,8 @@ def main():
             l_ms = ev_time(lambda: C.volume_render_images(lspec, lcam, lopt))
             # (a launch of 3 M rays does not pay for marking 48 M cells; with marks kept on the tree:)
             lmarked = ltree._spec()
-            lmarked.child_marks = C.mark_empty_leaves(lspec)
+            lmarked.child_marks = C.mark_empty_leaves(lspec, lopt.sigma_thresh)
+            lmarked.child_marks_thresh = lopt.sigma_thresh
             l_marked_ms = ev_time(lambda: C.volume_render_images(lmarked, lcam, lopt))
             l_mark_ms = ev_time(lambda: C.mark_empty_leaves(lspec), n=2)
             del lmarked
@@ -772,7 +827,8 @@ def main():
     line = {
         "metric": "Mrays/s fwd, 512^3 sparse SH16 tree",
         "value": round(fwd_mrays, 3), "unit": "Mrays/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(fwd_ms, 4), "higher_is_better": True,
+        "warmup": args.warmup, "ms_per_step": round(fwd_ms, 4), "ms_per_step_median": step_spread["forward"]["median_ms"],
+        "ms_per_step_min": step_spread["forward"]["min_ms"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "rays_hit": roofline["rays_hit"], "mrays_hit_s": round(roofline["rays_hit"] / (fwd_ms * 1e-3) / 1e6, 1),
         "msamples_s": round(roofline["samples"] / (fwd_ms * 1e-3) / 1e6, 1),
@@ -781,6 +837,7 @@ def main():
                    "leaves": tree.info["leaves"], "occupancy": round(tree.info["occupancy"], 5),
                    "data_gib": round(data_bytes / 2**30, 3)},
         "roofline": roofline,
+        "step_times": step_spread,
         "fwd_per_call": per_call,
         "fwd_static_tree": static_tree,
         "fwd_bwd": fwd_bwd,

@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define SVOX_ABI_VERSION 2
+#define SVOX_ABI_VERSION 3
 
 typedef enum SvoxStatus {
     SVOX_OK = 0,
@@ -68,7 +68,9 @@ typedef struct SvoxTreeSpec {
     int32_t extra_cols;
     int32_t weight_accum_max;    /* nonzero: max-reduce into weight_accum, zero: sum */
     int32_t dtype;               /* SvoxDType of data/extra_data/offset/scaling/weight_accum */
-    const int32_t* child_marks;  /* optional (NULL: none): what svox_mark_empty_leaves wrote for this tree */
+    const int32_t* child_marks;  /* optional (NULL: none): what svox_mark_empty_leaves / svox_mark_leaves_below wrote for this tree */
+    float child_marks_thresh;    /* the sigma_thresh those marks were made with (0 for svox_mark_empty_leaves) */
+    int32_t child_marks_softplus;/* nonzero: they were made with density_softplus */
 } SvoxTreeSpec;
 
 /* RaysSpec, svox/csrc/include/data_spec.hpp:51-63 */
@@ -115,7 +117,8 @@ typedef struct SvoxMarchStats {
     uint64_t samples_bwd;     /* leaf visits of one backward march (no early stop) */
     uint64_t samples_bwd_pos; /* of those, visits with sigma > 0 */
     uint64_t levels;          /* child-table entries read by a root-to-leaf walk, forward march */
-    uint64_t reserved;
+    uint64_t samples_tail;    /* of `samples`: visits after the last shaded leaf of their ray (all visits of a ray
+                                 that shades nothing); not counted where the march stops early (stop_thresh) */
 } SvoxMarchStats;
 
 int svox_abi_version(void);
@@ -127,8 +130,17 @@ const char* svox_status_string(int status);
  * any size run the way batches of 512 Ki rays and more do (several 64-ray chunks per wavefront, idle
  * lanes refilled), so that small test batches reach those kernels.  Bit 2: forward renders never take
  * the kernel that walks and shades on two wavefronts; bit 3: they always do where it applies (launches
- * of one 64-ray wavefront per tile or chunk, no weight accumulator), whatever their size. */
+ * of one 64-ray wavefront per tile or chunk, no weight accumulator), whatever their size.  Bit 4: the bounded waits
+ * of that kernel give up at the first look that finds nothing (so that a test can see what a give-up leaves
+ * behind; every kernel still ends normally).  The flags belong to the calling thread. */
 void svox_set_debug_flags(int flags);
+
+/* No counterpart in the reference.  The forward kernel that walks and shades on two wavefronts hands leaves over
+ * through bounded waits (4 Mi looks); a wavefront whose wait ever ran out leaves NaN in its pixels, marks its rays'
+ * notes "to be marched" (the backward pass then marches them: the gradient stays right) and counts itself here.
+ * *count_out: such wavefronts since the library was loaded, on the current device; 0 in any healthy run.  The call
+ * waits for all work queued on the device. */
+int svox_give_up_count(int64_t* count_out);
 
 /* query_vertical(TreeSpec&, Tensor indices) -> (values, node_ids); svox/csrc/svox_kernel.cu:120-143.
  * indices (n_points,3) scalar; values_out (n_points, data_dim) scalar; node_ids_out (n_points) int64. */
@@ -321,6 +333,18 @@ int svox_se_grad_image_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, c
 #define SVOX_EMPTY_LEAF (-2)
 int svox_mark_empty_leaves(const SvoxTreeSpec* tree, int32_t* marks_out, void* stream);
 
+/* No counterpart in the reference.  svox_mark_empty_leaves for a forward render with thresholds: a leaf is marked
+ * when its density -- after the shifted softplus of rt_kernel.cu:276-277 if density_softplus is nonzero -- is not
+ * > sigma_thresh (>= 0), i.e. exactly when trace_ray skips it (rt_kernel.cu:278).  The caller passes the marks
+ * with SvoxTreeSpec.child_marks_thresh = sigma_thresh and .child_marks_softplus = density_softplus.  A forward
+ * render whose options carry the same two values then shades every leaf that is not marked and reads its density
+ * together with its colour coefficients instead of in a round trip of its own.  Calls that need leaves the marks
+ * hide (a smaller or negative sigma_thresh, the other softplus setting; the backward passes, se_grad and the noting
+ * forward passes, which work on every leaf with sigma > 0, unless the marks were made with threshold 0) leave the
+ * marks aside and read the child table.  Results are bit-identical with and without marks. */
+int svox_mark_leaves_below(const SvoxTreeSpec* tree, float sigma_thresh, int32_t density_softplus,
+                           int32_t* marks_out, void* stream);
+
 /* grid_weight_render(data, CameraSpec&, RenderOptions&, offset, scaling) -> {grid_weight, grid_hit};
  * svox.cpp:38-40, 120, rt_kernel.cu:1174-1203 (kernel :898-1003).
  * Marches the pixel rays of one camera through a dense density grid data (reso, reso, reso): per
@@ -349,27 +373,12 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
  * negative SvoxStatus for a tree or options no kernel accepts.  Results do not depend on the family. */
 int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt);
 
-/* No counterpart in the reference; a measurement aid.  The march kernels read scattered pieces of the
- * tree, and how many scattered cache lines per microsecond the memory system serves is the ceiling
- * their launches run against.  This launch measures it: `blocks` blocks of 256 lanes; every group of
- * `lanes_per_unit` consecutive lanes (1, 4, 8 or 16) reads, 16 bytes per lane, the first
- * lanes_per_unit * 16 bytes of 4 * iters pseudo-random `unit_bytes`-sized units (64, 128 or 256; at
- * least lanes_per_unit * 16) of buffer[0, bytes), four reads in flight per lane; nothing is written
- * unless a checksum that cannot occur does (`sink`: 16 bytes per lane of the launch, may be left
- * uninitialised).  The caller times the call: blocks * 256 * 4 * iters / lanes_per_unit units.  A buffer
- * that fits one L2 (4 MiB) gives the rate of L2 hits, a large one the rate of L2 misses; units of 128
- * bytes read whole (8 lanes) give the bytes a counter should report for a known number of lines. */
-int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t lanes_per_unit, int32_t iters,
-                      int32_t blocks, void* sink, void* stream);
-
-/* No counterpart in the reference; the measurement aid for the backward kernels, whose gradient records
- * reach memory as fp32 atomic adds.  `blocks` blocks of 256 lanes; in each of `iters` rounds the 64 lanes
- * of a wavefront add 1.0f to 64 / run_floats runs of `run_floats` consecutive floats (1, 4, 16 or 64; a run
- * of 16 floats that starts on a 64-byte boundary is one 64-byte request) at pseudo-random run-aligned
- * places of scratch[0, bytes), which the caller gives up to the probe (float contents are changed).
- * The caller times the call: blocks * 256 * iters adds in blocks * 256 * iters / min(run_floats, 16)
- * requests. */
-int svox_atomic_probe(void* scratch, int64_t bytes, int32_t run_floats, int32_t iters, int32_t blocks, void* stream);
+/* No counterpart in the reference.  1 if the noting calls (svox_volume_render_noted, svox_volume_render_images_noted)
+ * take notes for this tree under these options when given a workspace with a chunk per ray, 0 if they run as the
+ * plain forward calls and leave the workspace untouched (fp64, the one-ray-per-lane kernels, a weight accumulator, a
+ * negative sigma_thresh), or a negative SvoxStatus.  A caller that would only allocate the workspace for the notes
+ * asks first. */
+int svox_notes_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt);
 
 #ifdef __cplusplus
 }

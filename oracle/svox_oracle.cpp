@@ -303,7 +303,7 @@ inline T advance_t(T t, T delta_t, T tmax) {
 }
 
 struct Counters {
-    uint64_t rays = 0, rays_hit = 0, samples = 0, shaded = 0, bwd = 0, bwd_pos = 0, levels = 0;
+    uint64_t rays = 0, rays_hit = 0, samples = 0, shaded = 0, bwd = 0, bwd_pos = 0, levels = 0, tail = 0;
 };
 
 struct LeafVisit {
@@ -354,12 +354,16 @@ void trace_ray(const TreeView<T>& tr, const SvoxRenderOptions& opt, const T* ori
     const T pad = (T)opt.rgb_padding;
     const T d_rgb_pad = (T)(1 + 2 * opt.rgb_padding);
     T pos[3];
+    uint64_t since_shaded = 0;   // (statistics only: visits since the ray's last shaded leaf)
     while (t < rs.tmax) {
         for (int j = 0; j < 3; ++j) pos[j] = fma_(t, rs.dir[j], rs.origin[j]);
         T cube_sz;
         int levels = 0;
         const int64_t leaf = descend(tr, pos, &cube_sz, &levels);
-        if (leaf < 0) return;  // malformed tree
+        if (leaf < 0) {  // malformed tree
+            if (cnt) cnt->tail += since_shaded;
+            return;
+        }
         const T* val = tr.data + leaf * tr.K;
         T s0, s1;
         dda_unit(pos, rs.invdir, &s0, &s1);
@@ -371,9 +375,11 @@ void trace_ray(const TreeView<T>& tr, const SvoxRenderOptions& opt, const T* ori
             cnt->samples++;
             cnt->levels += (uint64_t)levels;
         }
+        since_shaded += 1;
         if (visits) visits->push_back({leaf, (double)t, (double)delta_t, (double)sigma});
         if (sigma > (T)opt.sigma_thresh) {
             if (cnt) cnt->shaded++;
+            since_shaded = 0;
             const T att = exp_sp<T>(-delta_t * rs.delta_scale * sigma);
             const T weight = light * (T(1) - att);
             if (opt.format != SVOX_FORMAT_RGBA) {
@@ -405,6 +411,7 @@ void trace_ray(const TreeView<T>& tr, const SvoxRenderOptions& opt, const T* ori
         }
         t = advance_t(t, delta_t, rs.tmax);
     }
+    if (cnt) cnt->tail += since_shaded;
     for (int j = 0; j < out_dim; ++j) out[j] = fma_(light, (T)opt.background_brightness, out[j]);
 }
 
@@ -734,6 +741,7 @@ void merge(SvoxMarchStats* dst, const Counters& c) {
     dst->samples_bwd += c.bwd;
     dst->samples_bwd_pos += c.bwd_pos;
     dst->levels += c.levels;
+    dst->samples_tail += c.tail;
 }
 
 int check_render_args(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
@@ -777,6 +785,7 @@ int render_impl(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const SvoxCa
             total.samples += local.samples;
             total.shaded += local.shaded;
             total.levels += local.levels;
+            total.tail += local.tail;
         }
     }
     if (stats) merge(stats, total);

@@ -41,6 +41,8 @@ class TreeSpec:
         self._weight_accum = None
         self._weight_accum_max = False
         self.child_marks = None   # optional: what mark_empty_leaves returned for this tree (no reference counterpart)
+        self.child_marks_thresh = 0.0        # ... and the sigma_thresh / density_softplus it was called with
+        self.child_marks_softplus = False
         self.owner = None         # optional: the N3Tree this spec was made from (its write counter)
 
 
@@ -175,8 +177,12 @@ def _pack_tree(tree, dtype=None, need_data=True):
         if marks.dtype != torch.int32 or marks.shape != tree.child.shape:
             raise RuntimeError("child_marks must be an int32 tensor shaped like child")
         spec.child_marks = marks.data_ptr()
+        spec.child_marks_thresh = float(getattr(tree, "child_marks_thresh", 0.0))
+        spec.child_marks_softplus = int(bool(getattr(tree, "child_marks_softplus", False)))
     else:
         spec.child_marks = None
+        spec.child_marks_thresh = 0.0
+        spec.child_marks_softplus = 0
     spec.capacity = int(tree.child.shape[0])
     spec.N = int(tree.child.shape[1])
     spec.data_dim = int(tree.data.shape[4])
@@ -352,24 +358,33 @@ AUTO_MARK_RAYS_PER_CELL = 0.7
 AUTO_MARK_MIN_RAYS = 1 << 18
 
 
-def _marks_for_this_call(tree, opt, n_rays):
-    """Marks of the empty leaves made for one large launch, or None where they would not pay or
-    would not be used (the fp32 octree kernels read them, and only for sigma_thresh >= 0)."""
+def _marks_for_this_call(tree, opt, n_rays, every_positive_leaf=False):
+    """Marks made for one large launch, or None where they would not pay or would not be used (the fp32
+    octree kernels read them, and only for sigma_thresh >= 0).  A forward launch gets marks made with its own
+    sigma_thresh (every leaf they let through is shaded); every_positive_leaf: the launch works on every leaf with
+    density > 0 whatever the threshold (noting forward passes, backward passes), so the marks are made with 0."""
     if AUTO_MARK_RAYS_PER_CELL is None or getattr(tree, "child_marks", None) is not None:
         return None
-    if tree.data.dtype != torch.float32 or tree.child.shape[1] != 2 or opt.density_softplus:
+    if tree.data.dtype != torch.float32 or tree.child.shape[1] != 2:
         return None
     if not opt.sigma_thresh >= 0 or n_rays < max(AUTO_MARK_MIN_RAYS, AUTO_MARK_RAYS_PER_CELL * tree.child.numel()):
         return None
-    return mark_empty_leaves(tree)
+    thresh = 0.0 if every_positive_leaf else float(opt.sigma_thresh)
+    if opt.density_softplus and thresh <= 0.0:
+        return None          # (the softplus of any stored density is > 0: nothing to mark)
+    return mark_empty_leaves(tree, thresh, bool(opt.density_softplus)), thresh
 
 
-def _attach_marks(spec, tree, opt, n_rays):
+def _attach_marks(spec, tree, opt, n_rays, every_positive_leaf=False):
     """Points the packed `spec` to marks made for this call, where they pay; returns the tensor,
     which the caller keeps until its launch is queued."""
-    marks = _marks_for_this_call(tree, opt, n_rays)
-    if marks is not None:
-        spec.child_marks = marks.data_ptr()
+    made = _marks_for_this_call(tree, opt, n_rays, every_positive_leaf)
+    if made is None:
+        return None
+    marks, thresh = made
+    spec.child_marks = marks.data_ptr()
+    spec.child_marks_thresh = thresh
+    spec.child_marks_softplus = int(bool(opt.density_softplus))
     return marks
 
 
@@ -399,7 +414,7 @@ def volume_render_images_backward(tree, cam, opt, grad_output, workspace=True):
     grad = torch.empty_like(tree.data)
     copt = opt._pack()
     ws, ws_bytes = _backward_workspace(tree, n * cspec.height * cspec.width) if workspace else (None, 0)
-    marks = _attach_marks(spec, tree, opt, n * cspec.height * cspec.width)  # noqa: F841
+    marks = _attach_marks(spec, tree, opt, n * cspec.height * cspec.width, True)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_images_backward_ws", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
               ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
@@ -419,8 +434,8 @@ def volume_render_images_noted(tree, cam, opt, records_per_ray=None):
     shape = (cspec.height, cspec.width, od) if single else (n, cspec.height, cspec.width, od)
     out = torch.empty(shape, dtype=tree.data.dtype, device=tree.data.device)
     copt = opt._pack()
-    ws, ws_bytes = _backward_workspace(tree, n * cspec.height * cspec.width, records_per_ray)
-    marks = _attach_marks(spec, tree, opt, n * cspec.height * cspec.width)  # noqa: F841
+    ws, ws_bytes = _notes_workspace(tree, spec, copt, n * cspec.height * cspec.width, records_per_ray)
+    marks = _attach_marks(spec, tree, opt, n * cspec.height * cspec.width, ws is not None)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_images_noted", ctypes.byref(spec), ctypes.byref(cspec), n, stride,
               ctypes.byref(copt), out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
@@ -498,6 +513,15 @@ def _backward_workspace(tree, n_rays, records_per_ray=None):
         return None, 0
 
 
+def _notes_workspace(tree, spec, copt, n_rays, records_per_ray=None):
+    """_backward_workspace for the notes of a forward pass: (None, 0) also where the library would take no notes
+    for this tree under these options (svox_notes_serve: the one-ray-per-lane kernels, a weight accumulator, a
+    negative sigma_thresh) -- the pass then runs as the plain forward pass and its caller keeps nothing."""
+    if _abi.load_library().svox_notes_serve(ctypes.byref(spec), ctypes.byref(copt)) != 1:
+        return None, 0
+    return _backward_workspace(tree, n_rays, records_per_ray)
+
+
 def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
     """zeros_like(tree.data) + scatter; rt_kernel.cu:1059-1083.
 
@@ -512,7 +536,7 @@ def volume_render_backward(tree, rays, opt, grad_output, workspace=True):
     grad = torch.empty_like(tree.data)
     copt = opt._pack()
     ws, ws_bytes = _backward_workspace(tree, rspec.n_rays) if workspace else (None, 0)
-    marks = _attach_marks(spec, tree, opt, rspec.n_rays)  # noqa: F841
+    marks = _attach_marks(spec, tree, opt, rspec.n_rays, True)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_backward_ws", ctypes.byref(spec), ctypes.byref(rspec),
               ctypes.byref(copt), grad_output.data_ptr(), grad.data_ptr(), 0,
@@ -533,6 +557,11 @@ def volume_render_backward_static(tree, rays, opt, grad_output, grad_data_out, a
     _same_dtype(grad_data_out, tree.data.dtype, "grad_data_out")
     if tuple(grad_data_out.shape) != tuple(tree.data.shape):
         raise RuntimeError("grad_data_out must have the shape of tree.data")
+    # (the library's workspace is looked up for the current device, which is set from tree.data below)
+    for name, x in (("grad_output", grad_output), ("grad_data_out", grad_data_out), ("rays.origins", rays.origins),
+                    ("rays.dirs", rays.dirs), ("rays.vdirs", rays.vdirs), ("child", tree.child)):
+        if x.device != tree.data.device:
+            raise RuntimeError(f"{name} must be on the device of tree.data ({tree.data.device}), got {x.device}")
     copt = opt._pack()
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_backward_static", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),
@@ -562,8 +591,8 @@ def volume_render_noted(tree, rays, opt, records_per_ray=None):
     od = _render_out_dim(spec, opt)
     out = torch.empty((rspec.n_rays, od), dtype=rays.origins.dtype, device=rays.origins.device)
     copt = opt._pack()
-    ws, ws_bytes = _backward_workspace(tree, rspec.n_rays, records_per_ray)
-    marks = _attach_marks(spec, tree, opt, rspec.n_rays)  # noqa: F841
+    ws, ws_bytes = _notes_workspace(tree, spec, copt, rspec.n_rays, records_per_ray)
+    marks = _attach_marks(spec, tree, opt, rspec.n_rays, ws is not None)  # noqa: F841
     with torch.cuda.device(tree.data.device):
         _call("svox_volume_render_noted", ctypes.byref(spec), ctypes.byref(rspec), ctypes.byref(copt),
               out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes, _stream(tree.data.device))
@@ -658,16 +687,20 @@ def se_grad_persp(tree, cam, opt, color, workspace=True):
     return result, grad, hessdiag
 
 
-def mark_empty_leaves(tree):
+def mark_empty_leaves(tree, sigma_thresh=0.0, density_softplus=False):
     """An int32 tensor shaped like tree.child: child with SVOX_EMPTY_LEAF (-2) in every leaf cell whose
-    density is not > 0 (no reference counterpart).  Set as TreeSpec.child_marks it lets the render
-    operators pass through empty leaves without reading their density; results are bit-identical.
+    density (after the shifted softplus, with density_softplus) is not > sigma_thresh (no reference counterpart).
+    Set as TreeSpec.child_marks -- with child_marks_thresh / child_marks_softplus saying how it was made -- it lets
+    the render operators pass through such leaves without reading their density; a forward render with the same
+    sigma_thresh then shades every leaf the marks let through and reads its density with its coefficients.  Calls
+    that need leaves the marks hide leave them aside; results are bit-identical.
     It describes the tree as it is now: make it again, or leave it out, after a write to the
     densities or the structure."""
     spec = _pack_tree(tree)
     marks = torch.empty_like(tree.child)
     with torch.cuda.device(tree.data.device):
-        _call("svox_mark_empty_leaves", ctypes.byref(spec), marks.data_ptr(), _stream(tree.data.device))
+        _call("svox_mark_leaves_below", ctypes.byref(spec), float(sigma_thresh), int(bool(density_softplus)),
+              marks.data_ptr(), _stream(tree.data.device))
     return marks
 
 
@@ -713,12 +746,13 @@ def volume_render_stats(tree, rays_or_cam, opt):
                   ctypes.byref(copt), counters.data_ptr(), _stream(tree.data.device))
     vals = counters.cpu().tolist()
     names = [f[0] for f in _abi.MarchStatsC._fields_]
-    return {n: int(v) for n, v in zip(names, vals) if n != "reserved"}
+    return {n: int(v) for n, v in zip(names, vals)}
 
 
 def octree_kernels_serve(tree, opt):
-    """True where the wavefront-per-tile octree kernels serve the render calls of `tree` under `opt`, False
-    where the one-ray-per-lane kernels do (fp64, N != 2, other basis sizes, partial component ranges)."""
+    """True where the wavefront-per-tile octree kernels serve the render calls of `tree` under `opt` (forward,
+    backward, se_grad, with or without density_softplus), False where the one-ray-per-lane kernels do (fp64,
+    N != 2, other basis sizes, partial component ranges)."""
     spec = _pack_tree(tree)
     copt = opt._pack()
     rc = _abi.load_library().svox_octree_kernels_serve(ctypes.byref(spec), ctypes.byref(copt))
@@ -728,35 +762,17 @@ def octree_kernels_serve(tree, opt):
     return bool(rc)
 
 
-def gather_probe(buffer, unit_bytes=64, iters=64, blocks=2048, lanes_per_unit=1):
-    """Queues the library's gather probe on `buffer` (a contiguous CUDA tensor): blocks * 256 lanes, every
-    `lanes_per_unit` consecutive lanes reading the first lanes_per_unit * 16 bytes of 4 * iters pseudo-random
-    `unit_bytes`-sized units.  Returns the number of units read; the caller times the call (a measurement
-    aid for the scattered-read ceiling of the march kernels)."""
-    if not buffer.is_contiguous():
-        raise ValueError("gather_probe: buffer must be contiguous")
-    sink = torch.empty((int(blocks) * 256, 4), dtype=torch.int32, device=buffer.device)
-    with torch.cuda.device(buffer.device):
-        _call("svox_gather_probe", buffer.data_ptr(), buffer.numel() * buffer.element_size(), int(unit_bytes),
-              int(lanes_per_unit), int(iters), int(blocks), sink.data_ptr(), _stream(buffer.device))
-    return int(blocks) * 256 * 4 * int(iters) // int(lanes_per_unit)
-
-
-def atomic_probe(scratch, run_floats=16, iters=64, blocks=4096):
-    """Queues the library's atomic-add probe on `scratch` (a contiguous float32 CUDA tensor whose contents are
-    given up): blocks * 256 lanes, each adding 1.0f `iters` times, the lanes of a wavefront to runs of
-    `run_floats` consecutive floats at pseudo-random places.  Returns (adds, 64-byte requests); the caller
-    times the call (a measurement aid for the ceiling of the backward kernels' atomics)."""
-    if not scratch.is_contiguous() or scratch.dtype != torch.float32:
-        raise ValueError("atomic_probe: scratch must be a contiguous float32 tensor")
-    with torch.cuda.device(scratch.device):
-        _call("svox_atomic_probe", scratch.data_ptr(), scratch.numel() * 4, int(run_floats), int(iters), int(blocks),
-              _stream(scratch.device))
-    adds = int(blocks) * 256 * int(iters)
-    return adds, adds // min(int(run_floats), 16)
+def give_up_count():
+    """How many wavefronts of the two-wavefront forward kernel have given up a bounded wait since the library was
+    loaded (0 unless something is badly wrong; their pixels are NaN and their rays' notes say "march me").
+    Waits for the device."""
+    n = ctypes.c_int64(0)
+    _call("svox_give_up_count", ctypes.byref(n))
+    return int(n.value)
 
 
 def set_debug_flags(flags):
-    """bit 0: route every call to the generic kernels; bit 1: small ray batches run like large ones;
-    bit 2 / bit 3: forward renders never / always take the two-wavefront kernel"""
+    """Of the calling thread.  bit 0: route every call to the generic kernels; bit 1: small ray batches run like
+    large ones; bit 2 / bit 3: forward renders never / always take the two-wavefront kernel; bit 4: the bounded
+    waits of that kernel give up at the first look that finds nothing (tests of what a give-up leaves behind)"""
     _abi.load_library().svox_set_debug_flags(int(flags))

@@ -22,7 +22,7 @@ c_int64 = ctypes.c_int64
 c_float = ctypes.c_float
 
 
-ABI_VERSION = 2   # SVOX_ABI_VERSION of include/svox_hip.h: the struct layouts below
+ABI_VERSION = 3   # SVOX_ABI_VERSION of include/svox_hip.h: the struct layouts below
 
 
 class TreeSpecC(ctypes.Structure):
@@ -42,6 +42,8 @@ class TreeSpecC(ctypes.Structure):
         ("weight_accum_max", c_int32),
         ("dtype", c_int32),
         ("child_marks", c_void_p),
+        ("child_marks_thresh", c_float),
+        ("child_marks_softplus", c_int32),
     ]
 
 
@@ -91,11 +93,11 @@ class MarchStatsC(ctypes.Structure):
         ("samples_bwd", ctypes.c_uint64),
         ("samples_bwd_pos", ctypes.c_uint64),
         ("levels", ctypes.c_uint64),
-        ("reserved", ctypes.c_uint64),
+        ("samples_tail", ctypes.c_uint64),
     ]
 
     def as_dict(self):
-        return {name: int(getattr(self, name)) for name, _ in self._fields_ if name != "reserved"}
+        return {name: int(getattr(self, name)) for name, _ in self._fields_}
 
 
 P = ctypes.POINTER
@@ -130,8 +132,6 @@ SIGNATURES = {
     "svox_volume_render_backward_workspace_bytes": (c_int64, [c_int64, c_int32]),
     "svox_notes_pool_info": (ctypes.c_int, [c_int64, c_int64, P(c_int64), P(c_int64)]),
     "svox_octree_kernels_serve": (ctypes.c_int, [P(TreeSpecC), P(RenderOptionsC)]),
-    "svox_gather_probe": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
-    "svox_atomic_probe": (ctypes.c_int, [c_void_p, c_int64, c_int32, c_int32, c_int32, c_void_p]),
     "svox_volume_render_noted": (
         ctypes.c_int, [P(TreeSpecC), P(RaysSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_int64, c_void_p]),
     "svox_volume_render_backward_noted": (
@@ -161,6 +161,9 @@ SIGNATURES = {
         ctypes.c_int, [P(TreeSpecC), P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p, c_void_p,
                        c_void_p, c_int64, c_void_p]),
     "svox_mark_empty_leaves": (ctypes.c_int, [P(TreeSpecC), c_void_p, c_void_p]),
+    "svox_mark_leaves_below": (ctypes.c_int, [P(TreeSpecC), c_float, c_int32, c_void_p, c_void_p]),
+    "svox_notes_serve": (ctypes.c_int, [P(TreeSpecC), P(RenderOptionsC)]),
+    "svox_give_up_count": (ctypes.c_int, [P(c_int64)]),
     "svox_grid_weight_render": (
         ctypes.c_int, [c_void_p, c_int32, c_int32, P(CameraSpecC), P(RenderOptionsC), c_void_p, c_void_p, c_void_p,
                        c_void_p, c_void_p]),

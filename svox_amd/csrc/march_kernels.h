@@ -555,10 +555,13 @@ struct ShadeShared<D, false> {
 // lane p mod 64.  One item is the reference's dot product for one channel, evaluated in the
 // reference's order (coefficient 0 first) from 16-byte loads of the leaf record and the owner
 // lane's basis, followed by the sigmoid.
-template <class P, bool kRows>
+// kWithSigma: the densities of the entries are not known yet (a launch whose marks say that every leaf on the list
+// is shaded): the lane of an entry's last channel also reads the density, the scalar after its coefficients, and
+// leaves it in sigma_out[slot * 64 + owner].
+template <class P, bool kRows, bool kWithSigma = false>
 __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
                                               ShadeShared<(P::kBasis > 0 ? P::kBasis : 1), kRows>& sh,
-                                              int n_entries, int lane) {
+                                              int n_entries, int lane, float* sigma_out = nullptr) {
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     const int n_items = n_entries * 3;
@@ -568,6 +571,10 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
         const int who = sh.who[e];
         const int owner = who & 63, slot = who >> 6;
         const float* rec = data + (int64_t)leaf * K;
+        float density = 0.0f;
+        if constexpr (kWithSigma) {
+            if (c == 2) density = rec[K - 1];
+        }
         float s;
         if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
             s = sigmoid_(rec[c]);
@@ -591,6 +598,9 @@ __device__ __forceinline__ void shade_entries(const float* __restrict__ data,
             s = sigmoid_(tmp);
         }
         sh.colour[(slot * kMarchThreads + owner) * 3 + c] = s;
+        if constexpr (kWithSigma) {
+            if (c == 2) sigma_out[slot * kMarchThreads + owner] = density;
+        }
     }
 }
 
@@ -639,6 +649,20 @@ __device__ __forceinline__ void fetch_sigma(const float* __restrict__ data, cons
     }
 }
 
+// density_softplus (rt_kernel.cu:276-277): the march works on log(1 + exp(sigma - 1)) of the stored density.
+// q_sigma: in the stored densities of the queued leaves, out the densities the march uses; q_raw keeps the stored
+// ones (the gradient's chain factor sigmoid(raw - 1), rt_kernel.cu:471-474, and the notes need them).  A slot
+// without a leaf, or with a leaf marked empty, stays at 0.
+__device__ __forceinline__ void soften_sigma(bool softplus, const int32_t* q_leaf, float* q_sigma, float* q_raw) {
+#pragma unroll
+    for (int q = 0; q < kQueue; ++q) q_raw[q] = q_sigma[q];
+    if (softplus) {
+#pragma unroll
+        for (int q = 0; q < kQueue; ++q)
+            q_sigma[q] = (uint32_t)q_leaf[q] < (uint32_t)kEmptyLeafBit ? softplus_m1(q_raw[q]) : 0.0f;
+    }
+}
+
 // Shade list: the (lane, slot) pairs with sigma > thresh, compacted by ballot and prefix count
 // (`skip`: none of this lane's).  Returns the number of entries.
 template <class Shared>
@@ -648,6 +672,25 @@ __device__ __forceinline__ int build_shade_list(Shared& sh, const int32_t* q_lea
 #pragma unroll
     for (int q = 0; q < kQueue; ++q) {
         const bool want = !skip && q_leaf[q] >= 0 && q_sigma[q] > thresh;
+        const unsigned long long m = __ballot(want);
+        if (want) {
+            const int e = n_entries + rank_in(m);
+            sh.leaf[e] = q_leaf[q];
+            sh.who[e] = (uint8_t)(lane | (q << 6));
+        }
+        n_entries += __popcll(m);
+    }
+    return n_entries;
+}
+
+// The same list where the marks of the launch say that every leaf they let through is shaded (the marks were made
+// with the launch's own sigma_thresh): every queued leaf that is not marked joins, its density still unread.
+template <class Shared>
+__device__ __forceinline__ int build_shade_list_all(Shared& sh, const int32_t* q_leaf, int lane) {
+    int n_entries = 0;
+#pragma unroll
+    for (int q = 0; q < kQueue; ++q) {
+        const bool want = (uint32_t)q_leaf[q] < (uint32_t)kEmptyLeafBit;
         const unsigned long long m = __ballot(want);
         if (want) {
             const int e = n_entries + rank_in(m);
@@ -680,6 +723,9 @@ struct ReplaySpace {
     // bitmap as `only` does those rays and no others
     unsigned long long* undone;
     const unsigned long long* only;
+    // > 0: the looks in a row after which a waiting wavefront of render_forward_split_kernel gives up, in place of
+    // kSpinLimit (set by a debug flag, so that a test can see what a give-up leaves behind)
+    int32_t spin_limit;
 };
 
 // whether the workspace carries the stamp this launch expects
@@ -719,8 +765,8 @@ enum BackwardMode { kBackwardPlain = 0, kBackwardSecond = 1 };
 // Head of a ray's notes, kept in the spare floats of its first chunk (after the 15 records): the
 // link to the next chunk, the number of notes (-1: they did not fit; 0 also for a ray that misses
 // the tree), the ray's delta_scale (rt_kernel.cu:228), a flag (1.0f: the ray misses the tree, 2.0f:
-// its walk broke off in a malformed tree, else 0.0f) and the sum of the backward pass's first march
-// where the noting pass could form it (NoteTaker::finish).
+// its walk broke off in a malformed tree, 3.0f: the launch gave up on the ray -- count -1, no sum --, else 0.0f)
+// and the sum of the backward pass's first march where the noting pass could form it (NoteTaker::finish).
 constexpr int kChunkRecords = 15;
 constexpr int kChunkFloat2 = (kChunkRecords + 1) * 3;   // 384 bytes
 constexpr int kHeadFloat2 = kChunkRecords * 3;          // float2 index of {link, count}, then {delta_scale, -}
@@ -792,6 +838,13 @@ struct NoteTaker {
     // the notes are incomplete; then the ray's delta_scale and 2.0f if the walk broke off in a
     // malformed tree; then, from a noting pass that had the gradient of the picture at hand, the sum
     // the backward pass forms in its first march (render_backward_kernel<kBackwardSecond> starts from it).
+    // The notes of a ray whose launch gave up on it (the bounded wait of render_forward_split_kernel ran out): no
+    // count and no sum of the first march (flag 3.0f): the backward pass marches this ray twice.
+    __device__ __forceinline__ void give_up(float dscale) {
+        ((float*)(first + kHeadFloat2))[1] = __int_as_float(-1);
+        first[kHeadFloat2 + 1] = make_float2(dscale, 3.0f);
+        first[kHeadFloat2 + 2] = make_float2(0.0f, 0.0f);
+    }
     __device__ __forceinline__ void finish(bool broken, float dscale, float march1_sum = 0.0f) {
         ((float*)(first + kHeadFloat2))[1] = __int_as_float(lost || broken ? -1 : count);
         first[kHeadFloat2 + 1] = make_float2(dscale, broken ? 2.0f : 0.0f);
@@ -855,15 +908,22 @@ struct March1Sum {
 // the colours of the leaves at or below sigma_thresh are evaluated too.  With out == nullptr only the
 // notes are taken (the backward pass without a forward pass before it); kGrad: that backward pass's
 // grad_out is given, and the sum of its first march is formed on the way (March1Sum).
-template <class P, class Source, bool kAccum, bool kRefill, bool kNoted = false, bool kGrad = false>
+// kAllShaded: tr.child is a marked copy of the child table made with this launch's sigma_thresh (and softplus
+// setting): a leaf that is not marked has sigma > sigma_thresh, so the round has no density phase -- every
+// unmarked leaf goes on the shade list and its density arrives with its coefficients (one round trip to memory
+// per round instead of two that wait for one another).
+template <class P, class Source, bool kAccum, bool kRefill, bool kNoted = false, bool kGrad = false,
+          bool kAllShaded = false>
 __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<float> tr, Source src,
                                                                        SvoxRenderOptions opt,
                                                                        float* __restrict__ out, ReplaySpace ws,
                                                                        const float* __restrict__ grad_out = nullptr) {
+    static_assert(!kAllShaded || (!kNoted && !kAccum), "notes and weights look at leaves the marks may hide");
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
     __shared__ ShadeShared<D, P::kForwardRows> sh;
+    __shared__ float sh_sigma[kAllShaded ? kQueue * kMarchThreads : 1];
     const int lane = threadIdx.x;
     float offset[3], scaling[3];
     load_transform(tr, offset, scaling);
@@ -945,19 +1005,29 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
         bool broken;
         walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt);
         // ---- sigma
-        float q_sigma[kQueue];
-        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
-        if (opt.density_softplus) {   // rt_kernel.cu:276-277 (the launcher passes no marks with this option)
-#pragma unroll
-            for (int q = 0; q < kQueue; ++q) q_sigma[q] = q_leaf[q] >= 0 ? softplus_m1(q_sigma[q]) : 0.0f;
+        float q_sigma[kQueue], q_raw[kQueue];   // (q_raw: what the notes keep, the stored density)
+        int n_entries;
+        if constexpr (kAllShaded) {
+            n_entries = build_shade_list_all(sh, q_leaf, lane);
+        } else {
+            fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+            soften_sigma(opt.density_softplus, q_leaf, q_sigma, q_raw);
+            // ---- shade list
+            n_entries = build_shade_list(sh, q_leaf, q_sigma, kNoted ? 0.0f : sigma_thresh, lane);
         }
-        // ---- shade list
-        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, kNoted ? 0.0f : sigma_thresh, lane);
         bool stopped = false;
         if (n_entries > 0) {   // most rounds of a ray pass through empty space: nothing to shade
             wave_lds_sync();   // list and view directions are visible to every lane
-            shade_entries<P, P::kForwardRows>(tr.data, sh, n_entries, lane);
+            shade_entries<P, P::kForwardRows, kAllShaded>(tr.data, sh, n_entries, lane, sh_sigma);
             wave_lds_sync();
+            if constexpr (kAllShaded) {
+#pragma unroll
+                for (int q = 0; q < kQueue; ++q) {
+                    const bool listed = (uint32_t)q_leaf[q] < (uint32_t)kEmptyLeafBit;
+                    const float raw = sh_sigma[q * kMarchThreads + lane];
+                    q_sigma[q] = listed ? (opt.density_softplus ? softplus_m1(raw) : raw) : 0.0f;
+                }
+            }
             // ---- composite
             // the attenuations and padded colours of the four slots do not depend on one another: they
             // are evaluated side by side, and only the products with the transmittance form a chain
@@ -990,7 +1060,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                 stopped = stopped || (take && light <= stop_thresh);
                 if constexpr (kNoted) {
                     const bool note = active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
-                    notes.take(ws, shared_next, shared_end, lane, note, q_leaf[q], q_dt[q], q_sigma[q], q_s[q]);
+                    notes.take(ws, shared_next, shared_end, lane, note, q_leaf[q], q_dt[q], q_raw[q], q_s[q]);
                     if constexpr (kGrad) {
                         if (note) sum1.leaf(q_dt[q], q_sigma[q], r.dscale, q_s[q], d_rgb_pad, pad);
                     }
@@ -1307,16 +1377,18 @@ struct RecordList {
     __device__ __forceinline__ void add_held(const uint8_t* order) {
         const bool mine = lane < n;
         const int rec = mine ? (order ? order[lane] : lane) : 0;
-        int my_rec = rec;
-        int my_leaf = leaves()[rec];
-        int my_owner = owners()[rec];
-        // Every lane must hold its record before any lane reads it by readlane.  The compiler does not
-        // know that readlane looks into other lanes: without this it moves the reads above into the loop
-        // below, which the lanes beyond K never enter, and their registers stay unset.
-        asm volatile("" : "+v"(my_rec), "+v"(my_leaf), "+v"(my_owner));
-        for (int e = lane; e < K; e += kMarchThreads) {
-            const int c = P::kFormat == SVOX_FORMAT_RGBA ? e : e / D;
-            const int i = P::kFormat == SVOX_FORMAT_RGBA ? 0 : e - c * D;
+        const int my_rec = rec;
+        const int my_leaf = leaves()[rec];
+        const int my_owner = owners()[rec];
+        // readlane looks into other lanes, so every lane must hold its record and must stay in step with the
+        // others: the loop below is one every lane runs (its trip count depends on K alone), and a lane whose
+        // element lies beyond the record only leaves out the additions.
+        for (int e0 = 0; e0 < K; e0 += kMarchThreads) {
+            const int e = e0 + lane;
+            const bool on = e < K;
+            const int c_raw = P::kFormat == SVOX_FORMAT_RGBA ? e : e / D;
+            const int c = c_raw < 3 ? c_raw : 3;                              // (3: the density element, and lanes that are not `on`)
+            const int i = P::kFormat == SVOX_FORMAT_RGBA || c == 3 ? 0 : e - c * D;
             const bool with_basis = P::kFormat != SVOX_FORMAT_RGBA && c < 3;
             int32_t cur = -1;
             float acc = 0.0f;
@@ -1342,7 +1414,7 @@ struct RecordList {
                 for (int u = 0; u < kHeldBlock; ++u) {
                     if (at + u < n) {
                         if (leaf[u] != cur) {
-                            if (cur >= 0) atomicAdd(grad_data + (int64_t)cur * K + e, acc);
+                            if (on && cur >= 0) atomicAdd(grad_data + (int64_t)cur * K + e, acc);
                             cur = leaf[u];
                             acc = 0.0f;
                         }
@@ -1350,7 +1422,7 @@ struct RecordList {
                     }
                 }
             }
-            if (cur >= 0) atomicAdd(grad_data + (int64_t)cur * K + e, acc);
+            if (on && cur >= 0) atomicAdd(grad_data + (int64_t)cur * K + e, acc);
         }
     }
 
@@ -1488,27 +1560,40 @@ struct SplitBox {
     int32_t taken[kMarchThreads];          // set by the shading: leaves taken out so far (| kEndedBit)
 };
 
-// The two counters are read and written as relaxed atomics of the workgroup: the compiler then neither
-// keeps them in registers nor moves them across one another, and, unlike a volatile access (which it
-// leaves on the generic address path: a flat instruction with a wait for every store), it still knows
-// that they live in LDS and issues plain LDS reads and writes.
+// The two counters are read and written as atomics of the workgroup (unlike a volatile access, which the compiler
+// leaves on the generic address path -- a flat instruction with a wait for every store --, it still knows that they
+// live in LDS and issues plain LDS reads and writes).  A count is published with release order after the ring
+// entries it covers were written (or read), and read with acquire order before they are read (or overwritten):
+// the hand-over does not lean on the order in which one wavefront's LDS operations happen to be carried out.
+#ifdef SVOX_BOX_RELAXED
+constexpr int kBoxLoadOrder = __ATOMIC_RELAXED, kBoxStoreOrder = __ATOMIC_RELAXED;
+#else
+constexpr int kBoxLoadOrder = __ATOMIC_ACQUIRE, kBoxStoreOrder = __ATOMIC_RELEASE;
+#endif
 __device__ __forceinline__ int32_t box_read(const int32_t* at) {
-    return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return __hip_atomic_load(at, kBoxLoadOrder, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 __device__ __forceinline__ void box_write(int32_t* at, int32_t value) {
-    __hip_atomic_store(at, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __hip_atomic_store(at, value, kBoxStoreOrder, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-template <class P, class Source, bool kNoted = false, bool kGrad = false>
+// Wavefronts of render_forward_split_kernel that gave up waiting since the library was loaded (svox_give_up_count).
+__device__ unsigned int split_give_ups = 0;
+
+// kAllShaded: as in render_forward_kernel -- the marks were made with this launch's sigma_thresh, every leaf the
+// walk hands over is shaded, and its density is read with its coefficients.
+template <class P, class Source, bool kNoted = false, bool kGrad = false, bool kAllShaded = false>
 __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(TreeDev<float> tr, Source src,
                                                                              SvoxRenderOptions opt,
                                                                              float* __restrict__ out, ReplaySpace ws,
                                                                              const float* __restrict__ grad_out = nullptr) {
+    static_assert(!kAllShaded || !kNoted, "notes look at leaves the marks may hide");
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
     __shared__ ShadeShared<D, P::kForwardRows> sh;
     __shared__ SplitBox box;
+    __shared__ float sh_sigma[kAllShaded ? kQueue * kMarchThreads : 1];
     if constexpr (kNoted) {
         if (blockIdx.x == 0 && threadIdx.x < kStampWords) ws.stamp_at[threadIdx.x] = ws.stamp[threadIdx.x];
     }
@@ -1520,6 +1605,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
     const float pad = opt.rgb_padding;
     const float d_rgb_pad = 1 + 2 * opt.rgb_padding;
     const float step = opt.step_size, sigma_thresh = opt.sigma_thresh, stop_thresh = opt.stop_thresh;
+    const int spin_limit = ws.spin_limit > 0 ? ws.spin_limit : kSpinLimit;
 
     const int64_t item = chunk_of_block(blockIdx.x, gridDim.x, src.xcd_group) * (int64_t)kMarchThreads + lane;
     RayState<float> r;
@@ -1583,7 +1669,10 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
             if (!__any(live)) break;
             const bool go = live && written - (taken & ~kEndedBit) < kRing;
             if (!__any(go)) {   // every ring is full: the shading is behind
-                if (++spins > kSpinLimit) break;
+                if (++spins > spin_limit) {
+                    if (lane == 0) atomicAdd(&split_give_ups, 1u);
+                    break;
+                }
                 __builtin_amdgcn_s_sleep(1);
                 continue;
             }
@@ -1598,9 +1687,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
                 box.dt[at] = dt;
                 written += 1;
             }
-            // (a wavefront's LDS operations are carried out in order: the leaf is in the ring before the
-            // count says so; only the compiler has to be told)
-            asm volatile("" ::: "memory");
+            // (release: the leaf is in the ring before the count says so)
             if (put) box_write(&box.written[lane], written);
         }
         return;
@@ -1620,8 +1707,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
     if constexpr (kNoted) notes.begin(ws, active ? slot : 0);
     if constexpr (kNoted && kGrad) sum1.begin(grad_out, active ? slot : 0);
     while (true) {
-        const int32_t w = box_read(&box.written[lane]);
-        asm volatile("" ::: "memory");   // the ring is read after the count, not before
+        const int32_t w = box_read(&box.written[lane]);   // (acquire: the ring is read after the count, not before)
         const int32_t avail = (w & ~(kEndedBit | kBrokenBit)) - taken;
         if (active && (w & kEndedBit) && avail == 0) {
             // the ray left the tree: the background shows through what is left of the light
@@ -1638,9 +1724,16 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         // (waiting for fuller hands -- two or four leaves per lane, a few looks of patience -- and a ring
         // of 16 were measured: no gain, the larger ring costs LDS)
         if (!__any(n_take > 0)) {   // the walk has found nothing new yet
-            if (++spins > kSpinLimit) {
-                // cannot happen while the walk runs; a picture with NaN in it says so if it ever does
-                if (active && out) out[slot * 3] = out[slot * 3 + 1] = out[slot * 3 + 2] = __int_as_float(0x7fc00000);
+            if (++spins > spin_limit) {
+                // Cannot happen while the walk runs.  If it ever does, nothing plausible is left behind: the pixel
+                // is NaN, the ray's notes say "march me" (the backward pass then does, twice), and the library's
+                // give-up counter tells the host (svox_give_up_count).
+                if (active && out && !painted)
+                    out[slot * 3] = out[slot * 3 + 1] = out[slot * 3 + 2] = __int_as_float(0x7fc00000);
+                if constexpr (kNoted) {
+                    if (active) notes.give_up(r.dscale);
+                }
+                if (lane == 0) atomicAdd(&split_give_ups, 1u);
                 break;
             }
             __builtin_amdgcn_s_sleep(1);
@@ -1658,18 +1751,27 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         wave_lds_sync();   // the leaves are out of the ring before the count gives their places back
         taken += n_take;
         if (n_take > 0) box_write(&box.taken[lane], taken);
-        float q_sigma[kQueue];
-        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
-        if (opt.density_softplus) {
-#pragma unroll
-            for (int q = 0; q < kQueue; ++q) q_sigma[q] = q_leaf[q] >= 0 ? softplus_m1(q_sigma[q]) : 0.0f;
+        float q_sigma[kQueue], q_raw[kQueue];
+        int n_entries;
+        if constexpr (kAllShaded) {
+            n_entries = build_shade_list_all(sh, q_leaf, lane);
+        } else {
+            fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+            soften_sigma(opt.density_softplus, q_leaf, q_sigma, q_raw);
+            n_entries = build_shade_list(sh, q_leaf, q_sigma, kNoted ? 0.0f : sigma_thresh, lane);
         }
-        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, kNoted ? 0.0f : sigma_thresh, lane);
         bool stopped = false;
         if (n_entries > 0) {
             wave_lds_sync();
-            shade_entries<P, P::kForwardRows>(tr.data, sh, n_entries, lane);
+            shade_entries<P, P::kForwardRows, kAllShaded>(tr.data, sh, n_entries, lane, sh_sigma);
             wave_lds_sync();
+            if constexpr (kAllShaded) {
+#pragma unroll
+                for (int q = 0; q < kQueue; ++q) {
+                    const float raw = sh_sigma[q * kMarchThreads + lane];
+                    q_sigma[q] = q_leaf[q] >= 0 ? (opt.density_softplus ? softplus_m1(raw) : raw) : 0.0f;
+                }
+            }
             float q_att[kQueue], q_rgb[kQueue][3], q_s[kQueue][3];
 #pragma unroll
             for (int q = 0; q < kQueue; ++q) {
@@ -1691,7 +1793,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
                 stopped = stopped || (take && light <= stop_thresh);
                 if constexpr (kNoted) {
                     const bool note = active && q_leaf[q] >= 0 && q_sigma[q] > 0.0f;
-                    notes.take(ws, shared_next, shared_end, lane, note, q_leaf[q], q_dt[q], q_sigma[q], q_s[q]);
+                    notes.take(ws, shared_next, shared_end, lane, note, q_leaf[q], q_dt[q], q_raw[q], q_s[q]);
                     if constexpr (kGrad) {
                         if (note) sum1.leaf(q_dt[q], q_sigma[q], r.dscale, q_s[q], d_rgb_pad, pad);
                     }
@@ -1759,11 +1861,14 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         if (!Source::kItemsAreSlots && ws.only && slot >= 0 && !((ws.only[slot >> 6] >> (slot & 63)) & 1ull)) return;
         if (slot >= 0 && setup_ray(r, origin, dir, scaling)) {
             float march1_sum = 0.0f;
+            bool first_march_too = false;
             if constexpr (kMode == kBackwardSecond) {
                 const float2* head = ws.base + slot * kChunkFloat2 + kHeadFloat2;
                 // (a walk that broke off in a malformed tree: the reference adds nothing for such a ray)
-                if (head[1].y != 0.0f) return;
-                march1_sum = head[2].x;
+                if (head[1].y == 2.0f) return;
+                // (a ray the noting launch gave up on has no sum: both marches)
+                first_march_too = head[1].y == 3.0f;
+                march1_sum = first_march_too ? 0.0f : head[2].x;
             }
             if constexpr (P::kFormat != SVOX_FORMAT_RGBA) {
                 float basis[D];
@@ -1778,7 +1883,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             accum = march1_sum;
             tmin = r.t;
             cur.restart();
-            phase = kMode == kBackwardSecond ? kMarch2 : kMarch1;
+            phase = kMode == kBackwardSecond && !first_march_too ? kMarch2 : kMarch1;
             active = true;
         }
     };
@@ -1803,7 +1908,9 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
         float q_sigma[kQueue];
         walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt);
         // ---- sigma
+        float q_raw[kQueue];
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+        soften_sigma(opt.density_softplus, q_leaf, q_sigma, q_raw);
         // ---- shade list: every leaf with density
         const int n_entries = build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane);
         wave_lds_sync();
@@ -1850,6 +1957,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
                     }
                     accum = fma_(-weight, total_color, accum);
                     g_sigma = q_dt[q] * r.dscale * fma_(total_color, light, -accum);
+                    if (opt.density_softplus) g_sigma *= sigmoid_(q_raw[q] - 1.0f);   // rt_kernel.cu:471-474
                     emit = true;
                 }
             }
@@ -1973,11 +2081,12 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
             for (int k = 0; k < kReplayGroup; ++k) {
                 const bool have = work && base + k < count;
                 const int32_t leaf = __float_as_int(g.note[k][0].x);
-                const float dt = g.note[k][0].y, sigma = g.note[k][1].x;
+                const float dt = g.note[k][0].y, raw = g.note[k][1].x;   // (the stored density)
                 const float s[3] = {g.note[k][1].y, g.note[k][2].x, g.note[k][2].y};
                 float tmp2[3] = {0.f, 0.f, 0.f};
                 float g_sigma = 0.0f;
                 if (have) {
+                    const float sigma = opt.density_softplus ? softplus_m1(raw) : raw;
                     const float att = expf_fixed(-dt * sigma * dscale);
                     const float weight = light * (1.0f - att);
                     float total_color = 0.0f;
@@ -1998,6 +2107,7 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
                         }
                         accum = fma_(-weight, total_color, accum);
                         g_sigma = dt * dscale * fma_(total_color, light, -accum);
+                        if (opt.density_softplus) g_sigma *= sigmoid_(raw - 1.0f);
                     }
                 }
                 if (pass == 1) records.append(have, leaf, tmp2, g_sigma);
@@ -2264,8 +2374,9 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         bool broken;
         walk_turns(tr, r, cur, step, active, broken, q_leaf, q_dt);
         // ---- sigma
-        float q_sigma[kQueue];
+        float q_sigma[kQueue], q_raw[kQueue];
         fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+        soften_sigma(opt.density_softplus, q_leaf, q_sigma, q_raw);
         // ---- shade list
         const int n_entries = build_shade_list(sh, q_leaf, q_sigma, 0.0f, lane);
         wave_lds_sync();
@@ -2295,6 +2406,9 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
                         caccum[c] = fma_(weight, col[c], caccum[c]);
                     }
                 } else {
+                    // (density_softplus: the chain factor of rt_kernel.cu:693-703; 1 and 0 without it)
+                    const float sg = opt.density_softplus ? sigmoid_(q_raw[q] - 1.0f) : 1.0f;
+                    const float d_sg = sg * (1.0f - sg);
 #pragma unroll
                     for (int c = 0; c < 3; ++c) {
                         if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
@@ -2304,8 +2418,13 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
                         }
                         caccum[c] = fma_(-weight, col[c], caccum[c]);
                         const float gs = q_dt[q] * r.dscale * fma_(col[c], light, -caccum[c]);
-                        g_sigma += gs * resid[c];
-                        h_sigma += gs * gs;
+                        if (opt.density_softplus) {
+                            g_sigma += gs * resid[c] * sg;
+                            h_sigma += fma_(gs * gs * sg, sg, gs * d_sg);
+                        } else {
+                            g_sigma += gs * resid[c];
+                            h_sigma += gs * gs;
+                        }
                     }
                     emit = true;
                 }
@@ -2470,14 +2589,17 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
             // record have their addresses from scalars and those of four records are in flight together
             // (RecordList::add_held).
             const bool mine = lane < n;
-            int my_rec = mine ? (grouped ? group.order[lane] : lane) : 0;
-            int my_leaf = l_leaf[my_rec];
-            int my_owner = l_owner[my_rec];
-            asm volatile("" : "+v"(my_rec), "+v"(my_leaf), "+v"(my_owner));   // (set in every lane before any readlane)
+            const int my_rec = mine ? (grouped ? group.order[lane] : lane) : 0;
+            const int my_leaf = l_leaf[my_rec];
+            const int my_owner = l_owner[my_rec];
             constexpr int kBlock = 4;
-            for (int e = lane; e < K; e += kMarchThreads) {
-                const int c = kRgba ? e : e / D;
-                const int i = kRgba ? 0 : e - c * D;
+            // (a loop every lane runs, so that every lane holds its record when readlane looks: see add_held)
+            for (int e0 = 0; e0 < K; e0 += kMarchThreads) {
+                const int e = e0 + lane;
+                const bool on = e < K;
+                const int c_raw = kRgba ? e : e / D;
+                const int c = c_raw < 3 ? c_raw : 3;
+                const int i = kRgba || c == 3 ? 0 : e - c * D;
                 const int cc = c < 3 ? c : 0;
                 int32_t cur = -1;
                 float acc[2] = {0.0f, 0.0f};
@@ -2499,7 +2621,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
                     for (int u = 0; u < kBlock; ++u) {
                         if (at + u < n) {
                             if (leaf[u] != cur) {
-                                if (cur >= 0) emit(cur, e, acc);
+                                if (on && cur >= 0) emit(cur, e, acc);
                                 cur = leaf[u];
                                 acc[0] = acc[1] = 0.0f;
                             }
@@ -2509,7 +2631,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
                         }
                     }
                 }
-                if (cur >= 0) emit(cur, e, acc);
+                if (on && cur >= 0) emit(cur, e, acc);
             }
         } else {
             add_records_by_leaf<K, 2>(
@@ -2588,11 +2710,12 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
             for (int k = 0; k < kReplayGroup; ++k) {
                 const bool have = work && base + k < count;
                 const int32_t leaf = __float_as_int(g.note[k][0].x);
-                const float dt = g.note[k][0].y, sigma = g.note[k][1].x;
+                const float dt = g.note[k][0].y, raw = g.note[k][1].x;   // (the stored density)
                 const float s[3] = {g.note[k][1].y, g.note[k][2].x, g.note[k][2].y};
                 float gci[3] = {0.f, 0.f, 0.f};
                 float g_sigma = 0.0f, h_sigma = 0.0f;
                 if (have) {
+                    const float sigma = opt.density_softplus ? softplus_m1(raw) : raw;
                     const float att = expf_fixed(-dt * sigma * dscale);
                     const float weight = light * (1.0f - att);
                     float col[3];
@@ -2609,6 +2732,8 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
                             caccum[c] = fma_(weight, col[c], caccum[c]);
                         }
                     } else {
+                        const float sg = opt.density_softplus ? sigmoid_(raw - 1.0f) : 1.0f;
+                        const float d_sg = sg * (1.0f - sg);
 #pragma unroll
                         for (int c = 0; c < 3; ++c) {
                             if constexpr (kRgba) {
@@ -2618,8 +2743,13 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
                             }
                             caccum[c] = fma_(-weight, col[c], caccum[c]);
                             const float gs = dt * dscale * fma_(col[c], light, -caccum[c]);
-                            g_sigma += gs * resid[c];
-                            h_sigma += gs * gs;
+                            if (opt.density_softplus) {
+                                g_sigma += gs * resid[c] * sg;
+                                h_sigma += fma_(gs * gs * sg, sg, gs * d_sg);
+                            } else {
+                                g_sigma += gs * resid[c];
+                                h_sigma += gs * gs;
+                            }
                         }
                     }
                 }
@@ -2728,6 +2858,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_stats_kernel(TreeDev<T> 
     const int64_t slot = src.fetch_item(blockIdx.x * (int64_t)kMarchThreads + threadIdx.x, opt, offset, scaling,
                                         origin, dir, vdir);
     unsigned long long c_rays = 0, c_hit = 0, c_samples = 0, c_shaded = 0, c_bwd = 0, c_bwd_pos = 0, c_levels = 0;
+    unsigned long long c_tail = 0;
     if (slot >= 0) {
         c_rays = 1;
         RayState<T> r;
@@ -2735,6 +2866,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_stats_kernel(TreeDev<T> 
             c_hit = 1;
             T light = T(1);
             bool fwd_live = true;
+            unsigned since_shaded = 0;   // forward visits since the ray's last shaded leaf
             while (r.t < r.tmax) {
                 T delta_t;
                 const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
@@ -2746,14 +2878,17 @@ __global__ __launch_bounds__(kMarchThreads) void render_stats_kernel(TreeDev<T> 
                 if (fwd_live) {
                     c_samples += 1;
                     c_levels += (unsigned)v.levels;
+                    since_shaded += 1;
                     if (sigma > (T)opt.sigma_thresh) {
                         c_shaded += 1;
+                        since_shaded = 0;
                         light *= exp_sp<T>(-delta_t * r.dscale * sigma);
                         if (light <= (T)opt.stop_thresh) fwd_live = false;
                     }
                 }
                 advance(r, delta_t);
             }
+            c_tail = since_shaded;
         }
     }
     // every lane reaches the reductions
@@ -2764,6 +2899,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_stats_kernel(TreeDev<T> 
     c_bwd = wave_sum(c_bwd);
     c_bwd_pos = wave_sum(c_bwd_pos);
     c_levels = wave_sum(c_levels);
+    c_tail = wave_sum(c_tail);
     if ((threadIdx.x & 63) == 0) {
         atomicAdd(stats + 0, c_rays);
         atomicAdd(stats + 1, c_hit);
@@ -2772,6 +2908,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_stats_kernel(TreeDev<T> 
         atomicAdd(stats + 4, c_bwd);
         atomicAdd(stats + 5, c_bwd_pos);
         atomicAdd(stats + 6, c_levels);
+        atomicAdd(stats + 7, c_tail);
     }
 }
 

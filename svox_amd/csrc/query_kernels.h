@@ -174,58 +174,6 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(TreeDev<T> tr, con
     }
 }
 
-// Measurement aid (svox_gather_probe): every group of `lanes` consecutive lanes reads the first
-// lanes * 16 bytes of 4 * iters pseudo-random units of the buffer, 16 bytes per lane, four reads in
-// flight.  The checksum keeps the reads alive; the store never happens for data a caller can have (it
-// would need two exact 32-bit values).
-__device__ __forceinline__ uint32_t probe_hash(uint32_t x) {
-    x ^= x >> 16;
-    x *= 0x7feb352dU;
-    x ^= x >> 15;
-    x *= 0x846ca68bU;
-    x ^= x >> 16;
-    return x;
-}
-__global__ __launch_bounds__(256) void gather_probe_kernel(const uint4* __restrict__ buffer, uint64_t n_units,
-                                                           int unit16, int lanes, int iters,
-                                                           uint4* __restrict__ sink) {
-    uint4 acc = make_uint4(0u, 0u, 0u, 0u);
-    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
-    const uint32_t piece = tid % (uint32_t)lanes;
-    uint32_t seed = tid / (uint32_t)lanes;
-    for (int it = 0; it < iters; ++it) {
-        uint4 v[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            seed = probe_hash(seed + 0x9e3779b9u * (uint32_t)(k + 1));
-            const uint64_t unit = ((uint64_t)seed * n_units) >> 32;
-            v[k] = buffer[unit * (uint64_t)unit16 + piece];
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            acc.x ^= v[k].x;
-            acc.y += v[k].y;
-            acc.z ^= v[k].z;
-            acc.w += v[k].w;
-        }
-    }
-    if (acc.x == 0x12345678u && acc.y == 0x9abcdef0u) sink[blockIdx.x * 256u + threadIdx.x] = acc;
-}
-
-// Measurement aid (svox_atomic_probe): per round the wavefront adds 1.0f to 64 / run consecutive-float runs
-// at pseudo-random run-aligned places.
-__global__ __launch_bounds__(256) void atomic_probe_kernel(float* __restrict__ scratch, uint64_t n_runs, int run,
-                                                           int iters) {
-    const int lane = threadIdx.x & 63;
-    uint32_t seed = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 977u;
-    for (int it = 0; it < iters; ++it) {
-        seed = probe_hash(seed + 0x9e3779b9u);
-        const uint32_t s = probe_hash(seed + (uint32_t)(lane / run));
-        const uint64_t at = ((uint64_t)s * n_runs) >> 32;
-        atomicAdd(scratch + at * (uint64_t)run + (lane % run), 1.0f);
-    }
-}
-
 // calc_corner_kernel, svox_kernel.cu:91-115: climb parent links from the leaf's node to the
 // root; per level result = (result + cell index) / N.
 template <typename T>
@@ -260,16 +208,23 @@ __global__ __launch_bounds__(kQueryThreads) void corners_kernel(const int32_t* _
     out[q * 3 + 2] = res[2];
 }
 
-// The child table with the empty leaves marked: a leaf cell (child == 0) whose density is not > 0
-// receives SVOX_EMPTY_LEAF, every other cell its child entry.  One thread per cell.
+// The child table with the leaves a render skips marked: a leaf cell (child == 0) whose density -- after the shifted
+// softplus of rt_kernel.cu:276-277 where `softplus` says so -- is not > thresh receives SVOX_EMPTY_LEAF, every other
+// cell its child entry.  One thread per cell.
 template <typename T>
-__global__ __launch_bounds__(256) void mark_empty_leaves_kernel(const T* __restrict__ data,
-                                                                const int32_t* __restrict__ child, int64_t cells,
-                                                                int K, int32_t* __restrict__ marks) {
+__global__ __launch_bounds__(256) void mark_leaves_kernel(const T* __restrict__ data, const int32_t* __restrict__ child,
+                                                          int64_t cells, int K, T thresh, bool softplus,
+                                                          int32_t* __restrict__ marks) {
     const int64_t i = blockIdx.x * 256ll + threadIdx.x;
     if (i >= cells) return;
     const int32_t c = child[i];
-    marks[i] = c != 0 ? c : (data[i * K + (K - 1)] > T(0) ? 0 : SVOX_EMPTY_LEAF);
+    int32_t m = c;
+    if (c == 0) {
+        T sigma = data[i * K + (K - 1)];
+        if (softplus) sigma = softplus_m1(sigma);
+        m = sigma > thresh ? 0 : SVOX_EMPTY_LEAF;
+    }
+    marks[i] = m;
 }
 
 // Zero-fill used in place of a memset so that a caller may capture the call in a graph.

@@ -26,9 +26,45 @@ namespace {
 using namespace svox;
 
 thread_local char g_error[512] = "";
-// bit 0: always take the generic kernels; bit 1: small batches run like large ones;
-// bit 2: forward launches never take the two-wavefront kernel; bit 3: they always do (where it applies)
-int g_debug_flags = 0;
+// Debug flags of the calling thread (svox_set_debug_flags): bit 0: always take the generic kernels; bit 1: small
+// batches run like large ones; bit 2: forward launches never take the two-wavefront kernel; bit 3: they always
+// do (where it applies).  Per thread, so that one thread's tests cannot change the kernels of another's calls.
+thread_local int g_debug_flags = 0;
+
+// Launch-shape overrides for experiments, read from the environment once, when the first launch of the process
+// picks a shape; the library has no other mutable state besides g_error / g_debug_flags (per thread) and the
+// per-device address of `scratch`.  Every field is 0 / -1 ("not set") in normal use:
+//   SVOX_PER_WAVE      rays a persistent wavefront of a batch launch owns (64, 128, 256, 512 or 1024)
+//   SVOX_REFILL        idle lanes at which such a wavefront takes new rays (1..64)
+//   SVOX_XCD_GROUP     consecutive image tiles handed to one XCD (1..4096)
+//   SVOX_TILE_ORDER    0: 16x16 blocks of an image row by row, 1: ring by ring from the middle
+//   SVOX_IMAGE_RUN     16x16 blocks of one image in a row before the next image's, in multi-image launches
+//   SVOX_SPLIT_FORWARD 0 / 1: forward launches never / always on two wavefronts per tile
+//   SVOX_SPLIT_BLOCKS  largest forward launch (in tiles) that takes two wavefronts per tile
+//   SVOX_REPLAY_SHIFT  4 or 6: log2 of the rays a wavefront of the replay kernels takes
+struct Tuning {
+    int per_wave = 0, refill = 0, xcd_group = 0, tile_order = -1, image_run = -1, split_forward = -1, replay_shift = -1;
+    long split_blocks = -1;
+};
+const Tuning& tuning() {
+    static const Tuning t = [] {
+        Tuning v;
+        auto num = [](const char* name, long unset) {
+            const char* e = getenv(name);
+            return e ? atol(e) : unset;
+        };
+        v.per_wave = (int)num("SVOX_PER_WAVE", 0);
+        v.refill = (int)num("SVOX_REFILL", 0);
+        v.xcd_group = (int)num("SVOX_XCD_GROUP", 0);
+        v.tile_order = (int)num("SVOX_TILE_ORDER", -1);
+        v.image_run = (int)num("SVOX_IMAGE_RUN", -1);
+        v.split_forward = (int)num("SVOX_SPLIT_FORWARD", -1);
+        v.split_blocks = num("SVOX_SPLIT_BLOCKS", -1);
+        v.replay_shift = (int)num("SVOX_REPLAY_SHIFT", -1);
+        return v;
+    }();
+    return t;
+}
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -177,13 +213,13 @@ int check_rays(const SvoxRaysSpec* rays) {
     return SVOX_OK;
 }
 
-// default options on an fp32 octree whose record matches the format: the specialised kernels
-// (density_softplus only in the forward kernel: `softplus_ok`).  Returns what SVOX_DISPATCH_OCTREE
+// default options on an fp32 octree whose record matches the format: the specialised kernels (with or without
+// density_softplus, which they apply to the densities they fetch).  Returns what SVOX_DISPATCH_OCTREE
 // switches on: 0 for RGBA, basis_dim for spherical harmonics, kLobeKernels + basis_dim for lobes (spherical
 // gaussians and anisotropic ones), -1 for everything the generic kernels serve.
 constexpr int kLobeKernels = 100;
-int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, bool softplus_ok = false) {
-    if (!octree_fast_ok(tree) || (opt->density_softplus && !softplus_ok)) return -1;
+int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
+    if (!octree_fast_ok(tree)) return -1;
     if (opt->format == SVOX_FORMAT_RGBA) return tree->data_dim == 4 ? 0 : -1;
     if (opt->format != SVOX_FORMAT_SH && opt->format != SVOX_FORMAT_SG && opt->format != SVOX_FORMAT_ASG) return -1;
     const int D = opt->basis_dim;
@@ -203,46 +239,53 @@ Lobes lobes_of(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
     return Lobes{(const float*)tree->extra_data, tree->extra_cols, opt->format};
 }
 
-// The tree as the octree march kernels see it: with the caller's marks of the empty leaves in place
-// of the child table where they apply (no leaf with sigma <= 0 may contribute: sigma_thresh >= 0).
-TreeDev<float> march_tree(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
+// Whether a launch that works on every leaf with density > need_thresh (the forward pass: opt->sigma_thresh; the
+// backward passes, se_grad and the noting passes: 0) may read the caller's marks in place of the child table: the
+// marks hide the leaves whose density is not > child_marks_thresh, which must all be leaves the launch skips.
+bool marks_apply(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, float need_thresh) {
+    return tree->child_marks && tree->child_marks_thresh >= 0.0f && need_thresh >= tree->child_marks_thresh &&
+           (tree->child_marks_softplus != 0) == (opt->density_softplus != 0);
+}
+// ... and whether the marks hide exactly the leaves the launch skips: every leaf they let through is shaded.
+bool marks_decide(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, float need_thresh) {
+    return marks_apply(tree, opt, need_thresh) && need_thresh == tree->child_marks_thresh;
+}
+
+// The tree as the octree march kernels see it: with the caller's marks in place of the child table where they apply.
+TreeDev<float> march_tree(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, float need_thresh = 0.0f) {
     TreeDev<float> d = make_tree<float>(tree);
-    // (softplus of any stored density is > 0: no leaf is empty then)
-    if (tree->child_marks && opt->sigma_thresh >= 0.0f && !opt->density_softplus) d.child = tree->child_marks;
+    if (marks_apply(tree, opt, need_thresh)) d.child = tree->child_marks;
     return d;
+}
+
+// the workspace argument of a forward launch that takes no notes
+ReplaySpace no_notes() {
+    ReplaySpace ws{};
+    ws.spin_limit = (g_debug_flags & 16) ? 1 : 0;
+    return ws;
 }
 
 // Items (rays) a persistent wavefront owns.  With few rays every wavefront gets one 64-item chunk so
 // that the launch spreads over as many SIMDs as possible; with many, several chunks, which lets lanes
 // whose rays end early pick up new ones (measured on 1M random rays: forward best at 256 rays per
 // wavefront, backward -- two marches per ray, longer-lived lanes -- at 512).
-// SVOX_PER_WAVE / SVOX_REFILL override the choice for experiments.
 int pick_per_wave(int64_t total_items, bool backward) {
-    static const int forced = [] {
-        const char* e = getenv("SVOX_PER_WAVE");
-        return e ? atoi(e) : 0;
-    }();
+    const int forced = tuning().per_wave;
     if (forced == 64 || forced == 128 || forced == 256 || forced == 512 || forced == 1024) return forced;
     if (total_items < (int64_t)64 * 1024 * 8 && !(g_debug_flags & 2)) return 64;
     return backward ? 512 : 256;
 }
 
 int pick_refill() {
-    static const int forced = [] {
-        const char* e = getenv("SVOX_REFILL");
-        return e ? atoi(e) : 0;
-    }();
+    const int forced = tuning().refill;
     return forced >= 1 && forced <= 64 ? forced : 16;
 }
 
 // Image tiles handed to one XCD in a row (chunk_of_block): 16 tiles are four 16x16 pixel blocks.
 // Measured on 8 poses of 800x800: 1 -> 16 shortens the launch by 2-3 %, larger runs gain no more and
-// start to unbalance the XCDs.  SVOX_XCD_GROUP overrides it for experiments.
+// start to unbalance the XCDs.
 int pick_xcd_group() {
-    static const int forced = [] {
-        const char* e = getenv("SVOX_XCD_GROUP");
-        return e ? atoi(e) : 0;
-    }();
+    const int forced = tuning().xcd_group;
     return forced >= 1 && forced <= 4096 ? forced : 16;
 }
 
@@ -294,19 +337,12 @@ ImageSource<T> image_source(const SvoxCameraSpec* cam, int n_images, int64_t pos
     // blocks (slabs of the tree) share more leaves in L2 than rings do.  Measured (us, rows / rings):
     // one 800x800 pose of the sparse SH16 tree 317 / 304, 2 poses 344 / 314, 8 poses 695 / 670,
     // 16 poses 1159 / 1174; one pose of the dense 128^3 tree 385 / 340; 4 NDC poses 3538 / 3957.
-    // SVOX_TILE_ORDER (0 rows, 1 rings) overrides it for experiments.
     {
-        static const int forced = [] {
-            const char* e = getenv("SVOX_TILE_ORDER");
-            return e ? atoi(e) : -1;
-        }();
+        const int forced = tuning().tile_order;
         s.inside_out = forced == 0 || forced == 1 ? forced : (opt->ndc_width > 0 ? 0 : 1);
     }
     if (n_images > 1) {
-        static const int forced = [] {
-            const char* e = getenv("SVOX_IMAGE_RUN");
-            return e ? atoi(e) : -1;
-        }();
+        const int forced = tuning().image_run;
         s.run = forced >= 0 ? forced : 4;
     }
     return s;
@@ -346,17 +382,10 @@ unsigned blocks_for(int64_t items, int per_block) { return (unsigned)((items + p
 // 0.75 (four).  Where every tile is heavy and the GPU full it costs: four 1008x756 NDC poses (47 628
 // tiles) 3 %, two of them 1 % (one gains 2 %), a batch of 256 Ki unrelated rays 33 %.  Hence: images of
 // up to 98 304 tiles (eight 800x800 poses are 80 000) -- but 16 384 under NDC, where every ray passes
-// through the tree --, ray batches of up to 128 Ki rays.  SVOX_SPLIT_FORWARD=1 / 0 forces / forbids it;
-// SVOX_SPLIT_BLOCKS sets the largest launch that takes it (experiments).
+// through the tree --, ray batches of up to 128 Ki rays.
 bool use_split_forward(unsigned blocks, bool image, const SvoxRenderOptions* opt) {
-    static const int forced = [] {
-        const char* e = getenv("SVOX_SPLIT_FORWARD");
-        return e ? atoi(e) : -1;
-    }();
-    static const long limit = [] {
-        const char* e = getenv("SVOX_SPLIT_BLOCKS");
-        return e ? atol(e) : -1l;
-    }();
+    const int forced = tuning().split_forward;
+    const long limit = tuning().split_blocks;
     if (g_debug_flags & 12) return (g_debug_flags & 8) != 0;
     if (forced >= 0) return forced > 0;
     if (limit >= 0) return (long)blocks <= limit;
@@ -373,28 +402,38 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
                     void* out, hipStream_t stream) {
     const int64_t items = total_items_of(src);
     if constexpr (sizeof(T) == 4) {
-        const int D = fast_basis(tree, opt, true);
+        const int D = fast_basis(tree, opt);
         if (D >= 0) {
             const unsigned blocks = blocks_for(items, src.per_wave);
             const Source dealt = dealt_out(src, blocks);
-#define SVOX_LAUNCH_FORWARD(ACCUM, REFILL)                                                                     \
-    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, ACCUM, REFILL>), dim3(blocks), \
-                                               dim3(kMarchThreads), 0, stream, march_tree(tree, opt), dealt,    \
-                                               *opt, (float*)out, ReplaySpace{}))
+            const TreeDev<float> tr = march_tree(tree, opt, opt->sigma_thresh);
+            const ReplaySpace none = no_notes();
+            // marks made with this launch's own threshold: every leaf they let through is shaded
+            const bool all_shaded = !tree->weight_accum && marks_decide(tree, opt, opt->sigma_thresh);
+#define SVOX_LAUNCH_FORWARD(ACCUM, REFILL, ALL)                                                                   \
+    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, ACCUM, REFILL, false, false, ALL>), \
+                                               dim3(blocks), dim3(kMarchThreads), 0, stream, tr, dealt, *opt,      \
+                                               (float*)out, none))
             const bool refill = src.per_wave > kMarchThreads;
             if (!refill && !tree->weight_accum && use_split_forward(blocks, is_image_source(src), opt)) {
-                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false>), dim3(blocks),
-                                                           dim3(kSplitThreads), 0, stream, march_tree(tree, opt), dealt,
-                                                           *opt, (float*)out, ReplaySpace{}));
+                if (all_shaded) {
+                    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false, false, true>),
+                                                               dim3(blocks), dim3(kSplitThreads), 0, stream, tr, dealt,
+                                                               *opt, (float*)out, none));
+                } else {
+                    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false>),
+                                                               dim3(blocks), dim3(kSplitThreads), 0, stream, tr, dealt,
+                                                               *opt, (float*)out, none));
+                }
                 return;
             }
             if (tree->weight_accum) {
                 // accumulation is an analysis pass: one variant is enough
-                SVOX_LAUNCH_FORWARD(true, true);
+                SVOX_LAUNCH_FORWARD(true, true, false);
             } else if (refill) {
-                SVOX_LAUNCH_FORWARD(false, true);
+                if (all_shaded) { SVOX_LAUNCH_FORWARD(false, true, true); } else { SVOX_LAUNCH_FORWARD(false, true, false); }
             } else {
-                SVOX_LAUNCH_FORWARD(false, false);
+                if (all_shaded) { SVOX_LAUNCH_FORWARD(false, false, true); } else { SVOX_LAUNCH_FORWARD(false, false, false); }
             }
 #undef SVOX_LAUNCH_FORWARD
             return;
@@ -415,7 +454,7 @@ NoteStamp stamp_of(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays, const Svo
     uint32_t step_bits, thresh_bits;
     memcpy(&step_bits, &opt->step_size, 4);
     memcpy(&thresh_bits, &opt->sigma_thresh, 4);
-    st.word[0] = 0x73766f786e6f7465ull ^ (unsigned long long)rays->n_rays;
+    st.word[0] = 0x73766f786e6f7465ull ^ (unsigned long long)rays->n_rays ^ (opt->density_softplus ? 1ull << 62 : 0ull);
     st.word[1] = (unsigned long long)(uintptr_t)tree->data;
     st.word[2] = (unsigned long long)(uintptr_t)rays->origins;
     st.word[3] = ((unsigned long long)thresh_bits << 32) | step_bits;
@@ -502,6 +541,7 @@ int launch_noted(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOp
     const int rc = zero_fill(ws.stocks_taken, 16, stream);
     if (rc) return rc;
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
+    ws.spin_limit = (g_debug_flags & 16) ? 1 : 0;
     const bool refill = src.per_wave > kMarchThreads;
     const bool split = !refill && use_split_forward(blocks, is_image_source(src), opt);
     const dim3 threads(split ? kSplitThreads : kMarchThreads);
@@ -603,10 +643,12 @@ int se_grad_prepare(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, void
 // Can notes be taken (launch_noted) and used (replay_backward_kernel)?  The octree kernels, a forward
 // pass whose threshold does not admit leaves the backward pass ignores, no weight accumulator, and a
 // workspace with a chunk for every ray.
+bool notes_possible(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
+    return tree->dtype == SVOX_F32 && fast_basis(tree, opt) >= 0 && !tree->weight_accum && opt->sigma_thresh >= 0.0f;
+}
 bool noted_ok(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt, int64_t n_slots, void* workspace,
                      int64_t workspace_bytes) {
-    if (tree->dtype != SVOX_F32 || fast_basis(tree, opt) < 0 || tree->weight_accum) return false;
-    if (!(opt->sigma_thresh >= 0.0f)) return false;
+    if (!notes_possible(tree, opt)) return false;
     ReplaySpace ws;
     return carve_workspace(workspace, workspace_bytes, n_slots, &ws);
 }
@@ -623,12 +665,9 @@ NoteStamp stamp_of_image(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, in
 // log2 of the rays a wavefront of the replay kernels takes: 16 rays for the pixels of images (neighbours,
 // long together) and for batches that do not fill the GPU with 64 (up to 64 Ki rays: 4 096 rays of a 16^3
 // tree 246 -> 196 us, 64 Ki rays 350 -> 333 us), 64 for larger ray batches (1 Mi rays: 0.68 against 0.83 ms
-// with 16).  SVOX_REPLAY_SHIFT = 4 or 6 overrides.
+// with 16).
 int replay_ray_shift(bool image, int64_t n_rays) {
-    static const int forced_shift = [] {
-        const char* e = getenv("SVOX_REPLAY_SHIFT");
-        return e ? atoi(e) : -1;
-    }();
+    const int forced_shift = tuning().replay_shift;
     return forced_shift == 4 || forced_shift == 6 ? forced_shift : (image || n_rays <= 65536 ? 4 : 6);
 }
 
@@ -1170,20 +1209,28 @@ int svox_se_grad_image_ws(const SvoxTreeSpec* tree, const SvoxCameraSpec* cam, c
                               workspace_bytes, n_slots, stamp_of_image(tree, cam, 1, &plain), (hipStream_t)stream);
 }
 
-int svox_mark_empty_leaves(const SvoxTreeSpec* tree, int32_t* marks_out, void* stream) {
+int svox_mark_leaves_below(const SvoxTreeSpec* tree, float sigma_thresh, int32_t density_softplus, int32_t* marks_out,
+                           void* stream) {
     int rc = check_tree(tree, true);
     if (rc) return rc;
     if (!marks_out) return fail(SVOX_ERR_NULL_POINTER, "marks_out is NULL");
+    if (!(sigma_thresh >= 0.0f)) return fail(SVOX_ERR_BAD_SHAPE, "marks need a sigma_thresh >= 0, got %g", (double)sigma_thresh);
     const int64_t cells = tree->capacity * tree->N * tree->N * tree->N;
     if (cells == 0) return SVOX_OK;
     const unsigned blocks = blocks_for(cells, 256);
     if (tree->dtype == SVOX_F32)
-        hipLaunchKernelGGL((mark_empty_leaves_kernel<float>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
-                           (const float*)tree->data, tree->child, cells, tree->data_dim, marks_out);
+        hipLaunchKernelGGL((mark_leaves_kernel<float>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                           (const float*)tree->data, tree->child, cells, tree->data_dim, sigma_thresh,
+                           density_softplus != 0, marks_out);
     else
-        hipLaunchKernelGGL((mark_empty_leaves_kernel<double>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
-                           (const double*)tree->data, tree->child, cells, tree->data_dim, marks_out);
-    return check_launch("mark_empty_leaves");
+        hipLaunchKernelGGL((mark_leaves_kernel<double>), dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                           (const double*)tree->data, tree->child, cells, tree->data_dim, (double)sigma_thresh,
+                           density_softplus != 0, marks_out);
+    return check_launch("mark_leaves_below");
+}
+
+int svox_mark_empty_leaves(const SvoxTreeSpec* tree, int32_t* marks_out, void* stream) {
+    return svox_mark_leaves_below(tree, 0.0f, 0, marks_out, stream);
 }
 
 int svox_grid_weight_render(const void* data, int32_t reso, int32_t dtype, const SvoxCameraSpec* cam,
@@ -1261,37 +1308,24 @@ int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions*
     int od;
     const int rc = check_render(tree, opt, &od);
     if (rc) return rc;
-    return fast_basis(tree, opt, true) >= 0 ? 1 : 0;
+    return fast_basis(tree, opt) >= 0 ? 1 : 0;
 }
 
-int svox_gather_probe(const void* buffer, int64_t bytes, int32_t unit_bytes, int32_t lanes_per_unit, int32_t iters,
-                      int32_t blocks, void* sink, void* stream) {
-    if (!buffer || !sink) return fail(SVOX_ERR_NULL_POINTER, "svox_gather_probe: NULL buffer or sink");
-    if (unit_bytes != 64 && unit_bytes != 128 && unit_bytes != 256)
-        return fail(SVOX_ERR_BAD_SHAPE, "svox_gather_probe: unit_bytes must be 64, 128 or 256");
-    if ((lanes_per_unit != 1 && lanes_per_unit != 4 && lanes_per_unit != 8 && lanes_per_unit != 16) ||
-        lanes_per_unit * 16 > unit_bytes)
-        return fail(SVOX_ERR_BAD_SHAPE, "svox_gather_probe: lanes_per_unit must be 1, 4, 8 or 16 and fit the unit");
-    if (((uintptr_t)buffer & 15u) || bytes < unit_bytes || bytes / unit_bytes > 0xffffffffll || iters < 1 ||
-        blocks < 1 || blocks > (1 << 20))
-        return fail(SVOX_ERR_BAD_SHAPE, "svox_gather_probe: buffer, iters or blocks out of range");
-    hipLaunchKernelGGL(gather_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       (const uint4*)buffer, (uint64_t)(bytes / unit_bytes), unit_bytes / 16, lanes_per_unit, iters,
-                       (uint4*)sink);
-    return check_launch("gather_probe");
+int svox_notes_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
+    int od;
+    const int rc = check_render(tree, opt, &od);
+    if (rc) return rc;
+    return notes_possible(tree, opt) ? 1 : 0;
 }
 
-int svox_atomic_probe(void* scratch, int64_t bytes, int32_t run_floats, int32_t iters, int32_t blocks, void* stream) {
-    if (!scratch) return fail(SVOX_ERR_NULL_POINTER, "svox_atomic_probe: NULL scratch");
-    if (run_floats != 1 && run_floats != 4 && run_floats != 16 && run_floats != 64)
-        return fail(SVOX_ERR_BAD_SHAPE, "svox_atomic_probe: run_floats must be 1, 4, 16 or 64");
-    const int64_t n_runs = bytes / (4 * (int64_t)run_floats);
-    if (((uintptr_t)scratch & 63u) || n_runs < 1 || n_runs > 0xffffffffll || iters < 1 || blocks < 1 ||
-        blocks > (1 << 20))
-        return fail(SVOX_ERR_BAD_SHAPE, "svox_atomic_probe: scratch (64-byte aligned), iters or blocks out of range");
-    hipLaunchKernelGGL(atomic_probe_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       (float*)scratch, (uint64_t)n_runs, run_floats, iters);
-    return check_launch("atomic_probe");
+int svox_give_up_count(int64_t* count_out) {
+    if (!count_out) return fail(SVOX_ERR_NULL_POINTER, "count_out is NULL");
+    unsigned int n = 0;
+    hipError_t err = hipDeviceSynchronize();
+    if (err == hipSuccess) err = hipMemcpyFromSymbol(&n, HIP_SYMBOL(split_give_ups), sizeof(n), 0, hipMemcpyDeviceToHost);
+    if (err != hipSuccess) return fail(SVOX_ERR_LAUNCH, "svox.give_up_count: %s", hipGetErrorString(err));
+    *count_out = (int64_t)n;
+    return SVOX_OK;
 }
 
 }  // extern "C"

@@ -641,15 +641,22 @@ class N3Tree(nn.Module):
         if getattr(self, "_leaf_marks", None) is not None:
             if self._leaf_marks_key == self._marks_key():
                 spec.child_marks = self._leaf_marks
+                spec.child_marks_thresh, spec.child_marks_softplus = getattr(self, "_leaf_marks_made_with", (0.0, False))
             else:
                 self._leaf_marks = None      # the tree has changed since: the marks are void
         return spec
 
     # ------------------------------------------------------------------ marks of the empty leaves
-    def mark_empty_leaves(self):
+    def mark_empty_leaves(self, sigma_thresh=0.0, density_softplus=False):
         """For a tree that will be rendered many times as it is (beyond the reference): note which
         leaves have no density, so that the renderers pass through them without reading it.  Renders
         are bit-identical and faster on sparse scenes.
+
+        sigma_thresh, density_softplus: of the renders that will follow.  With 0 / False (the default) the marks
+        serve every render, backward pass and se_grad call of a renderer without density_softplus.  Marks made
+        with a renderer's own `sigma_thresh` (1e-2 for `fast=True`) let its forward renders also skip the leaves
+        below the threshold and read a leaf's density together with its colour; calls that need those leaves
+        (backward passes, renders with a smaller threshold) then run without marks.
 
         The marks describe the tree as it is now.  They are dropped by every method of the tree and
         its views that writes values or changes the structure, and by in-place torch operations on
@@ -657,7 +664,8 @@ class N3Tree(nn.Module):
         `tree.data.data -= ...` as in svox's own toy example -- does not: call `tree.touch()`
         (or `clear_leaf_marks()`, or this method again) after such a write."""
         self._leaf_marks = None
-        self._leaf_marks = _C.mark_empty_leaves(self._spec())
+        self._leaf_marks = _C.mark_empty_leaves(self._spec(), sigma_thresh, density_softplus)
+        self._leaf_marks_made_with = (float(sigma_thresh), bool(density_softplus))
         self._leaf_marks_key = self._marks_key()
         return self
 

@@ -27,3 +27,21 @@ def gpu():
     from svox_amd.csrc import _abi
     _abi.load_library()  # raises if the HIP library is not built: GPU tests never fall back
     return torch.device("cuda:0")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """How close to the gradient gate the kernels ran: the worst error of every test that compared a gradient."""
+    try:
+        from util import GATE_LOG
+    except ImportError:
+        return
+    if not GATE_LOG:
+        return
+    worst = {}
+    for label, err, limit, slack in GATE_LOG:
+        key = (label, limit, slack)
+        worst[key] = max(worst.get(key, 0.0), err)
+    tr = terminalreporter
+    tr.write_sep("-", "gradient gate: worst relative error per test (limit; * = order slack of the oracle taken off)")
+    for (label, limit, slack), err in sorted(worst.items(), key=lambda kv: -kv[1] / kv[0][1])[:60]:
+        tr.write_line(f"  {err:9.3e} of {limit:.0e}{'*' if slack else ' '} {label}")

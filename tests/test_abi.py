@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_host_only_calls():
     lib = _abi.load_library()
-    assert lib.svox_abi_version() == _abi.ABI_VERSION == 2
+    assert lib.svox_abi_version() == _abi.ABI_VERSION == 3
     assert lib.svox_status_string(0) == b"ok" and lib.svox_status_string(-2) == b"bad shape"
     assert lib.svox_out_data_dim(0, -1, 4) == 3
     assert lib.svox_out_data_dim(1, 16, 49) == 3

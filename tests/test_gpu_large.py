@@ -1,5 +1,5 @@
-"""Trees whose data tensor has more than 2^31 elements (64-bit addressing inside the kernels) and
-full-size property checks that need no CPU oracle."""
+"""Trees whose data tensor has more than 2^31 elements (64-bit addressing inside the kernels), the
+benchmark configurations at full size against the CPU oracle, and full-size property checks."""
 import numpy as np
 import pytest
 import torch
@@ -313,3 +313,83 @@ def test_config2_dense128_sh9_query_and_render_against_the_oracle(gpu, oracle_mo
     out.backward(go.to(gpu))
     err, ok = grad_close(dev.data.grad.cpu().numpy(), ref_grad)
     assert ok, ("autograd", err)
+
+
+def _benchmark_tree_and_oracle(gpu, oracle_mod):
+    tree = synth.shell_tree(depth=9, n_spheres=24, data_format="SH16", seed=0, device=gpu)
+    host = oracle_mod.Tree(tree.data.detach().cpu().numpy(), tree.child.cpu().numpy(), tree.parent_depth.cpu().numpy(),
+                           tree.offset.cpu().numpy(), tree.invradius.cpu().numpy())
+    return tree, host
+
+
+def test_config3_eight_poses_in_one_call_against_the_oracle(gpu, oracle_mod):
+    """The benchmark's timed forward step at full size: the 512^3 sparse SH16 tree, 8 poses of 800x800 as ONE
+    render_persp call on the stack of poses (the empty leaves are marked inside the call, the launch runs on two
+    wavefronts per tile), fast thresholds.  Every picture and every pose's visit counts equal the oracle's
+    (render_image_kernel, rt_kernel.cu:799-819)."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 16 * 2 ** 30:
+        pytest.skip("needs 16 GB of free device memory")
+    tree, host = _benchmark_tree_and_oracle(gpu, oracle_mod)
+    W = H = 800
+    fx = 1111.111
+    poses = synth.orbit_poses(8, seed=1, radius=4.0)
+    r = svox.VolumeRenderer(tree, step_size=5e-4)
+    opt = r._get_options(True)
+    assert C._marks_for_this_call(tree._spec(), opt, 8 * W * H) is not None   # the call is one that marks
+    with torch.no_grad():
+        imgs = r.render_persp(torch.stack(poses).to(gpu), width=W, height=H, fx=fx, fast=True)
+    assert imgs.shape == (8, H, W, 3)
+    got = imgs.cpu().numpy()
+    threads = min(16, oracle_mod.max_threads())
+    from svox_amd.renderer import _make_camera_spec
+    shaded = 0
+    for i, pose in enumerate(poses):
+        ref, ref_stats = oracle_mod.volume_render_image(host, pose, fx, fx, W, H, opt, want_stats=True, n_threads=threads)
+        assert np.array_equal(got[i], ref), f"pose {i}: {np.abs(got[i] - ref).max()}"
+        stats = C.volume_render_stats(tree._spec(), _make_camera_spec(pose.to(gpu).contiguous(), W, H, fx, fx), opt)
+        for k in ("rays", "rays_hit", "samples", "samples_shaded", "levels", "samples_tail"):
+            assert stats[k] == ref_stats[k], (i, k)
+        shaded += stats["samples_shaded"]
+    assert shaded > 4_000_000
+
+
+def test_config4_training_step_against_the_oracle(gpu, oracle_mod):
+    """The benchmark's training step at full size: 1 Mi rays drawn from the 8 poses, through autograd as the
+    benchmark runs it (the forward pass keeps notes, the backward pass replays them).  The picture equals the
+    oracle's trace_ray with the fast thresholds (rt_kernel.cu:222-321); the gradient is within 1e-4 of the oracle's
+    exact sum of trace_ray_backward's terms (rt_kernel.cu:323-477, 1059-1083) -- random rays seldom share a leaf,
+    so no allowance for the order of the additions is made here."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 16 * 2 ** 30:
+        pytest.skip("needs 16 GB of free device memory")
+    tree, host = _benchmark_tree_and_oracle(gpu, oracle_mod)
+    W = H = 800
+    fx = 1111.111
+    poses = synth.orbit_poses(8, seed=1, radius=4.0)
+    g = torch.Generator().manual_seed(7)
+    B = 1 << 20
+    per_pose = [svox.VolumeRenderer.persp_rays(p, W, H, fx) for p in poses]
+    pick = torch.randint(0, 8 * W * H, (B,), generator=g)
+    all_o = torch.cat([x.origins for x in per_pose])
+    all_d = torch.cat([x.dirs for x in per_pose])
+    o, d = all_o[pick].contiguous(), all_d[pick].contiguous()
+    del all_o, all_d, per_pose
+    go = torch.randn(B, 3, generator=g) * 1e-2
+    r = svox.VolumeRenderer(tree, step_size=5e-4)
+    opt = r._get_options(True)
+    tree.data.grad = None
+    out = r(svox.Rays(o.to(gpu), d.to(gpu), d.to(gpu)), fast=True)
+    out.backward(go.to(gpu))
+    threads = min(16, oracle_mod.max_threads())
+    ref = oracle_mod.volume_render(host, o, d, d, opt, n_threads=threads)
+    assert np.array_equal(out.detach().cpu().numpy(), ref)
+    ref_grad = oracle_mod.volume_render_backward(host, o, d, d, opt, go, n_threads=threads)
+    assert np.abs(ref_grad).max() > 0
+    err, ok = grad_close(tree.data.grad.cpu().numpy(), ref_grad, what="config 4, notes replayed")
+    assert ok, err
+    # the same gradient from the stateless operator (one noting march in a workspace of its own)
+    grad = C.volume_render_backward(tree._spec(), rays_spec(svox.Rays(o, d, d), gpu), opt, go.to(gpu))
+    err, ok = grad_close(grad.cpu().numpy(), ref_grad, what="config 4, stateless backward")
+    assert ok, err
+    tree.data.grad = None

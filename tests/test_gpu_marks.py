@@ -219,3 +219,98 @@ def test_large_multi_pose_launch_marks_the_leaves_for_itself(gpu, monkeypatch):
     C.volume_render_images(tree._spec(), cam, options(tree, step_size=1e-3, sigma_thresh=-1.0))
     C.volume_render_images(tree._spec(), cam, options(tree, step_size=1e-3, density_softplus=True))
     assert made == [1]
+
+
+@pytest.mark.parametrize("softplus", [False, True])
+def test_marks_made_with_a_threshold(gpu, softplus):
+    """svox_mark_leaves_below: a leaf is marked exactly when trace_ray would skip it (rt_kernel.cu:276-278)."""
+    tree = synth.dense_tree(3, "SH4", seed=2, zero_fraction=0.3, sigma="lognormal")
+    tree.data.data[0, 0, 0, 1, -1] = float("nan")
+    tree.data.data[1, 1, 0, 1, -1] = -1.0
+    tree = tree.to(gpu)
+    thresh = 0.75
+    marks = C.mark_empty_leaves(tree._spec(), thresh, softplus)
+    raw = tree.data.data[..., -1]
+    sigma = torch.log(1 + torch.exp(raw - 1)) if softplus else raw
+    keep = sigma > thresh
+    near = (sigma - thresh).abs() < 1e-5          # (the device's logf may round another way right at the threshold)
+    want = torch.where(tree.child != 0, tree.child, torch.where(keep, torch.zeros_like(tree.child), torch.full_like(tree.child, -2)))
+    agree = (marks == want) | (near & (tree.child == 0))
+    assert bool(agree.all()) and (marks == -2).any() and (marks == 0).any()
+    spec = tree._spec()
+    with pytest.raises(RuntimeError, match="sigma_thresh"):
+        C.mark_empty_leaves(spec, -1.0)
+
+
+@pytest.mark.parametrize("flags", [0, 2, 4, 8])
+@pytest.mark.parametrize("fmt", ["RGBA", "SH9", "SH16"])
+def test_marks_that_decide_the_shading(gpu, oracle_mod, fmt, flags):
+    """Marks made with the render's own sigma_thresh: the forward kernels shade every leaf the marks let through
+    without a look at its density first.  Pictures equal the oracle's bit for bit on every forward kernel; calls that
+    need the leaves such marks hide (a smaller threshold, the backward pass, notes, se_grad) leave them aside."""
+    tree = synth.shell_tree(depth=6, n_spheres=6, data_format=fmt, seed=31, sigma_range=(0.002, 60.0))
+    rays = synth.sphere_rays(3000, seed=9)
+    opt = options(tree, step_size=1e-3, sigma_thresh=0.5, stop_thresh=1e-2, rgb_padding=0.001)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    want = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    c2w = synth.orbit_poses(2, seed=4, radius=2.5)
+    want_img = np.stack([oracle_mod.volume_render_image(ot, p, 60.0, 60.0, 75, 53, opt) for p in c2w])
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    cam = cam_spec(torch.stack(c2w).to(gpu), 75, 53, 60.0)
+    decided = dev._spec()
+    decided.child_marks = C.mark_empty_leaves(dev._spec(), opt.sigma_thresh)
+    decided.child_marks_thresh = opt.sigma_thresh
+    sigma = dev.data.data[..., -1]
+    between = ((sigma > 0) & (sigma <= 0.5) & (dev.child == 0)).sum().item()
+    assert between > 100 and (decided.child_marks == -2).sum().item() > between     # leaves only these marks hide
+    go = (torch.randn(3000, 3, generator=torch.Generator().manual_seed(1)) * 1e-2).to(gpu)
+    C.set_debug_flags(flags)
+    try:
+        assert np.array_equal(C.volume_render(decided, rs, opt).cpu().numpy(), want)
+        assert np.array_equal(C.volume_render_images(decided, cam, opt).cpu().numpy(), want_img)
+        # a smaller threshold needs leaves the marks hide: the marks are left aside
+        low = options(tree, step_size=1e-3, sigma_thresh=0.1, stop_thresh=1e-2, rgb_padding=0.001)
+        want_low = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, low)
+        assert np.array_equal(C.volume_render(decided, rs, low).cpu().numpy(), want_low)
+        assert not np.array_equal(want_low, want)
+        # a larger threshold may use them as plain marks
+        high = options(tree, step_size=1e-3, sigma_thresh=2.0, stop_thresh=1e-2, rgb_padding=0.001)
+        want_high = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, high)
+        assert np.array_equal(C.volume_render(decided, rs, high).cpu().numpy(), want_high)
+        if flags in (0, 2):
+            want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go.cpu())
+            for workspace in (True, False):
+                g = C.volume_render_backward(decided, rs, opt, go, workspace=workspace)
+                err, ok = grad_close(g.cpu().numpy(), want_g, what=f"marks with a threshold, workspace {workspace}")
+                assert ok, err
+            out, notes = C.volume_render_noted(decided, rs, opt)
+            assert np.array_equal(out.cpu().numpy(), want)
+            g = C.volume_render_backward_noted(decided, rs, opt, go, notes)
+            err, ok = grad_close(g.cpu().numpy(), want_g, what="marks with a threshold, notes")
+            assert ok, err
+    finally:
+        C.set_debug_flags(0)
+
+
+def test_the_tree_keeps_marks_made_with_a_threshold(gpu, oracle_mod):
+    tree = synth.shell_tree(depth=5, n_spheres=5, data_format="SH4", seed=3, sigma_range=(0.002, 60.0))
+    rays = synth.sphere_rays(2000, seed=2)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    dev = on_gpu(tree, gpu)
+    r = svox.VolumeRenderer(dev, step_size=1e-3)
+    r.sigma_thresh = 0.5
+    opt = r._get_options(True)
+    dev.mark_empty_leaves(sigma_thresh=0.5)
+    spec = dev._spec()
+    assert spec.child_marks is not None and spec.child_marks_thresh == 0.5 and not spec.child_marks_softplus
+    grays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu))
+    with torch.no_grad():
+        out = r(grays, fast=True)
+    assert np.array_equal(out.cpu().numpy(), oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt))
+    # a training step on the same tree: notes and backward pass see every leaf with density
+    go = torch.randn(2000, 3, generator=torch.Generator().manual_seed(5)) * 1e-2
+    r(grays, fast=True).backward(go.to(gpu))
+    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    err, ok = grad_close(dev.data.grad.cpu().numpy(), want_g)
+    assert ok, err

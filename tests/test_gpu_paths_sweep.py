@@ -5,7 +5,10 @@ thresholds, random background.  Paths: forward, marching backward with and witho
 forward + replayed backward, se_grad with and without a workspace -- each with the rays handled as a
 small batch and as a large one (debug flag 2), on the plain tree and with the empty leaves marked; the
 forward pass, the noted forward pass and se_grad also on either of the small-launch kernels (debug
-flags 4 and 8).
+flags 4 and 8).  With marks made with the case's own sigma_thresh (svox_mark_leaves_below: the forward kernels
+then shade every leaf the marks let through and read its density with its coefficients) the forward pass runs on
+all four kernel choices, and the backward and noted passes once each (they leave such marks aside when the
+threshold is not 0).
 
 Bars: pictures equal to the oracle's bit for bit; gradients within 1e-4 relative of the oracle's exact
 sum (fp32 terms added in float64) beyond the order slack of fp32 additions, elements below 1e-3 of the
@@ -84,6 +87,9 @@ def test_every_render_path_against_the_exact_sum_oracle(gpu, oracle_mod, case):
     plain = dev._spec()
     marked = dev._spec()
     marked.child_marks = C.mark_empty_leaves(plain)
+    decided = dev._spec()
+    decided.child_marks = C.mark_empty_leaves(plain, opt.sigma_thresh)
+    decided.child_marks_thresh = opt.sigma_thresh
     failures = []
     paths = ("fwd", "bwd", "bwd_nows", "noted", "se", "se_nows")
     combos = list(itertools.product((0, 2), ((plain, "plain"), (marked, "marked")), paths))
@@ -91,6 +97,8 @@ def test_every_render_path_against_the_exact_sum_oracle(gpu, oracle_mod, case):
     # small-launch kernels (one wavefront per 64 rays that walks and shades; two wavefronts, one for
     # each), whatever the launch size would choose
     combos += list(itertools.product((4, 8), ((plain, "plain"), (marked, "marked")), ("fwd", "noted", "se")))
+    combos += list(itertools.product((0, 2, 4, 8), ((decided, "decided"),), ("fwd",)))
+    combos += list(itertools.product((0,), ((decided, "decided"),), ("bwd", "noted", "se")))
     for flags, (spec, spec_name), name in combos:
         tag = f"{name}/flags{flags}/{spec_name}"
         C.set_debug_flags(flags)

@@ -835,10 +835,10 @@ def test_render_of_a_saved_and_loaded_tree(gpu, oracle_mod, tmp_path):
 
 @pytest.mark.parametrize("fmt", ["SH9", "RGBA"])
 def test_density_softplus_on_the_octree_forward_kernel(gpu, oracle_mod, fmt):
-    """density_softplus (rt_kernel.cu:276-277) in the specialised forward kernel: bit for bit what the
+    """density_softplus (rt_kernel.cu:276-277) in the specialised forward kernels: bit for bit what the
     generic kernel gives (one softplus routine on the device), 1e-5 from the oracle (another logf),
-    for a ray batch handled both ways and for an image; marks of empty leaves play no part (the
-    softplus of any stored density is > 0).  The backward pass of this option stays on the generic kernels."""
+    for a ray batch handled both ways and for an image; marks made without the option play no part (the
+    softplus of any stored density is > 0), marks made with it and the render's threshold decide the shading."""
     tree = synth.shell_tree(depth=6, n_spheres=5, data_format=fmt, seed=17, sigma_range=(0.5, 30.0))
     with torch.no_grad():
         tree.data[..., -1] -= 3.0                 # stored densities of both signs
@@ -850,17 +850,23 @@ def test_density_softplus_on_the_octree_forward_kernel(gpu, oracle_mod, fmt):
     rs = rays_spec(rays, gpu)
     marked = dev._spec()
     marked.child_marks = C.mark_empty_leaves(dev._spec())
+    decided = dev._spec()
+    decided.child_marks = C.mark_empty_leaves(dev._spec(), opt.sigma_thresh, True)
+    decided.child_marks_thresh, decided.child_marks_softplus = opt.sigma_thresh, True
+    assert (decided.child_marks == -2).any()
     C.set_debug_flags(1)
     try:
         generic = C.volume_render(dev._spec(), rs, opt)
     finally:
         C.set_debug_flags(0)
     assert np.abs(generic.cpu().numpy() - ref).max() <= 1e-5
-    for flags in (0, 2):
+    assert C.octree_kernels_serve(dev._spec(), opt)
+    for flags in (0, 2, 4, 8):
         C.set_debug_flags(flags)
         try:
             assert torch.equal(C.volume_render(dev._spec(), rs, opt), generic), flags
             assert torch.equal(C.volume_render(marked, rs, opt), generic), flags
+            assert torch.equal(C.volume_render(decided, rs, opt), generic), flags
         finally:
             C.set_debug_flags(0)
     c2w = synth.orbit_poses(1, seed=4, radius=2.5)[0]
@@ -868,37 +874,241 @@ def test_density_softplus_on_the_octree_forward_kernel(gpu, oracle_mod, fmt):
     img = C.volume_render_image(dev._spec(), cam, opt)
     want = oracle_mod.volume_render_image(ot, c2w, 60.0, 60.0, 75, 53, opt)
     assert np.abs(img.cpu().numpy() - want).max() <= 1e-5
+    assert torch.equal(C.volume_render_image(decided, cam, opt), img)
     C.set_debug_flags(1)
     try:
         assert torch.equal(C.volume_render_image(dev._spec(), cam, opt), img)
     finally:
         C.set_debug_flags(0)
-    # through the renderer: forward on the octree kernel, gradient by the generic backward kernel
-    r = svox.VolumeRenderer(dev, step_size=1e-3, density_softplus=True, rgb_padding=0.001)
-    go = (torch.randn(3000, 3, generator=torch.Generator().manual_seed(2)) * 1e-2).to(gpu)
-    out = r(svox.Rays(rs.origins, rs.dirs, rs.vdirs), fast=True)
-    assert torch.equal(out.detach(), generic)
-    out.backward(go)
-    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go.cpu())
-    err, ok = grad_close(dev.data.grad.cpu().numpy(), want_g, rel=2e-4)   # (logf and its derivative from two libraries)
+
+
+# logf and expf of two libraries (the device's and the host's) meet in the softplus and in its derivative
+SOFTPLUS_GATE = 2e-4
+
+
+@pytest.mark.parametrize("fmt", ["SH9", "RGBA", "SH16"])
+def test_density_softplus_gradients_on_the_octree_kernels(gpu, oracle_mod, fmt):
+    """density_softplus in the backward pass and in se_grad (rt_kernel.cu:376, 440, 471-474, 518-710) on the octree
+    kernels: marching backward with and without a workspace, notes taken by either forward kernel and replayed,
+    autograd through the renderer, se_grad marching and from notes, ray batches handled as small and as large ones,
+    and an image -- against the oracle, and against the one-ray-per-lane kernels that served this option before."""
+    tree = synth.shell_tree(depth=6, n_spheres=5, data_format=fmt, seed=17, sigma_range=(0.5, 30.0))
+    with torch.no_grad():
+        tree.data[..., -1] -= 3.0
+    n = 3000
+    rays = synth.sphere_rays(n, seed=4)
+    opt = options(tree, step_size=1e-3, density_softplus=True, fast=True, rgb_padding=0.001)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    go = torch.randn(n, 3, generator=torch.Generator().manual_seed(2)) * 1e-2
+    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go, n_threads=8)
+    ref = torch.rand(n, 3, generator=torch.Generator().manual_seed(7))
+    want_se = oracle_mod.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, opt, n_threads=8)
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    spec = dev._spec()
+    assert C.octree_kernels_serve(spec, opt)
+    plain_out = C.volume_render(spec, rs, opt)
+
+    def close(got, want, what):
+        err, ok = grad_close(got.cpu().numpy(), want, rel=SOFTPLUS_GATE, what=what)
+        assert ok, (what, err)
+
+    for flags in (0, 2, 4, 8):
+        C.set_debug_flags(flags)
+        try:
+            if flags in (0, 2):
+                for workspace in (True, False):
+                    close(C.volume_render_backward(spec, rs, opt, go.to(gpu), workspace=workspace), want_g,
+                          f"softplus backward flags {flags} workspace {workspace}")
+                got = C.se_grad(spec, rs, ref.to(gpu), opt, workspace=False)
+                assert np.abs(got[0].cpu().numpy() - want_se[0]).max() <= 1e-5
+                close(got[1], want_se[1], f"softplus se_grad gradient flags {flags}")
+                close(got[2], want_se[2], f"softplus se_grad hessian flags {flags}")
+            out, notes = C.volume_render_noted(spec, rs, opt)
+            assert notes is not None and torch.equal(out, plain_out)
+            close(C.volume_render_backward_noted(spec, rs, opt, go.to(gpu), notes), want_g, f"softplus notes flags {flags}")
+            got = C.se_grad(spec, rs, ref.to(gpu), opt, workspace=True)
+            assert np.abs(got[0].cpu().numpy() - want_se[0]).max() <= 1e-5
+            close(got[1], want_se[1], f"softplus se_grad from notes, gradient, flags {flags}")
+            close(got[2], want_se[2], f"softplus se_grad from notes, hessian, flags {flags}")
+        finally:
+            C.set_debug_flags(0)
+    # the one-ray-per-lane kernels on the same device: the same softplus routine, so only the order of the sums differs
+    C.set_debug_flags(1)
+    try:
+        generic_g = C.volume_render_backward(spec, rs, opt, go.to(gpu))
+        generic_se = C.se_grad(spec, rs, ref.to(gpu), opt)
+    finally:
+        C.set_debug_flags(0)
+    err, ok = grad_close(C.volume_render_backward(spec, rs, opt, go.to(gpu)).cpu().numpy(), generic_g.cpu().numpy(),
+                         what="softplus backward, octree against generic kernels")
     assert ok, err
+    got = C.se_grad(spec, rs, ref.to(gpu), opt)
+    assert torch.equal(got[0], generic_se[0])
+    for a, b, what in zip(got[1:], generic_se[1:], ("gradient", "hessian")):
+        err, ok = grad_close(a.cpu().numpy(), b.cpu().numpy(), what=f"softplus se_grad {what}, octree against generic kernels")
+        assert ok, (what, err)
+    # through the renderer (notes kept between the passes), rays and an image
+    r = svox.VolumeRenderer(dev, step_size=1e-3, density_softplus=True, rgb_padding=0.001)
+    dev.data.grad = None
+    out = r(svox.Rays(rs.origins, rs.dirs, rs.vdirs), fast=True)
+    assert torch.equal(out.detach(), plain_out)
+    out.backward(go.to(gpu))
+    close(dev.data.grad, want_g, "softplus autograd")
+    c2w = synth.orbit_poses(1, seed=4, radius=2.5)[0]
+    igo = torch.randn(53, 75, 3, generator=torch.Generator().manual_seed(3)) * 1e-2
+    want_ig = oracle_mod.volume_render_image_backward(ot, c2w, 60.0, 60.0, 75, 53, opt, igo)
+    dev.data.grad = None
+    r.render_persp(c2w.to(gpu), width=75, height=53, fx=60.0, fast=True).backward(igo.to(gpu))
+    close(dev.data.grad, want_ig, "softplus autograd image")
+    iref = torch.rand(53, 75, 3, generator=torch.Generator().manual_seed(9))
+    want_ise = oracle_mod.se_grad_image(ot, c2w, 60.0, 60.0, 75, 53, iref, opt)
+    got = r.se_grad_persp(c2w.to(gpu), iref.to(gpu), width=75, height=53, fx=60.0)
+    assert np.abs(got[0].cpu().numpy() - want_ise[0]).max() <= 1e-5
+    close(got[1], want_ise[1], "softplus se_grad_persp gradient")
+    close(got[2], want_ise[2], "softplus se_grad_persp hessian")
+    dev.data.grad = None
 
 
-def test_gather_probe_runs_and_checks_its_arguments(gpu):
-    """The measurement aid reads and writes nothing a caller can see; bad arguments are refused."""
-    buf = torch.arange(1 << 18, dtype=torch.int32, device=gpu)
-    before = buf.clone()
-    assert C.gather_probe(buf, unit_bytes=64, iters=3, blocks=8) == 8 * 256 * 4 * 3
-    assert C.gather_probe(buf, unit_bytes=256, iters=1, blocks=1) == 1024
-    assert C.gather_probe(buf, unit_bytes=128, iters=2, blocks=2, lanes_per_unit=8) == 2 * 256 * 4 * 2 // 8
-    with pytest.raises(RuntimeError):
-        C.gather_probe(buf, unit_bytes=64, lanes_per_unit=8)        # 8 lanes x 16 bytes do not fit 64
-    torch.cuda.synchronize()
-    assert torch.equal(buf, before)
-    with pytest.raises(RuntimeError):
-        C.gather_probe(buf, unit_bytes=48)
-    with pytest.raises(RuntimeError):
-        C.gather_probe(buf[:8], unit_bytes=64)
+@pytest.mark.parametrize("fmt", ["RGBA", "SH4", "SH16", "SH25"])
+def test_gradient_gate_without_order_slack(gpu, oracle_mod, fmt):
+    """The plain gate -- 1e-4 relative to the oracle's exact sum, no allowance for the order of the additions -- on a
+    scene where few rays meet in a leaf (a 128^3 shell tree, 3 000 rays): every family of kernels that forms
+    gradients (marching backward, replay of notes taken by either forward kernel, se_grad marching and from notes,
+    for ray batches handled as small and as large ones and for an image)."""
+    tree = synth.shell_tree(depth=7, n_spheres=6, data_format=fmt, seed=23, sigma_range=(5.0, 120.0))
+    n = 3000
+    rays = synth.sphere_rays(n, seed=12)
+    opt = options(tree, step_size=1e-3, fast=True, background_brightness=0.5)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    go = torch.randn(n, 3, generator=torch.Generator().manual_seed(2)) * 1e-2
+    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go, n_threads=8)
+    ref = torch.rand(n, 3, generator=torch.Generator().manual_seed(7))
+    want_se = oracle_mod.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, opt, n_threads=8)
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    spec = dev._spec()
+
+    def close(got, want, what):
+        err, ok = grad_close(got.cpu().numpy(), want, what=what)
+        assert ok, (what, err)
+
+    for flags in (0, 2, 4, 8):
+        C.set_debug_flags(flags)
+        try:
+            if flags in (0, 2):
+                close(C.volume_render_backward(spec, rs, opt, go.to(gpu), workspace=False), want_g, f"marching, flags {flags}")
+                got = C.se_grad(spec, rs, ref.to(gpu), opt, workspace=False)
+                close(got[1], want_se[1], f"se_grad marching, gradient, flags {flags}")
+                close(got[2], want_se[2], f"se_grad marching, hessian, flags {flags}")
+            close(C.volume_render_backward(spec, rs, opt, go.to(gpu), workspace=True), want_g, f"noting march + replay, flags {flags}")
+            out, notes = C.volume_render_noted(spec, rs, opt)
+            close(C.volume_render_backward_noted(spec, rs, opt, go.to(gpu), notes), want_g, f"replay, flags {flags}")
+            got = C.se_grad(spec, rs, ref.to(gpu), opt, workspace=True)
+            close(got[1], want_se[1], f"se_grad replay, gradient, flags {flags}")
+            close(got[2], want_se[2], f"se_grad replay, hessian, flags {flags}")
+        finally:
+            C.set_debug_flags(0)
+    c2w = synth.orbit_poses(1, seed=4, radius=2.5)[0]
+    W, H, fx = 96, 80, 90.0
+    igo = torch.randn(H, W, 3, generator=torch.Generator().manual_seed(3)) * 1e-2
+    want_ig = oracle_mod.volume_render_image_backward(ot, c2w, fx, fx, W, H, opt, igo, n_threads=8)
+    cam = cam_spec(c2w, W, H, fx, device=gpu)
+    for workspace in (True, False):
+        close(C.volume_render_image_backward(spec, cam, opt, igo.to(gpu), workspace=workspace), want_ig,
+              f"image, workspace {workspace}")
+    out, notes = C.volume_render_images_noted(spec, cam, opt)
+    close(C.volume_render_images_backward_noted(spec, cam, opt, igo.to(gpu), notes), want_ig, "image replay")
+
+
+def test_notes_are_kept_only_where_they_are_taken(gpu):
+    """A renderer whose tree or options the noting kernels do not serve (N = 3, a negative sigma_thresh, a weight
+    accumulator) runs the plain forward pass: no workspace is allocated, the autograd context keeps nothing, and
+    the notes budget never looks at a counter nobody wrote."""
+    from svox_amd import renderer as R
+    rays = synth.sphere_rays(500, seed=1)
+    kept = []
+    orig = R._C.volume_render_noted
+
+    def spy(*a, **k):
+        out, notes = orig(*a, **k)
+        kept.append(notes)
+        return out, notes
+
+    R._C.volume_render_noted = spy
+    try:
+        cases = []
+        t3 = svox.N3Tree(N=3, data_format="SH4", init_refine=1, device=gpu)
+        t3.data.data.normal_()
+        t3.data.data[..., -1].abs_()
+        cases.append((svox.VolumeRenderer(t3, step_size=1e-2), False))
+        t2 = on_gpu(synth.dense_tree(3, "SH4", seed=0, sigma="lognormal"), gpu)
+        neg = svox.VolumeRenderer(t2, step_size=1e-2)
+        neg.sigma_thresh = -1.0
+        cases.append((neg, False))
+        cases.append((svox.VolumeRenderer(t2, step_size=1e-2, density_softplus=True), True))
+        cases.append((svox.VolumeRenderer(t2, step_size=1e-2), True))
+        for r, takes in cases:
+            kept.clear()
+            grays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu))
+            for _ in range(3):
+                r.tree.data.grad = None
+                r(grays).sum().backward()
+                torch.cuda.synchronize()
+            assert len(kept) == 3 and all((k is not None) == takes for k in kept), (takes, kept)
+            assert r.notes_budget.factor == 1
+            if not takes:
+                assert r.notes_budget._pending is None
+    finally:
+        R._C.volume_render_noted = orig
+
+
+def test_what_a_give_up_of_the_two_wavefront_kernel_leaves_behind(gpu, oracle_mod):
+    """The waits between the walking and the shading wavefront are bounded.  With the bound at one look (debug flag
+    16: the shading gives up as soon as it finds nothing new, the walk once its ring is full) every kernel still ends;
+    the pixels of the rays given up on are NaN, never a plausible colour; their notes say "march me", so the gradient
+    that follows is the right one; and the library's counter tells the host."""
+    tree = synth.shell_tree(depth=6, n_spheres=5, data_format="SH9", seed=3)
+    rays = synth.sphere_rays(4000, seed=6)
+    opt = options(tree, step_size=1e-3, fast=True)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    want = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    go = torch.randn(4000, 3, generator=torch.Generator().manual_seed(2)) * 1e-2
+    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    before = C.give_up_count()
+    C.set_debug_flags(8 | 16)
+    try:
+        out = C.volume_render(dev._spec(), rs, opt).cpu().numpy()
+        noted, notes = C.volume_render_noted(dev._spec(), rs, opt)
+    finally:
+        C.set_debug_flags(0)
+    gave_up = np.isnan(out).any(axis=1)
+    assert gave_up.any() and C.give_up_count() > before
+    assert np.array_equal(out[~gave_up], want[~gave_up])           # the others are untouched
+    noted = noted.cpu().numpy()
+    bad = np.isnan(noted).any(axis=1)
+    assert np.array_equal(noted[~bad], want[~bad])
+    g = C.volume_render_backward_noted(dev._spec(), rs, opt, go.to(gpu), notes)
+    err, ok = grad_close(g.cpu().numpy(), want_g, what="gradient after a give-up")
+    assert ok, err
+    # the stateless backward operator takes its notes with grad_out at hand (the sum of the first march rides along)
+    C.set_debug_flags(8 | 16)
+    try:
+        g = C.volume_render_backward(dev._spec(), rs, opt, go.to(gpu))
+    finally:
+        C.set_debug_flags(0)
+    err, ok = grad_close(g.cpu().numpy(), want_g, what="stateless gradient after a give-up")
+    assert ok, err
+    # and a healthy run gives up nowhere
+    now = C.give_up_count()
+    C.set_debug_flags(8)
+    try:
+        assert np.array_equal(C.volume_render(dev._spec(), rs, opt).cpu().numpy(), want)
+    finally:
+        C.set_debug_flags(0)
+    assert C.give_up_count() == now
 
 
 def test_a_training_step_replays_from_a_hip_graph(gpu):
@@ -946,17 +1156,3 @@ def test_a_training_step_replays_from_a_hip_graph(gpu):
         err, ok = grad_close(tree.data.detach().cpu().numpy(), eager_data[i].cpu().numpy(), rel=1e-5)
         assert ok, (i, err)
         assert float((torch.rand(1000, device=gpu) * 2).sum()) > 0          # eager work between the replays
-
-
-def test_atomic_probe_adds_what_it_says(gpu):
-    """The measurement aid for atomics: every add is 1.0f, so the scratch sums to the number of adds."""
-    scratch = torch.zeros(1 << 16, dtype=torch.float32, device=gpu)
-    adds, requests = C.atomic_probe(scratch, run_floats=16, iters=5, blocks=3)
-    assert adds == 3 * 256 * 5 and requests == adds // 16
-    assert float(scratch.double().sum()) == adds
-    adds, requests = C.atomic_probe(scratch, run_floats=1, iters=2, blocks=2)
-    assert requests == adds
-    with pytest.raises(RuntimeError):
-        C.atomic_probe(scratch, run_floats=3)
-    with pytest.raises(RuntimeError):
-        C.atomic_probe(scratch[1:17], run_floats=16)       # not 64-byte aligned

@@ -49,7 +49,17 @@ def rel_err(a, b):
 ORDER_SLACK_FACTOR = 2.0
 
 
-def grad_close(got, ref, rel=1e-4, slack=None):
+# Worst error of every grad_close call of the session, by label: tests/conftest.py prints them after the run, so that
+# the log shows how close to the gate the kernels run and not only that they passed.
+GATE_LOG = []
+
+
+def _caller_label():
+    test = os.environ.get("PYTEST_CURRENT_TEST", "")
+    return test.split(" ")[0].split("::", 1)[-1] if test else "?"
+
+
+def grad_close(got, ref, rel=1e-4, slack=None, what=None):
     """Element-wise gradient comparison against the oracle's exact sum: every element must be within
     `rel` of the reference, relative to the reference's own magnitude or, for elements below it, to a
     floor of 1e-3 of the largest gradient.
@@ -67,9 +77,11 @@ def grad_close(got, ref, rel=1e-4, slack=None):
     if slack is not None:
         diff = np.maximum(diff - ORDER_SLACK_FACTOR * np.asarray(slack, dtype=np.float64), 0.0)
     err = diff / np.maximum(np.abs(ref), floor if floor > 0 else 1.0)
+    worst = float(err.max()) if err.size else 0.0
+    GATE_LOG.append((_caller_label() + (f" [{what}]" if what else ""), worst, rel, slack is not None))
     if os.environ.get("SVOX_TEST_VERBOSE"):
-        print(f"[grad_close] worst relative error {float(err.max()):.3e} (limit {rel:.0e})", flush=True)
-    return float(err.max()), err.max() <= rel
+        print(f"[grad_close] worst relative error {worst:.3e} (limit {rel:.0e})", flush=True)
+    return worst, worst <= rel
 
 
 def on_gpu(tree, device):
