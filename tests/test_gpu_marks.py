@@ -207,18 +207,27 @@ def test_large_multi_pose_launch_marks_the_leaves_for_itself(gpu, monkeypatch):
     monkeypatch.setattr(C, "AUTO_MARK_MIN_RAYS", 3 * 160 * 120)   # (the floor on the number of rays: just met)
     made = []
     real = C.mark_empty_leaves
-    monkeypatch.setattr(C, "mark_empty_leaves", lambda t: made.append(1) or real(t))
+    monkeypatch.setattr(C, "mark_empty_leaves", lambda t, *how: made.append(how) or real(t, *how))
     with_marks = C.volume_render_images(tree._spec(), cam, opt)
-    assert made == [1]
+    assert made == [(opt.sigma_thresh, False)]          # made with the call's own threshold: they decide the shading
     monkeypatch.setattr(C, "AUTO_MARK_RAYS_PER_CELL", None)
     without = C.volume_render_images(tree._spec(), cam, opt)
-    assert made == [1] and torch.equal(with_marks, without)
+    assert len(made) == 1 and torch.equal(with_marks, without)
     monkeypatch.setattr(C, "AUTO_MARK_RAYS_PER_CELL", 0.7)
     small = cam_spec(torch.stack(synth.orbit_poses(2, seed=4, radius=2.5)).to(gpu), 16, 12, 13.0)
     C.volume_render_images(tree._spec(), small, opt)                          # too few rays to pay
     C.volume_render_images(tree._spec(), cam, options(tree, step_size=1e-3, sigma_thresh=-1.0))
     C.volume_render_images(tree._spec(), cam, options(tree, step_size=1e-3, density_softplus=True))
-    assert made == [1]
+    assert len(made) == 1
+    # a call that takes notes works on every leaf with density: its marks are made with threshold 0
+    out, notes = C.volume_render_images_noted(tree._spec(), cam, opt)
+    assert notes is not None and made[1:] == [(0.0, False)] and torch.equal(out, with_marks)
+    # with the softplus, a threshold above 0 marks leaves too
+    soft = options(tree, step_size=1e-3, density_softplus=True, fast=True)
+    a = C.volume_render_images(tree._spec(), cam, soft)
+    assert made[2:] == [(soft.sigma_thresh, True)]
+    monkeypatch.setattr(C, "AUTO_MARK_RAYS_PER_CELL", None)
+    assert torch.equal(C.volume_render_images(tree._spec(), cam, soft), a)
 
 
 @pytest.mark.parametrize("softplus", [False, True])

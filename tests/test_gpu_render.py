@@ -841,7 +841,9 @@ def test_density_softplus_on_the_octree_forward_kernel(gpu, oracle_mod, fmt):
     softplus of any stored density is > 0), marks made with it and the render's threshold decide the shading."""
     tree = synth.shell_tree(depth=6, n_spheres=5, data_format=fmt, seed=17, sigma_range=(0.5, 30.0))
     with torch.no_grad():
-        tree.data[..., -1] -= 3.0                 # stored densities of both signs
+        sigma = tree.data[..., -1]
+        sigma -= 3.0                              # stored densities of both signs
+        sigma[sigma == -3.0] = -8.0               # (the softplus of the empty leaves lies below the fast threshold)
     rays = synth.sphere_rays(3000, seed=4)
     opt = options(tree, step_size=1e-3, density_softplus=True, fast=True, rgb_padding=0.001)
     ot = oracle_mod.Tree.from_n3tree(tree)
@@ -882,8 +884,8 @@ def test_density_softplus_on_the_octree_forward_kernel(gpu, oracle_mod, fmt):
         C.set_debug_flags(0)
 
 
-# logf and expf of two libraries (the device's and the host's) meet in the softplus and in its derivative
-SOFTPLUS_GATE = 2e-4
+# (logf of two libraries, the device's and the host's, meet in the softplus: measured 2e-5 to 5e-5)
+SOFTPLUS_GATE = 1e-4
 
 
 @pytest.mark.parametrize("fmt", ["SH9", "RGBA", "SH16"])
