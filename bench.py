@@ -307,6 +307,8 @@ def main():
         "rays_hit": int(sum(s["rays_hit"] for s in pose_stats)),
         "samples": int(sum(s["samples"] for s in pose_stats)),
         "samples_shaded": int(sum(s["samples_shaded"] for s in pose_stats)),
+        # visits after the last shaded leaf of their ray (all visits of a ray that shades nothing)
+        "samples_tail": int(sum(s["samples_tail"] for s in pose_stats)),
         "samples_per_ray": round(sum(s["samples"] for s in pose_stats) / n_rays_step, 2),
         "shaded_per_ray": round(sum(s["samples_shaded"] for s in pose_stats) / n_rays_step, 2),
         "msamples_s": round(sum(s["samples"] for s in pose_stats) / (durs.mean() * 1e3), 1),

@@ -1580,20 +1580,19 @@ __device__ __forceinline__ void box_write(int32_t* at, int32_t value) {
 // Wavefronts of render_forward_split_kernel that gave up waiting since the library was loaded (svox_give_up_count).
 __device__ unsigned int split_give_ups = 0;
 
-// kAllShaded: as in render_forward_kernel -- the marks were made with this launch's sigma_thresh, every leaf the
-// walk hands over is shaded, and its density is read with its coefficients.
-template <class P, class Source, bool kNoted = false, bool kGrad = false, bool kAllShaded = false>
+// (The density phase stays also where the marks of a launch say that every leaf they let through is shaded,
+// render_forward_kernel's kAllShaded: here the walk is the critical path, and the density read of a leaf brings the
+// last line of its record into L2 ahead of the coefficient reads.)
+template <class P, class Source, bool kNoted = false, bool kGrad = false>
 __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(TreeDev<float> tr, Source src,
                                                                              SvoxRenderOptions opt,
                                                                              float* __restrict__ out, ReplaySpace ws,
                                                                              const float* __restrict__ grad_out = nullptr) {
-    static_assert(!kAllShaded || !kNoted, "notes look at leaves the marks may hide");
     constexpr int D = P::kBasis > 0 ? P::kBasis : 1;
     constexpr int K = P::kRecord;
     __shared__ int32_t path[(kPathLevels + 1) * kMarchThreads];
     __shared__ ShadeShared<D, P::kForwardRows> sh;
     __shared__ SplitBox box;
-    __shared__ float sh_sigma[kAllShaded ? kQueue * kMarchThreads : 1];
     if constexpr (kNoted) {
         if (blockIdx.x == 0 && threadIdx.x < kStampWords) ws.stamp_at[threadIdx.x] = ws.stamp[threadIdx.x];
     }
@@ -1752,26 +1751,14 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
         taken += n_take;
         if (n_take > 0) box_write(&box.taken[lane], taken);
         float q_sigma[kQueue], q_raw[kQueue];
-        int n_entries;
-        if constexpr (kAllShaded) {
-            n_entries = build_shade_list_all(sh, q_leaf, lane);
-        } else {
-            fetch_sigma<K>(tr.data, q_leaf, q_sigma);
-            soften_sigma(opt.density_softplus, q_leaf, q_sigma, q_raw);
-            n_entries = build_shade_list(sh, q_leaf, q_sigma, kNoted ? 0.0f : sigma_thresh, lane);
-        }
+        fetch_sigma<K>(tr.data, q_leaf, q_sigma);
+        soften_sigma(opt.density_softplus, q_leaf, q_sigma, q_raw);
+        const int n_entries = build_shade_list(sh, q_leaf, q_sigma, kNoted ? 0.0f : sigma_thresh, lane);
         bool stopped = false;
         if (n_entries > 0) {
             wave_lds_sync();
-            shade_entries<P, P::kForwardRows, kAllShaded>(tr.data, sh, n_entries, lane, sh_sigma);
+            shade_entries<P, P::kForwardRows>(tr.data, sh, n_entries, lane);
             wave_lds_sync();
-            if constexpr (kAllShaded) {
-#pragma unroll
-                for (int q = 0; q < kQueue; ++q) {
-                    const float raw = sh_sigma[q * kMarchThreads + lane];
-                    q_sigma[q] = q_leaf[q] >= 0 ? (opt.density_softplus ? softplus_m1(raw) : raw) : 0.0f;
-                }
-            }
             float q_att[kQueue], q_rgb[kQueue][3], q_s[kQueue][3];
 #pragma unroll
             for (int q = 0; q < kQueue; ++q) {

@@ -408,7 +408,13 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
             const Source dealt = dealt_out(src, blocks);
             const TreeDev<float> tr = march_tree(tree, opt, opt->sigma_thresh);
             const ReplaySpace none = no_notes();
-            // marks made with this launch's own threshold: every leaf they let through is shaded
+            // Marks made with this launch's own threshold: every leaf they let through is shaded, and the kernel with
+            // one wavefront per tile or chunk then reads a leaf's density with its coefficients (one round trip per
+            // round instead of two that wait for one another: 4 NDC poses 3.10 -> 2.93 ms).  The two-wavefront kernel
+            // keeps its density phase: there the walk is the critical path, the density read of a leaf brings the
+            // last line of its record into L2 ahead of the coefficient reads, and without it the kernel needs more
+            // registers (5 instead of 6 wavefronts per SIMD): measured 0.70 -> 0.73 ms on 8 poses of 800x800,
+            // although the launch sends 17 % fewer requests to L2.
             const bool all_shaded = !tree->weight_accum && marks_decide(tree, opt, opt->sigma_thresh);
 #define SVOX_LAUNCH_FORWARD(ACCUM, REFILL, ALL)                                                                   \
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_kernel<P, Source, ACCUM, REFILL, false, false, ALL>), \
@@ -416,15 +422,9 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
                                                (float*)out, none))
             const bool refill = src.per_wave > kMarchThreads;
             if (!refill && !tree->weight_accum && use_split_forward(blocks, is_image_source(src), opt)) {
-                if (all_shaded) {
-                    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false, false, true>),
-                                                               dim3(blocks), dim3(kSplitThreads), 0, stream, tr, dealt,
-                                                               *opt, (float*)out, none));
-                } else {
-                    SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false>),
-                                                               dim3(blocks), dim3(kSplitThreads), 0, stream, tr, dealt,
-                                                               *opt, (float*)out, none));
-                }
+                SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false>),
+                                                           dim3(blocks), dim3(kSplitThreads), 0, stream, tr, dealt,
+                                                           *opt, (float*)out, none));
                 return;
             }
             if (tree->weight_accum) {

@@ -43,5 +43,5 @@ def pytest_terminal_summary(terminalreporter):
         worst[key] = max(worst.get(key, 0.0), err)
     tr = terminalreporter
     tr.write_sep("-", "gradient gate: worst relative error per test (limit; * = order slack of the oracle taken off)")
-    for (label, limit, slack), err in sorted(worst.items(), key=lambda kv: -kv[1] / kv[0][1])[:60]:
+    for (label, limit, slack), err in sorted(worst.items(), key=lambda kv: -kv[1] / kv[0][1])[:30]:
         tr.write_line(f"  {err:9.3e} of {limit:.0e}{'*' if slack else ' '} {label}")
