@@ -59,6 +59,21 @@ __device__ __forceinline__ void dda_unit(const T* cen, const T* invdir, T* tmin,
     *tmax = hi;
 }
 
+// _dda_unit for a point inside the unit cube -- the leaf-local position of a sample, every coordinate in [0, 1) --
+// as the octree walk uses it: the length tmax - tmin of the segment.  There the entry distance is 0 (on every axis
+// t1 = -c * inv and t2 = t1 + inv lie on either side of 0, so min(t1, t2) <= 0), and the larger of t1 and t2 is t2
+// where inv > 0 and t1 elsewhere, i.e. t1 + max(inv, 0): the same roundings and the same value as dda_unit gives
+// (an axis whose inv is NaN drops out of both), in half the instructions of the walk's innermost turn.
+__device__ __forceinline__ float leaf_exit(const float* cen, const float* invdir) {
+    float hi = 1e9f;
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        const float t1 = -cen[i] * invdir[i];
+        hi = min_(hi, t1 + max_(invdir[i], 0.0f));
+    }
+    return hi;
+}
+
 // cam2world_ray, rt_kernel.cu:758-772: pixel corner (no half-pixel offset), camera looking down
 // -z with +y up.  x and y are formed in double and rounded; the radicand is widened for `+ 1.0`.
 template <typename T>
@@ -355,9 +370,7 @@ __device__ __forceinline__ void walk_turn_flat(const TreeDev<float>& tr, RayStat
             broken = broken || leaf < 0;
         }
     }
-    float s0, s1;
-    dda_unit(local, r.inv, &s0, &s1);
-    const float delta_t = (s1 - s0) * inv_cube + step_size;
+    const float delta_t = leaf_exit(local, r.inv) * inv_cube + step_size;
     const bool ok = leaf >= 0;
     slot_leaf = ok ? leaf : -1;
     slot_dt = ok ? delta_t : 0.0f;

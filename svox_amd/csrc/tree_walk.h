@@ -185,10 +185,10 @@ __device__ __forceinline__ void descend_octree_multi(const int32_t* __restrict__
     }
 }
 
-// leaf-local position frac(pc * 2^levels) and the reciprocal cell count 2^-levels
+// leaf-local position frac(pc * 2^levels): s - floor(s), exact for the non-negative s of a clamped coordinate, in
+// one instruction
 __device__ __forceinline__ float leaf_local(float pc, float cube_sz) {
-    const float s = pc * cube_sz;
-    return s - floor_(s);
+    return __builtin_amdgcn_fractf(pc * cube_sz);
 }
 
 // Per-lane cursor that remembers the previous descent.  `path` points at this lane's column of an
