@@ -691,9 +691,10 @@ def main():
                     ev_time(lambda: C.volume_render_image(sgtree._spec(), gcam, sg_opt)), 4)
             finally:
                 C.set_debug_flags(0)
-        generic["note"] = ("fp32 SH, SG and ASG records of 1, 4, 9, 16 or 25 basis functions run on the octree kernels "
+        generic["note"] = ("fp32 SH, SG and ASG records of 1, 4, 9, 16 or 25 basis functions run on the wavefront-per-tile kernels, "
+                           "for any branching factor and with or without density_softplus "
                            "(`..._generic_kernel_ms`: the same call forced onto the one-ray-per-lane kernels, which "
-                           "serve fp64 and the other shapes)")
+                           "serve fp64, partial component ranges and the other record shapes)")
         del sgtree
         gtree64 = gtree.double()
         g64cam = _make_camera_spec(poses[0].double().contiguous(), W, H, fx, fx)
@@ -702,6 +703,27 @@ def main():
             opt64 = svox.VolumeRenderer(gtree64)._get_options(False)
             generic["fp64_sh9_ms"] = round(ev_time(lambda: C.volume_render_image(gtree64._spec(), g64cam, opt64)), 4)
             generic["fp64_query_4M_ms"] = round(ev_time(lambda: C.query_vertical(gtree64._spec(), pts64)), 4)
+        # a tree with branching factor 3 (81^3 leaves, SH9 records): the wavefront-per-tile kernels with the reference's
+        # floating-point walk, against the same calls forced onto the one-ray-per-lane kernels
+        t3 = svox.N3Tree(N=3, data_format="SH9", init_refine=3, device=dev)
+        g3 = torch.Generator().manual_seed(9)
+        t3.data.data.copy_((torch.randn(t3.data.shape, generator=g3) * 0.5).to(dev))
+        t3.data.data[..., -1] = (torch.exp(torch.randn(t3.child.shape, generator=g3))
+                                 * (torch.rand(t3.child.shape, generator=g3) < 0.5)).to(dev)
+        o3 = svox.VolumeRenderer(t3)._get_options(False)
+        go3 = (torch.randn(H, W, 3, generator=g3) * 1e-2).to(dev)
+        with torch.no_grad():
+            generic["fp32_n3_sh9_ms"] = round(ev_time(lambda: C.volume_render_image(t3._spec(), gcam, o3)), 4)
+        generic["fp32_n3_sh9_backward_ms"] = round(ev_time(lambda: C.volume_render_image_backward(t3._spec(), gcam, o3, go3)), 4)
+        C.set_debug_flags(1)
+        try:
+            with torch.no_grad():
+                generic["fp32_n3_sh9_generic_kernel_ms"] = round(ev_time(lambda: C.volume_render_image(t3._spec(), gcam, o3)), 4)
+            generic["fp32_n3_sh9_backward_generic_kernel_ms"] = round(
+                ev_time(lambda: C.volume_render_image_backward(t3._spec(), gcam, o3, go3)), 4)
+        finally:
+            C.set_debug_flags(0)
+        del t3, go3
         generic["mrays_s"] = {k[:-3]: round(W * H / v / 1e3, 1) for k, v in generic.items() if k.endswith("_ms") and "query" not in k}
         del gtree, gtree64, pts64
         torch.cuda.empty_cache()

@@ -349,28 +349,35 @@ __device__ __forceinline__ void walk_turn_flat(const TreeDev<float>& tr, RayStat
     float pc[3];
 #pragma unroll
     for (int j = 0; j < 3; ++j) pc[j] = clamp01(fma_(r.t, r.d[j], r.o[j]));
-    int32_t leaf = cur.seek_flat<kSeekBudget>(go, tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]),
-                                              cell_coord(pc[1]), cell_coord(pc[2]));
+    // (trees with another branching factor have no exact integer formulation: every lane takes the reference's
+    // floating-point walk below, from the root for every sample, and shares everything else with the octrees)
+    const bool octree = tr.N == 2;
+    int32_t leaf = go ? -1 : OctreeCursor::kIdle;
+    if (octree)
+        leaf = cur.seek_flat<kSeekBudget>(go, tr.child, (int32_t)(tr.capacity - 1), cell_coord(pc[0]), cell_coord(pc[1]),
+                                          cell_coord(pc[2]));
     // 2^levels and 2^-levels: dividing by the power of two is the multiplication by its reciprocal
     const float cube = __uint_as_float((uint32_t)(127 + cur.levels) << 23);
     float inv_cube = __uint_as_float((uint32_t)(127 - cur.levels) << 23);
+    float cells_per_axis = 1.0f;   // N^levels where it is no power of two
     float local[3];
 #pragma unroll
     for (int j = 0; j < 3; ++j) local[j] = leaf_local(pc[j], cube);
     const bool deep = leaf == -1;
     if (__any(deep)) {
         if (deep) {
-            // more levels than the integer coordinates hold (or a broken tree): floating-point walk
-            float cube_f;
+            // more levels than the integer coordinates hold, another branching factor, or a broken tree
             int levels_f;
 #pragma unroll
             for (int j = 0; j < 3; ++j) local[j] = pc[j];
-            leaf = (int32_t)descend_generic<float>(tr.child, tr.capacity, 2, local, &cube_f, &levels_f, true);
-            inv_cube = 1.0f / cube_f;
+            leaf = (int32_t)descend_generic<float>(tr.child, tr.capacity, tr.N, local, &cells_per_axis, &levels_f, true);
+            inv_cube = 1.0f / cells_per_axis;
             broken = broken || leaf < 0;
         }
     }
-    const float delta_t = leaf_exit(local, r.inv) * inv_cube + step_size;
+    const float segment = leaf_exit(local, r.inv);
+    // (rt_kernel.cu:274 divides by the cell count; for a power of two the product with the reciprocal is the same number)
+    const float delta_t = (octree ? segment * inv_cube : segment / cells_per_axis) + step_size;
     const bool ok = leaf >= 0;
     slot_leaf = ok ? leaf : -1;
     slot_dt = ok ? delta_t : 0.0f;

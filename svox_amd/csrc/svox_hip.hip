@@ -116,10 +116,15 @@ TreeDev<T> make_tree(const SvoxTreeSpec* t) {
     return d;
 }
 
-// an fp32 octree whose child table is smaller than 4 GiB (32-bit byte offsets, int32 cell indices)
-bool octree_fast_ok(const SvoxTreeSpec* t) {
-    return !(g_debug_flags & 1) && t->dtype == SVOX_F32 && t->N == 2 && t->capacity < (1ll << 27);
+// an fp32 tree whose cells number less than 2^30 (int32 cell indices with two spare bits; for an octree that is
+// fewer than 2^27 nodes and a child table below 4 GiB, which its walk addresses with 32-bit byte offsets).  Octrees
+// walk on integer coordinates from the previous path; other branching factors take the reference's floating-point
+// walk inside the same kernels and share the rounds, the shade list, the record lists and the notes.
+bool march_fast_ok(const SvoxTreeSpec* t) {
+    return !(g_debug_flags & 1) && t->dtype == SVOX_F32 && (double)t->capacity * t->N * t->N * t->N < 1073741824.0;
 }
+// ... and an octree among them: the point queries' integer walk
+bool octree_fast_ok(const SvoxTreeSpec* t) { return march_fast_ok(t) && t->N == 2; }
 
 int zero_fill(void* ptr, int64_t bytes, hipStream_t stream) {
     if (bytes <= 0) return SVOX_OK;
@@ -219,7 +224,7 @@ int check_rays(const SvoxRaysSpec* rays) {
 // gaussians and anisotropic ones), -1 for everything the generic kernels serve.
 constexpr int kLobeKernels = 100;
 int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
-    if (!octree_fast_ok(tree)) return -1;
+    if (!march_fast_ok(tree)) return -1;
     if (opt->format == SVOX_FORMAT_RGBA) return tree->data_dim == 4 ? 0 : -1;
     if (opt->format != SVOX_FORMAT_SH && opt->format != SVOX_FORMAT_SG && opt->format != SVOX_FORMAT_ASG) return -1;
     const int D = opt->basis_dim;

@@ -100,7 +100,8 @@ def test_which_kernels_serve_which_trees(gpu):
     assert not serve(lobe_tree(5, seed=2, depth=4))                       # no kernel built for five lobes
     assert serve(lobe_tree(4, seed=2, depth=4, kind="ASG"))
     assert not serve(lobe_tree(6, seed=2, depth=4, kind="ASG"))
-    assert not serve(svox.N3Tree(N=3, data_format="SH4", init_refine=1))
+    assert serve(svox.N3Tree(N=3, data_format="SH4", init_refine=1))          # other branching factors: same kernels, float walk
+    assert not serve(svox.N3Tree(N=3, data_format="SH4", init_refine=1, dtype=torch.float64))
 
 
 @pytest.mark.parametrize("op", ["sum", "max"])

@@ -176,6 +176,95 @@ def test_generic_options_double_and_lobes(gpu, oracle_mod):
         assert ok, (name, err)
 
 
+def irregular_tree(N, fmt, seed, rounds=3):
+    """A tree of branching factor N refined at random (a few thousand leaves of several sizes), about half of them
+    with density."""
+    g = torch.Generator().manual_seed(seed)
+    tree = svox.N3Tree(N=N, data_format=fmt, init_refine=1, depth_limit=6)
+    for _ in range(rounds):
+        leaves = tree._all_leaves()
+        keep = min(0.5, 40.0 / leaves.shape[0] * (1 + _))          # (a round adds some 40 to 120 nodes of N^3 cells)
+        pick = torch.rand(leaves.shape[0], generator=g) < keep
+        if pick.any():
+            tree.refine(sel=tuple(leaves[pick].T))
+    tree.data.data.normal_(0, 0.5, generator=g)
+    sigma = tree.data.data[..., -1]
+    sigma.copy_(torch.exp(torch.randn(sigma.shape, generator=g)) * 8 * (torch.rand(sigma.shape, generator=g) < 0.5))
+    return tree
+
+
+@pytest.mark.parametrize("N,fmt", [(3, "SH4"), (3, "RGBA"), (4, "SH9"), (5, "SH1")])
+def test_other_branching_factors_on_the_wavefront_kernels(gpu, oracle_mod, N, fmt):
+    """fp32 trees with N != 2 (common.cuh:52-90 with N as a scalar; AT_DISPATCH over the same kernels, rt_kernel.cu:1029)
+    run on the wavefront-per-tile kernels: the walk is the reference's floating-point walk from the root (no integer
+    formulation is exact there), everything else -- rounds, shade list, record lists, notes, replays -- is shared with
+    the octrees.  Forward pictures equal the oracle's bit for bit on every forward kernel; gradients, se_grad and the
+    image paths meet the plain gate."""
+    tree = irregular_tree(N, fmt, seed=40 + N)
+    assert tree.n_leaves > 300
+    n = 2500
+    rays = synth.sphere_rays(n, seed=N)
+    opt = options(tree, step_size=2e-3, fast=True, background_brightness=0.25)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    want, want_stats = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt, want_stats=True)
+    go = torch.randn(n, 3, generator=torch.Generator().manual_seed(2)) * 1e-2
+    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go, n_threads=8)
+    ref = torch.rand(n, 3, generator=torch.Generator().manual_seed(7))
+    want_se = oracle_mod.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, opt, n_threads=8)
+    dev = on_gpu(tree, gpu)
+    rs = rays_spec(rays, gpu)
+    spec = dev._spec()
+    assert C.octree_kernels_serve(spec, opt)
+    marked = dev._spec()
+    marked.child_marks = C.mark_empty_leaves(spec)
+    stats = C.volume_render_stats(spec, rs, opt)
+    for k in ("rays", "rays_hit", "samples", "samples_shaded", "levels", "samples_tail"):
+        assert stats[k] == want_stats[k], k
+    assert stats["samples_shaded"] > 1000
+
+    def close(got, ref_, what):
+        err, ok = grad_close(got.cpu().numpy(), ref_, what=what)
+        assert ok, (what, err)
+
+    for flags in (0, 2, 4, 8):
+        C.set_debug_flags(flags)
+        try:
+            for sp in (spec, marked):
+                assert np.array_equal(C.volume_render(sp, rs, opt).cpu().numpy(), want), flags
+            out, notes = C.volume_render_noted(spec, rs, opt)
+            assert notes is not None and np.array_equal(out.cpu().numpy(), want)
+            close(C.volume_render_backward_noted(spec, rs, opt, go.to(gpu), notes), want_g, f"N={N} replay flags {flags}")
+            if flags in (0, 2):
+                for workspace in (True, False):
+                    close(C.volume_render_backward(spec, rs, opt, go.to(gpu), workspace=workspace), want_g,
+                          f"N={N} backward flags {flags} workspace {workspace}")
+                    got = C.se_grad(spec, rs, ref.to(gpu), opt, workspace=workspace)
+                    assert np.array_equal(got[0].cpu().numpy(), want_se[0])
+                    close(got[1], want_se[1], f"N={N} se_grad gradient flags {flags} workspace {workspace}")
+                    close(got[2], want_se[2], f"N={N} se_grad hessian flags {flags} workspace {workspace}")
+        finally:
+            C.set_debug_flags(0)
+    # the one-ray-per-lane kernels agree bit for bit on the picture
+    C.set_debug_flags(1)
+    try:
+        assert np.array_equal(C.volume_render(spec, rs, opt).cpu().numpy(), want)
+    finally:
+        C.set_debug_flags(0)
+    # images, through the renderer
+    c2w = synth.orbit_poses(2, seed=4, radius=2.5)
+    W, H, fx = 90, 70, 80.0
+    want_img = np.stack([oracle_mod.volume_render_image(ot, p, fx, fx, W, H, opt) for p in c2w])
+    r = svox.VolumeRenderer(dev, step_size=2e-3, background_brightness=0.25)
+    with torch.no_grad():
+        assert np.array_equal(r.render_persp(torch.stack(c2w).to(gpu), width=W, height=H, fx=fx, fast=True).cpu().numpy(), want_img)
+    igo = torch.randn(H, W, 3, generator=torch.Generator().manual_seed(3)) * 1e-2
+    want_ig = oracle_mod.volume_render_image_backward(ot, c2w[0], fx, fx, W, H, opt, igo)
+    dev.data.grad = None
+    r.render_persp(c2w[0].to(gpu), width=W, height=H, fx=fx, fast=True).backward(igo.to(gpu))
+    close(dev.data.grad, want_ig, f"N={N} image autograd")
+    dev.data.grad = None
+
+
 @pytest.mark.parametrize("generic", [0, 1])
 def test_weight_accumulation(gpu, oracle_mod, generic):
     """accumulate_weights (sum / max) through the renderer, batch and image, thresholds and early stop
@@ -1024,8 +1113,8 @@ def test_gradient_gate_without_order_slack(gpu, oracle_mod, fmt):
 
 
 def test_notes_are_kept_only_where_they_are_taken(gpu):
-    """A renderer whose tree or options the noting kernels do not serve (N = 3, a negative sigma_thresh, a weight
-    accumulator) runs the plain forward pass: no workspace is allocated, the autograd context keeps nothing, and
+    """A renderer whose tree or options the noting kernels do not serve (fp64 records, a partial component range, a
+    negative sigma_thresh) runs the plain forward pass: no workspace is allocated, the autograd context keeps nothing, and
     the notes budget never looks at a counter nobody wrote."""
     from svox_amd import renderer as R
     rays = synth.sphere_rays(500, seed=1)
@@ -1043,7 +1132,10 @@ def test_notes_are_kept_only_where_they_are_taken(gpu):
         t3 = svox.N3Tree(N=3, data_format="SH4", init_refine=1, device=gpu)
         t3.data.data.normal_()
         t3.data.data[..., -1].abs_()
-        cases.append((svox.VolumeRenderer(t3, step_size=1e-2), False))
+        cases.append((svox.VolumeRenderer(t3, step_size=1e-2), True))         # (N = 3 runs on the same kernels)
+        cases.append((svox.VolumeRenderer(t3, step_size=1e-2, max_comp=2), False))
+        t64 = on_gpu(synth.dense_tree(2, "SH4", seed=1, sigma="lognormal", dtype=torch.float64), gpu)
+        cases.append((svox.VolumeRenderer(t64, step_size=1e-2), False))
         t2 = on_gpu(synth.dense_tree(3, "SH4", seed=0, sigma="lognormal"), gpu)
         neg = svox.VolumeRenderer(t2, step_size=1e-2)
         neg.sigma_thresh = -1.0
@@ -1052,7 +1144,8 @@ def test_notes_are_kept_only_where_they_are_taken(gpu):
         cases.append((svox.VolumeRenderer(t2, step_size=1e-2), True))
         for r, takes in cases:
             kept.clear()
-            grays = svox.Rays(rays.origins.to(gpu), rays.dirs.to(gpu), rays.viewdirs.to(gpu))
+            dt = r.tree.data.dtype
+            grays = svox.Rays(rays.origins.to(gpu, dt), rays.dirs.to(gpu, dt), rays.viewdirs.to(gpu, dt))
             for _ in range(3):
                 r.tree.data.grad = None
                 r(grays).sum().backward()
