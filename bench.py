@@ -281,8 +281,14 @@ def main():
             traffic_source = (f"none: {prof_rel} was taken on other kernel sources (its stamp "
                               f"{m.group(1) if m else 'missing'}, these sources {stamp}); counters are not mixed with this run")
 
+    # which forward kernel the launcher picks for this launch (its rule goes by tiles of 64 pixels: up to 49 152
+    # where the marks decide the shading the two-wavefront kernel, beyond that the one-wavefront kernel that
+    # builds its shade list from the marks alone)
+    tiles = args.poses * ((W * H + 63) // 64)
+    dominant = ("render_forward_split_kernel<OctreePolicy<SH,16>, ImageSource>" if tiles <= 49152 else
+                "render_forward_kernel<OctreePolicy<SH,16>, ImageSource, all-shaded>")
     roofline = {
-        "bound": "hbm", "kernel": "render_forward_split_kernel<OctreePolicy<SH,16>, ImageSource>",
+        "bound": "hbm", "kernel": dominant,
         "launch": f"{args.poses} poses x {W}x{H} in one launch",
         "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
         "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": traffic, "traffic_source": traffic_source,

@@ -379,23 +379,29 @@ unsigned blocks_for(int64_t items, int per_block) { return (unsigned)((items + p
         default: { using P = OctreePolicy<SVOX_FORMAT_SG, 25>; __VA_ARGS__; } break; \
     }
 
-// Whether a forward launch of `blocks` 64-ray wavefronts takes render_forward_split_kernel (two
-// wavefronts per 64 rays: one walks, one shades).  It shortens the chain of a tile's longest ray, which
-// is what a launch that does not fill the GPU with heavy tiles waits for: measured on 800x800 images,
-// sparse 512^3 tree 0.43 -> 0.34 ms (one pose), 0.62 -> 0.56 (four), 0.92 -> 0.87 (eight; with the
-// empty leaves marked 0.81 -> 0.77), sixteen poses equal; dense 128^3 tree 0.54 -> 0.37 (one), 0.84 ->
-// 0.75 (four).  Where every tile is heavy and the GPU full it costs: four 1008x756 NDC poses (47 628
-// tiles) 3 %, two of them 1 % (one gains 2 %), a batch of 256 Ki unrelated rays 33 %.  Hence: images of
-// up to 98 304 tiles (eight 800x800 poses are 80 000) -- but 16 384 under NDC, where every ray passes
-// through the tree --, ray batches of up to 128 Ki rays.
-bool use_split_forward(unsigned blocks, bool image, const SvoxRenderOptions* opt) {
+// Whether a forward launch of `blocks` 64-ray wavefronts takes render_forward_split_kernel (two wavefronts per 64
+// rays: one walks, one shades).  It shortens the chain of a tile's longest ray, which is what a launch that does not
+// fill the GPU with heavy tiles waits for; where every tile is heavy and the GPU full, the second wavefront only
+// takes a place another tile could have.  Measured on 800x800 poses of the sparse 512^3 SH16 tree (ms, one / two
+// wavefronts per tile), orbit of radius 4 (18 % of the rays hit the tree): 1 pose 0.41 / 0.34, 2 poses 0.45 / 0.37,
+// 4 poses 0.62 / 0.56, 8 poses 0.90 / 0.85, 16 poses 1.55 / 1.60; radius 2.5 (49 % hit): 0.43 / 0.38, 0.57 / 0.54,
+// 0.97 / 0.95, 1.61 / 1.64, 2.91 / 3.14; radius 1.5 (every ray hits): 0.54 / 0.52, 0.88 / 0.90, 1.71 / 1.82,
+// 3.14 / 3.40, 5.92 / 6.49.  With marks that decide the shading (`decided`: the one-wavefront kernel then reads a
+// leaf's density with its coefficients, the two-wavefront kernel gains nothing from them) the balance tips earlier,
+// launches alone: radius 4, 4 poses 0.48 / 0.47, 8 poses 0.69 / 0.72, 16 poses 1.13 / 1.30; radius 2.5, 8 poses
+// 1.22 / 1.33.  The launcher cannot know how many rays hit, so the rule goes by tiles: images of up to 65 536 tiles
+// (six 800x800 poses) -- 49 152 with deciding marks, 16 384 under NDC, where every ray passes through the tree --,
+// ray batches of up to 128 Ki rays (dense 128^3 tree: 1 pose 0.54 / 0.37, 4 poses 0.84 / 0.75; 4 NDC poses of 47 628
+// tiles 3.54 / 3.67; 256 Ki unrelated rays 0.29 / 0.39).
+bool use_split_forward(unsigned blocks, bool image, const SvoxRenderOptions* opt, bool decided) {
     const int forced = tuning().split_forward;
     const long limit = tuning().split_blocks;
     if (g_debug_flags & 12) return (g_debug_flags & 8) != 0;
     if (forced >= 0) return forced > 0;
     if (limit >= 0) return (long)blocks <= limit;
     if (!image) return blocks <= 2048u;
-    return blocks <= (opt->ndc_width > 0 ? 16384u : 98304u);
+    if (opt->ndc_width > 0) return blocks <= 16384u;
+    return blocks <= (decided ? 49152u : 65536u);
 }
 template <typename T>
 constexpr bool is_image_source(const ImageSource<T>&) { return true; }
@@ -426,7 +432,7 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
                                                dim3(blocks), dim3(kMarchThreads), 0, stream, tr, dealt, *opt,      \
                                                (float*)out, none))
             const bool refill = src.per_wave > kMarchThreads;
-            if (!refill && !tree->weight_accum && use_split_forward(blocks, is_image_source(src), opt)) {
+            if (!refill && !tree->weight_accum && use_split_forward(blocks, is_image_source(src), opt, all_shaded)) {
                 SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL((render_forward_split_kernel<P, Source, false>),
                                                            dim3(blocks), dim3(kSplitThreads), 0, stream, tr, dealt,
                                                            *opt, (float*)out, none));
@@ -548,7 +554,7 @@ int launch_noted(const SvoxTreeSpec* tree, const Source& src, const SvoxRenderOp
     memcpy(ws.stamp, stamp.word, sizeof(ws.stamp));
     ws.spin_limit = (g_debug_flags & 16) ? 1 : 0;
     const bool refill = src.per_wave > kMarchThreads;
-    const bool split = !refill && use_split_forward(blocks, is_image_source(src), opt);
+    const bool split = !refill && use_split_forward(blocks, is_image_source(src), opt, false);
     const dim3 threads(split ? kSplitThreads : kMarchThreads);
 #define SVOX_LAUNCH_NOTING(KERNEL)                                                                                   \
     SVOX_DISPATCH_OCTREE(D, hipLaunchKernelGGL(KERNEL, dim3(blocks), threads, 0, stream, march_tree(tree, opt), dealt, \
