@@ -709,6 +709,15 @@ def main():
             opt64 = svox.VolumeRenderer(gtree64)._get_options(False)
             generic["fp64_sh9_ms"] = round(ev_time(lambda: C.volume_render_image(gtree64._spec(), g64cam, opt64)), 4)
             generic["fp64_query_4M_ms"] = round(ev_time(lambda: C.query_vertical(gtree64._spec(), pts64)), 4)
+        # gradient and se_grad of the fp64 pose (one-ray-per-lane kernels whose wavefronts add the records of a step
+        # together; zero-fills of the fp64 gradient, 0.54 GB, included)
+        g64 = torch.Generator().manual_seed(12)
+        go64 = (torch.randn(H, W, 3, generator=g64, dtype=torch.float64) * 1e-2).to(dev)
+        ref64 = torch.rand(H, W, 3, generator=g64, dtype=torch.float64).to(dev)
+        generic["fp64_sh9_backward_ms"] = round(
+            ev_time(lambda: C.volume_render_image_backward(gtree64._spec(), g64cam, opt64, go64), n=3), 4)
+        generic["fp64_sh9_se_grad_ms"] = round(ev_time(lambda: C.se_grad_persp(gtree64._spec(), g64cam, opt64, ref64), n=3), 4)
+        del go64, ref64
         # a tree with branching factor 3 (81^3 leaves, SH9 records): the wavefront-per-tile kernels with the reference's
         # floating-point walk, against the same calls forced onto the one-ray-per-lane kernels
         t3 = svox.N3Tree(N=3, data_format="SH9", init_refine=3, device=dev)

@@ -1116,72 +1116,138 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
 // ------------------------------------------------------------------------------------------------
 // backward
 // ------------------------------------------------------------------------------------------------
-// trace_ray_backward, rt_kernel.cu:323-477, generic flavour: two marches, the colour gradients in
-// the first, the density gradient in the second; both test sigma > 0 and never stop early.
+// trace_ray_backward, rt_kernel.cu:323-477, generic flavour: one ray per lane, the reference's two marches --
+// <render, grad_out> and the colour gradient in the first, the density gradient in the second; both test
+// sigma > 0 and never stop early.  The colour terms are the reference's products (basis[i] * tmp2) but are not
+// scattered lane by lane: a lane whose sample has density leaves its factors (tmp2 per channel) and the offset of its
+// leaf in LDS, the lanes of a step that did so are listed, and the wavefront adds the listed records flat -- scalar f
+// of the list from lane f mod 64, so that consecutive scalars of a record go out together, one request per 64 bytes
+// instead of one per scalar (the memory system takes atomic adds at a fixed rate of requests).  For that the lanes
+// of a wavefront stay in the loop of the first march until the last of them is through.  The basis of a ray and its
+// grad_out sit in LDS as well, where the runtime-indexed loops of the reference can address them (in registers such
+// arrays end up in scratch memory).
+// Dynamic LDS, in scalars of T per lane: basis_dim (1 for RGBA) + 2 * out_dim, then 8 bytes (leaf offset) and 1
+// byte (list) per lane: generic_backward_lds_bytes.
 template <typename T>
-__device__ void trace_backward_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt, const T* origin,
-                                       const T* dir, const T* vdir, const T* scaling, int out_dim,
-                                       const T* grad_out, T* grad_data) {
+__host__ __device__ inline size_t generic_backward_lds_bytes(int basis_dim, int out_dim) {
+    return (size_t)kMarchThreads * ((size_t)(basis_dim + 2 * out_dim) * sizeof(T) + sizeof(int64_t) + 1);
+}
+
+template <typename T, class Source>
+__global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
+    TreeDev<T> tr, Source src, SvoxRenderOptions opt, int out_dim, const T* __restrict__ grad_out,
+    T* __restrict__ grad_data) {
+    extern __shared__ __align__(16) unsigned char generic_lds[];
+    const int lane = threadIdx.x;
+    const bool rgba = opt.format == SVOX_FORMAT_RGBA;
+    const int bd = rgba ? 1 : opt.basis_dim;
+    T* const sh_basis = (T*)generic_lds;                                    // [lane * bd + i]
+    T* const sh_go = sh_basis + kMarchThreads * bd;                         // [c * 64 + lane]: grad_out of the ray
+    T* const sh_factor = sh_go + kMarchThreads * out_dim;                   // [c * 64 + lane]: tmp2 of the sample
+    int64_t* const sh_base = (int64_t*)(sh_factor + kMarchThreads * out_dim);   // [lane]: leaf * K
+    uint8_t* const sh_list = (uint8_t*)(sh_base + kMarchThreads);           // lanes with a record in this step
+
+    T offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    T origin[3], dir[3], vdir[3];
+    const int64_t item = blockIdx.x * (int64_t)kMarchThreads + lane;
+    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
     RayState<T> r;
-    if (!setup_ray(r, origin, dir, scaling)) return;
-    T basis[SVOX_MAX_BASIS_DIM];
-    precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
-    T go[SVOX_MAX_OUT_DIM];
-    for (int j = 0; j < out_dim; ++j) go[j] = grad_out[j];
+    bool alive = slot >= 0 && setup_ray(r, origin, dir, scaling);
+    if (alive) {
+        if (!rgba) {
+            T basis[SVOX_MAX_BASIS_DIM];
+            precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
+#pragma unroll
+            for (int i = 0; i < SVOX_MAX_BASIS_DIM; ++i)
+                if (i < bd) sh_basis[lane * bd + i] = basis[i];
+        }
+        for (int j = 0; j < out_dim; ++j) sh_go[j * kMarchThreads + lane] = grad_out[slot * out_dim + j];
+    }
+    wave_lds_sync();
+    const T* const my_basis = sh_basis + lane * bd;
     const T pad = (T)opt.rgb_padding;
     const T d_rgb_pad = (T)(1 + 2 * opt.rgb_padding);
-    const T tmin = r.t;
+    const int lo = rgba ? 0 : opt.min_comp;
+    const int n_comp = rgba ? 1 : (opt.max_comp - opt.min_comp + 1 > 0 ? opt.max_comp - opt.min_comp + 1 : 0);
+    const int per_record = out_dim * n_comp;
+    const T tmin = alive ? r.t : T(0);
     T accum = T(0);
     {
         T light = T(1);
-        while (r.t < r.tmax) {
-            T delta_t;
-            const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
-            if (v.leaf < 0) return;
-            const int64_t base = v.leaf * tr.K;
-            const T* val = tr.data + base;
-            T sigma = val[tr.K - 1];
-            if (opt.density_softplus) sigma = softplus_m1(sigma);
-            if (sigma > T(0)) {
-                const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
-                const T weight = light * (T(1) - att);
-                T total_color = T(0);
-                if (opt.format != SVOX_FORMAT_RGBA) {
-                    for (int c = 0; c < out_dim; ++c) {
-                        const int off = c * opt.basis_dim;
-                        T tmp = T(0);
-                        for (int i = opt.min_comp; i <= opt.max_comp; ++i)
-                            tmp = fma_(basis[i], val[off + i], tmp);
-                        const T sg = sigmoid_(tmp);
-                        const T tmp2 = (T)((double)(weight * sg) * (1.0 - (double)sg) * (double)go[c] *
-                                           (double)d_rgb_pad);
-                        for (int i = opt.min_comp; i <= opt.max_comp; ++i)
-                            atomicAdd(grad_data + base + off + i, basis[i] * tmp2);
-                        total_color = fma_(fma_(sg, d_rgb_pad, -pad), go[c], total_color);
-                    }
+        while (__any(alive && r.t < r.tmax)) {
+            bool emit = false;
+            if (alive && r.t < r.tmax) {
+                T delta_t;
+                const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+                if (v.leaf < 0) {
+                    alive = false;   // a broken tree: the reference leaves the ray here, second march included
                 } else {
-                    for (int c = 0; c < out_dim; ++c) {
-                        const T sg = sigmoid_(val[c]);
-                        atomicAdd(grad_data + base + c, weight * sg * (T(1) - sg) * go[c] * d_rgb_pad);
-                        total_color = fma_(fma_(sg, d_rgb_pad, -pad), go[c], total_color);
+                    const int64_t base = v.leaf * tr.K;
+                    const T* val = tr.data + base;
+                    T sigma = val[tr.K - 1];
+                    if (opt.density_softplus) sigma = softplus_m1(sigma);
+                    if (sigma > T(0)) {
+                        const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
+                        const T weight = light * (T(1) - att);
+                        T total_color = T(0);
+                        for (int c = 0; c < out_dim; ++c) {
+                            const T go_c = sh_go[c * kMarchThreads + lane];
+                            T sg;
+                            if (!rgba) {
+                                const int off = c * opt.basis_dim;
+                                T tmp = T(0);
+                                for (int i = opt.min_comp; i <= opt.max_comp; ++i)
+                                    tmp = fma_(my_basis[i], val[off + i], tmp);
+                                sg = sigmoid_(tmp);
+                                sh_factor[c * kMarchThreads + lane] =
+                                    (T)((double)(weight * sg) * (1.0 - (double)sg) * (double)go_c * (double)d_rgb_pad);
+                            } else {
+                                sg = sigmoid_(val[c]);
+                                sh_factor[c * kMarchThreads + lane] = weight * sg * (T(1) - sg) * go_c * d_rgb_pad;
+                            }
+                            total_color = fma_(fma_(sg, d_rgb_pad, -pad), go_c, total_color);
+                        }
+                        sh_base[lane] = base;
+                        emit = per_record > 0;
+                        light *= att;
+                        accum = fma_(weight, total_color, accum);
                     }
+                    advance(r, delta_t);
                 }
-                light *= att;
-                accum = fma_(weight, total_color, accum);
             }
-            advance(r, delta_t);
+            // the records of this step, added by the whole wavefront
+            const unsigned long long m = __ballot(emit);
+            if (m != 0) {
+                if (emit) sh_list[rank_in(m)] = (uint8_t)lane;
+                wave_lds_sync();
+                const int n_scalars = __popcll(m) * per_record;
+                for (int f = lane; f < n_scalars; f += kMarchThreads) {
+                    const int rec = f / per_record, e = f - rec * per_record;
+                    const int c = e / n_comp, i = lo + (e - c * n_comp);
+                    const int owner = sh_list[rec];
+                    const T factor = sh_factor[c * kMarchThreads + owner];
+                    if (rgba)
+                        atomicAdd(grad_data + sh_base[owner] + c, factor);
+                    else
+                        atomicAdd(grad_data + sh_base[owner] + c * opt.basis_dim + i, sh_basis[owner * bd + i] * factor);
+                }
+                wave_lds_sync();
+            }
         }
-        T total_grad = T(0);
-        for (int j = 0; j < out_dim; ++j) total_grad += go[j];
-        accum = fma_(light * (T)opt.background_brightness, total_grad, accum);
+        if (alive) {
+            T total_grad = T(0);
+            for (int j = 0; j < out_dim; ++j) total_grad += sh_go[j * kMarchThreads + lane];
+            accum = fma_(light * (T)opt.background_brightness, total_grad, accum);
+        }
     }
-    {
+    if (alive) {
         T light = T(1);
         r.t = tmin;
         while (r.t < r.tmax) {
             T delta_t;
             const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
-            if (v.leaf < 0) return;
+            if (v.leaf < 0) break;
             const int64_t base = v.leaf * tr.K;
             const T* val = tr.data + base;
             T sigma = val[tr.K - 1];
@@ -1191,23 +1257,23 @@ __device__ void trace_backward_generic(const TreeDev<T>& tr, const SvoxRenderOpt
                 const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
                 const T weight = light * (T(1) - att);
                 T total_color = T(0);
-                if (opt.format != SVOX_FORMAT_RGBA) {
-                    for (int c = 0; c < out_dim; ++c) {
+                for (int c = 0; c < out_dim; ++c) {
+                    const T go_c = sh_go[c * kMarchThreads + lane];
+                    T sg;
+                    if (!rgba) {
                         const int off = c * opt.basis_dim;
                         T tmp = T(0);
-                        for (int i = opt.min_comp; i <= opt.max_comp; ++i)
-                            tmp = fma_(basis[i], val[off + i], tmp);
-                        total_color = fma_(fma_(sigmoid_(tmp), d_rgb_pad, -pad), go[c], total_color);
+                        for (int i = opt.min_comp; i <= opt.max_comp; ++i) tmp = fma_(my_basis[i], val[off + i], tmp);
+                        sg = sigmoid_(tmp);
+                    } else {
+                        sg = sigmoid_(val[c]);
                     }
-                } else {
-                    for (int c = 0; c < out_dim; ++c)
-                        total_color = fma_(fma_(sigmoid_(val[c]), d_rgb_pad, -pad), go[c], total_color);
+                    total_color = fma_(fma_(sg, d_rgb_pad, -pad), go_c, total_color);
                 }
                 light *= att;
                 accum = fma_(-weight, total_color, accum);
                 const T chain = opt.density_softplus ? sigmoid_(raw_sigma - T(1)) : T(1);
-                atomicAdd(grad_data + base + tr.K - 1,
-                          delta_t * r.dscale * fma_(total_color, light, -accum) * chain);
+                atomicAdd(grad_data + base + tr.K - 1, delta_t * r.dscale * fma_(total_color, light, -accum) * chain);
             }
             advance(r, delta_t);
         }
@@ -1217,19 +1283,6 @@ __device__ void trace_backward_generic(const TreeDev<T>& tr, const SvoxRenderOpt
 // value of `v` in lane `k` (k uniform across the wavefront)
 __device__ __forceinline__ float read_lane(float v, int k) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), k));
-}
-
-template <typename T, class Source>
-__global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
-    TreeDev<T> tr, Source src, SvoxRenderOptions opt, int out_dim, const T* __restrict__ grad_out,
-    T* __restrict__ grad_data) {
-    T offset[3], scaling[3];
-    load_transform(tr, offset, scaling);
-    T origin[3], dir[3], vdir[3];
-    const int64_t item = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
-    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
-    if (slot < 0) return;
-    trace_backward_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, grad_out + slot * out_dim, grad_data);
 }
 
 // trace_ray_backward, octree flavour: a persistent wavefront working in the forward kernel's rounds
@@ -2150,28 +2203,58 @@ __device__ __forceinline__ T channel_sigmoid(const SvoxRenderOptions& opt, const
     return sigmoid_(tmp);
 }
 
-// trace_ray_se_grad_hess, rt_kernel.cu:479-715, generic flavour: three marches (residual; colour
+// trace_ray_se_grad_hess, rt_kernel.cu:479-715, generic flavour: one ray per lane, three marches (residual; colour
 // gradients and the rendered colour as a running suffix; density gradients), all with sigma > 0 and
 // no early stop.  The attenuation argument is spelled -delta_t * delta_scale * sigma in the first
 // march and -delta_t * sigma * delta_scale in the other two, as in the reference.  The reference's
-// out_dim atomics per sample on the density entry are summed first and added once.
-template <typename T>
-__device__ void trace_se_grad_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt, const T* origin,
-                                      const T* dir, const T* vdir, const T* scaling, int out_dim,
-                                      const T* color_ref, T* color_out, T* grad, T* hess) {
+// out_dim atomics per sample on the density entry are summed first and added once.  The colour terms of the second
+// march are added by the whole wavefront, flat over the records of the lanes that have one in the step, as in
+// render_backward_generic_kernel (same LDS layout: the second block of out_dim scalars per lane holds the ray's
+// residual instead of grad_out), into both arrays.
+template <typename T, class Source>
+__global__ __launch_bounds__(kMarchThreads) void se_grad_generic_kernel(TreeDev<T> tr, Source src,
+                                                                        SvoxRenderOptions opt, int out_dim,
+                                                                        const T* __restrict__ color_ref,
+                                                                        T* __restrict__ color_out,
+                                                                        T* __restrict__ grad, T* __restrict__ hess) {
+    extern __shared__ __align__(16) unsigned char generic_lds[];
+    const int lane = threadIdx.x;
+    const bool rgba = opt.format == SVOX_FORMAT_RGBA;
+    const int bd = rgba ? 1 : opt.basis_dim;
+    T* const sh_basis = (T*)generic_lds;                                    // [lane * bd + i]
+    T* const sh_resid = sh_basis + kMarchThreads * bd;                      // [c * 64 + lane]: residual of the ray
+    T* const sh_factor = sh_resid + kMarchThreads * out_dim;                // [c * 64 + lane]: grad_ci of the sample
+    int64_t* const sh_base = (int64_t*)(sh_factor + kMarchThreads * out_dim);   // [lane]: leaf * K
+    uint8_t* const sh_list = (uint8_t*)(sh_base + kMarchThreads);           // lanes with a record in this step
+
+    T offset[3], scaling[3];
+    load_transform(tr, offset, scaling);
+    T origin[3], dir[3], vdir[3];
+    const int64_t item = blockIdx.x * (int64_t)kMarchThreads + lane;
+    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
+    const T bg = (T)opt.background_brightness;
     RayState<T> r;
-    if (!setup_ray(r, origin, dir, scaling)) {
-        for (int j = 0; j < out_dim; ++j) color_out[j] = (T)opt.background_brightness;
-        return;
+    bool alive = slot >= 0 && setup_ray(r, origin, dir, scaling);
+    if (slot >= 0 && !alive) {
+        for (int j = 0; j < out_dim; ++j) color_out[slot * out_dim + j] = bg;
     }
-    T basis[SVOX_MAX_BASIS_DIM];
-    precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
+    if (alive && !rgba) {
+        T basis[SVOX_MAX_BASIS_DIM];
+        precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
+#pragma unroll
+        for (int i = 0; i < SVOX_MAX_BASIS_DIM; ++i)
+            if (i < bd) sh_basis[lane * bd + i] = basis[i];
+    }
+    wave_lds_sync();
+    const T* const my_basis = sh_basis + lane * bd;
     const T pad = (T)opt.rgb_padding;
     const T d_rgb_pad = (T)(1 + 2 * opt.rgb_padding);
-    const T bg = (T)opt.background_brightness;
-    const T tmin = r.t;
+    const int lo = rgba ? 0 : opt.min_comp;
+    const int n_comp = rgba ? 1 : (opt.max_comp - opt.min_comp + 1 > 0 ? opt.max_comp - opt.min_comp + 1 : 0);
+    const int per_record = out_dim * n_comp;
+    const T tmin = alive ? r.t : T(0);
     T resid[4] = {T(0), T(0), T(0), T(0)};
-    {
+    if (alive) {
         T light = T(1);
         while (r.t < r.tmax) {
             T delta_t;
@@ -2184,51 +2267,73 @@ __device__ void trace_se_grad_generic(const TreeDev<T>& tr, const SvoxRenderOpti
                 const T att = exp_sp<T>(-delta_t * r.dscale * sigma);
                 const T weight = light * (T(1) - att);
                 for (int c = 0; c < out_dim; ++c)
-                    resid[c] = fma_(weight, fma_(channel_sigmoid(opt, basis, val, c), d_rgb_pad, -pad), resid[c]);
+                    resid[c] = fma_(weight, fma_(channel_sigmoid(opt, my_basis, val, c), d_rgb_pad, -pad), resid[c]);
                 light *= att;
             }
             advance(r, delta_t);
         }
-        for (int j = 0; j < out_dim; ++j) resid[j] += fma_(light, bg, -color_ref[j]);
+        for (int j = 0; j < out_dim; ++j) {
+            resid[j] += fma_(light, bg, -color_ref[slot * out_dim + j]);
+            sh_resid[j * kMarchThreads + lane] = resid[j];
+        }
     }
+    wave_lds_sync();
     T color_accum[4] = {T(0), T(0), T(0), T(0)};
     {
         T light = T(1);
-        r.t = tmin;
-        while (r.t < r.tmax) {
-            T delta_t;
-            const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
-            if (v.leaf < 0) break;
-            const int64_t base = v.leaf * tr.K;
-            const T* val = tr.data + base;
-            T sigma = val[tr.K - 1];
-            if (opt.density_softplus) sigma = softplus_m1(sigma);
-            if (sigma > T(0)) {
-                const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
-                const T weight = light * (T(1) - att);
-                for (int c = 0; c < out_dim; ++c) {
-                    const T sg = channel_sigmoid(opt, basis, val, c);
-                    if (opt.format != SVOX_FORMAT_RGBA) {
-                        const T grad_ci = (T)((double)(weight * sg) * (1.0 - (double)sg) * (double)d_rgb_pad);
-                        const int off = c * opt.basis_dim;
-                        for (int i = opt.min_comp; i <= opt.max_comp; ++i) {
-                            const T grad_wi = basis[i] * grad_ci;
-                            atomicAdd(grad + base + off + i, grad_wi * resid[c]);
-                            atomicAdd(hess + base + off + i, grad_wi * grad_wi);
+        if (alive) r.t = tmin;
+        bool marching = alive;   // (a broken tree ends this march, not the ray: the reference breaks out of the loop)
+        while (__any(marching && r.t < r.tmax)) {
+            bool emit = false;
+            if (marching && r.t < r.tmax) {
+                T delta_t;
+                const Visit v = step_generic<T>(tr, r, (T)opt.step_size, &delta_t);
+                if (v.leaf < 0) {
+                    marching = false;
+                } else {
+                    const int64_t base = v.leaf * tr.K;
+                    const T* val = tr.data + base;
+                    T sigma = val[tr.K - 1];
+                    if (opt.density_softplus) sigma = softplus_m1(sigma);
+                    if (sigma > T(0)) {
+                        const T att = exp_sp<T>(-delta_t * sigma * r.dscale);
+                        const T weight = light * (T(1) - att);
+                        for (int c = 0; c < out_dim; ++c) {
+                            const T sg = channel_sigmoid(opt, my_basis, val, c);
+                            sh_factor[c * kMarchThreads + lane] =
+                                rgba ? weight * sg * (T(1) - sg) * d_rgb_pad
+                                     : (T)((double)(weight * sg) * (1.0 - (double)sg) * (double)d_rgb_pad);
+                            color_accum[c] = fma_(weight, fma_(sg, d_rgb_pad, -pad), color_accum[c]);
                         }
-                    } else {
-                        const T grad_ci = weight * sg * (T(1) - sg) * d_rgb_pad;
-                        atomicAdd(grad + base + c, grad_ci * resid[c]);
-                        atomicAdd(hess + base + c, grad_ci * grad_ci);
+                        sh_base[lane] = base;
+                        emit = per_record > 0;
+                        light *= att;
                     }
-                    color_accum[c] = fma_(weight, fma_(sg, d_rgb_pad, -pad), color_accum[c]);
+                    advance(r, delta_t);
                 }
-                light *= att;
             }
-            advance(r, delta_t);
+            const unsigned long long m = __ballot(emit);
+            if (m != 0) {
+                if (emit) sh_list[rank_in(m)] = (uint8_t)lane;
+                wave_lds_sync();
+                const int n_scalars = __popcll(m) * per_record;
+                for (int f = lane; f < n_scalars; f += kMarchThreads) {
+                    const int rec = f / per_record, e = f - rec * per_record;
+                    const int c = e / n_comp, i = lo + (e - c * n_comp);
+                    const int owner = sh_list[rec];
+                    const T grad_ci = sh_factor[c * kMarchThreads + owner];
+                    const T grad_wi = rgba ? grad_ci : sh_basis[owner * bd + i] * grad_ci;
+                    const int64_t at = sh_base[owner] + (rgba ? c : c * opt.basis_dim + i);
+                    atomicAdd(grad + at, grad_wi * sh_resid[c * kMarchThreads + owner]);
+                    atomicAdd(hess + at, grad_wi * grad_wi);
+                }
+                wave_lds_sync();
+            }
         }
-        for (int j = 0; j < out_dim; ++j) color_accum[j] = fma_(light, bg, color_accum[j]);
+        if (alive)
+            for (int j = 0; j < out_dim; ++j) color_accum[j] = fma_(light, bg, color_accum[j]);
     }
+    if (!alive) return;
     {
         T light = T(1);
         r.t = tmin;
@@ -2245,7 +2350,7 @@ __device__ void trace_se_grad_generic(const TreeDev<T>& tr, const SvoxRenderOpti
                 const T weight = light * (T(1) - att);
                 T color_curr[4];
                 for (int c = 0; c < out_dim; ++c) {
-                    color_curr[c] = fma_(channel_sigmoid(opt, basis, val, c), d_rgb_pad, -pad);
+                    color_curr[c] = fma_(channel_sigmoid(opt, my_basis, val, c), d_rgb_pad, -pad);
                     color_accum[c] = fma_(-weight, color_curr[c], color_accum[c]);
                 }
                 light *= att;
@@ -2269,23 +2374,7 @@ __device__ void trace_se_grad_generic(const TreeDev<T>& tr, const SvoxRenderOpti
             advance(r, delta_t);
         }
     }
-    for (int j = 0; j < out_dim; ++j) color_out[j] = resid[j] + color_ref[j];
-}
-
-template <typename T, class Source>
-__global__ __launch_bounds__(kMarchThreads) void se_grad_generic_kernel(TreeDev<T> tr, Source src,
-                                                                        SvoxRenderOptions opt, int out_dim,
-                                                                        const T* __restrict__ color_ref,
-                                                                        T* __restrict__ color_out,
-                                                                        T* __restrict__ grad, T* __restrict__ hess) {
-    T offset[3], scaling[3];
-    load_transform(tr, offset, scaling);
-    T origin[3], dir[3], vdir[3];
-    const int64_t item = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
-    const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
-    if (slot < 0) return;
-    trace_se_grad_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, color_ref + slot * out_dim,
-                             color_out + slot * out_dim, grad, hess);
+    for (int j = 0; j < out_dim; ++j) color_out[slot * out_dim + j] = resid[j] + color_ref[slot * out_dim + j];
 }
 
 // trace_ray_se_grad_hess, octree flavour: the backward kernel's persistent wavefront and rounds.

@@ -519,9 +519,10 @@ void launch_backward(const SvoxTreeSpec* tree, const Source& src, const SvoxRend
             return;
         }
     }
+    const int basis_rows = opt->format == SVOX_FORMAT_RGBA ? 1 : opt->basis_dim;
     hipLaunchKernelGGL((render_backward_generic_kernel<T, Source>), dim3(blocks_for(items, kMarchThreads)),
-                       dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (const T*)grad_out,
-                       (T*)grad_data);
+                       dim3(kMarchThreads), generic_backward_lds_bytes<T>(basis_rows, out_dim), stream,
+                       make_tree<T>(tree), src, *opt, out_dim, (const T*)grad_out, (T*)grad_data);
 }
 
 // The launch shape of the noting forward pass for the rays of `s`: that of a forward pass (a batch
@@ -634,9 +635,10 @@ void launch_se_grad(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
             return;
         }
     }
+    const int basis_rows = opt->format == SVOX_FORMAT_RGBA ? 1 : opt->basis_dim;
     hipLaunchKernelGGL((se_grad_generic_kernel<T, Source>), dim3(blocks_for(items, kMarchThreads)),
-                       dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (const T*)color_ref,
-                       (T*)color_out, (T*)grad, (T*)hess);
+                       dim3(kMarchThreads), generic_backward_lds_bytes<T>(basis_rows, out_dim), stream,
+                       make_tree<T>(tree), src, *opt, out_dim, (const T*)color_ref, (T*)color_out, (T*)grad, (T*)hess);
 }
 
 // shared argument checks and zero-fills of the two squared-error entry points
