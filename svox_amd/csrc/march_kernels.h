@@ -447,19 +447,26 @@ __device__ __forceinline__ void atomic_max_float(double* addr, double value) {
 // ------------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------------
-// trace_ray, rt_kernel.cu:222-321, generic flavour
+// trace_ray, rt_kernel.cu:222-321, generic flavour.  `basis` and `acc` are this lane's columns of two LDS arrays
+// laid out [index][lane] (stride kMarchThreads): the reference's loops index them at run time, and as register
+// arrays they would live in scratch memory.
 template <typename T>
 __device__ void trace_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt, const T* origin,
-                              const T* dir, const T* vdir, const T* scaling, int out_dim, T* out) {
+                              const T* dir, const T* vdir, const T* scaling, int out_dim, T* out, T* basis, T* acc) {
+    constexpr int S = kMarchThreads;
     RayState<T> r;
-    T acc[SVOX_MAX_OUT_DIM];
     if (!setup_ray(r, origin, dir, scaling)) {
         for (int j = 0; j < out_dim; ++j) out[j] = (T)opt.background_brightness;
         return;
     }
-    for (int j = 0; j < out_dim; ++j) acc[j] = T(0);
-    T basis[SVOX_MAX_BASIS_DIM];
-    precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
+    for (int j = 0; j < out_dim; ++j) acc[j * S] = T(0);
+    if (opt.format != SVOX_FORMAT_RGBA) {
+        T b[SVOX_MAX_BASIS_DIM];
+        precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, b);
+#pragma unroll
+        for (int i = 0; i < SVOX_MAX_BASIS_DIM; ++i)
+            if (i < opt.basis_dim) basis[i * S] = b[i];
+    }
     T light = T(1);
     const T pad = (T)opt.rgb_padding;
     const T d_rgb_pad = (T)(1 + 2 * opt.rgb_padding);
@@ -478,12 +485,12 @@ __device__ void trace_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt
                 for (int c = 0; c < out_dim; ++c) {
                     const int off = c * opt.basis_dim;
                     T tmp = T(0);
-                    for (int i = opt.min_comp; i <= opt.max_comp; ++i) tmp = fma_(basis[i], val[off + i], tmp);
-                    acc[c] = fma_(weight, fma_(sigmoid_(tmp), d_rgb_pad, -pad), acc[c]);
+                    for (int i = opt.min_comp; i <= opt.max_comp; ++i) tmp = fma_(basis[i * S], val[off + i], tmp);
+                    acc[c * S] = fma_(weight, fma_(sigmoid_(tmp), d_rgb_pad, -pad), acc[c * S]);
                 }
             } else {
                 for (int c = 0; c < out_dim; ++c)
-                    acc[c] = fma_(weight, fma_(sigmoid_(val[c]), d_rgb_pad, -pad), acc[c]);
+                    acc[c * S] = fma_(weight, fma_(sigmoid_(val[c]), d_rgb_pad, -pad), acc[c * S]);
             }
             light *= att;
             if (tr.weight_accum) {
@@ -494,7 +501,7 @@ __device__ void trace_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt
             }
             if (light <= (T)opt.stop_thresh) {
                 const T scale = (T)(1.0 / (1.0 - (double)light));
-                for (int j = 0; j < out_dim; ++j) acc[j] *= scale;
+                for (int j = 0; j < out_dim; ++j) acc[j * S] *= scale;
                 stopped = true;
                 break;
             }
@@ -502,8 +509,8 @@ __device__ void trace_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt
         advance(r, delta_t);
     }
     if (!stopped)
-        for (int j = 0; j < out_dim; ++j) acc[j] = fma_(light, (T)opt.background_brightness, acc[j]);
-    for (int j = 0; j < out_dim; ++j) out[j] = acc[j];
+        for (int j = 0; j < out_dim; ++j) acc[j * S] = fma_(light, (T)opt.background_brightness, acc[j * S]);
+    for (int j = 0; j < out_dim; ++j) out[j] = acc[j * S];
 }
 
 // colour of one leaf record for the octree flavour: 3 sigmoids of basis . coefficients.
@@ -534,17 +541,26 @@ __device__ __forceinline__ int rank_in(unsigned long long mask) {
 }
 
 // trace_ray for the generic policy: one ray per lane, no sharing of work between lanes
+template <typename T>
+__host__ __device__ inline size_t generic_forward_lds_bytes(int basis_dim, int out_dim) {
+    return (size_t)kMarchThreads * (size_t)(basis_dim + out_dim) * sizeof(T);
+}
 template <typename T, class Source>
 __global__ __launch_bounds__(kMarchThreads) void render_forward_generic_kernel(TreeDev<T> tr, Source src,
                                                                                SvoxRenderOptions opt, int out_dim,
                                                                                T* __restrict__ out) {
+    // dynamic LDS: (basis_dim + out_dim) scalars of T per lane, generic_forward_lds_bytes
+    extern __shared__ __align__(16) unsigned char generic_lds[];
+    T* const sh_basis = (T*)generic_lds;
+    T* const sh_acc = sh_basis + kMarchThreads * (opt.format == SVOX_FORMAT_RGBA ? 1 : opt.basis_dim);
     T offset[3], scaling[3];
     load_transform(tr, offset, scaling);
     T origin[3], dir[3], vdir[3];
     const int64_t item = blockIdx.x * (int64_t)kMarchThreads + threadIdx.x;
     const int64_t slot = src.fetch_item(item, opt, offset, scaling, origin, dir, vdir);
     if (slot < 0) return;
-    trace_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, out + slot * out_dim);
+    trace_generic<T>(tr, opt, origin, dir, vdir, scaling, out_dim, out + slot * out_dim, sh_basis + threadIdx.x,
+                     sh_acc + threadIdx.x);
 }
 
 constexpr int kQueue = 4;  // leaves a lane walks ahead before the wavefront shades them
@@ -1126,11 +1142,11 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
 // of a wavefront stay in the loop of the first march until the last of them is through.  The basis of a ray and its
 // grad_out sit in LDS as well, where the runtime-indexed loops of the reference can address them (in registers such
 // arrays end up in scratch memory).
-// Dynamic LDS, in scalars of T per lane: basis_dim (1 for RGBA) + 2 * out_dim, then 8 bytes (leaf offset) and 1
-// byte (list) per lane: generic_backward_lds_bytes.
+// Dynamic LDS, in scalars of T per lane: basis_dim (1 for RGBA) made odd, so that the lanes' rows start in different
+// banks, + 2 * out_dim, then 8 bytes (leaf offset) and 1 byte (list) per lane: generic_backward_lds_bytes.
 template <typename T>
 __host__ __device__ inline size_t generic_backward_lds_bytes(int basis_dim, int out_dim) {
-    return (size_t)kMarchThreads * ((size_t)(basis_dim + 2 * out_dim) * sizeof(T) + sizeof(int64_t) + 1);
+    return (size_t)kMarchThreads * ((size_t)((basis_dim | 1) + 2 * out_dim) * sizeof(T) + sizeof(int64_t) + 1);
 }
 
 template <typename T, class Source>
@@ -1140,7 +1156,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
     extern __shared__ __align__(16) unsigned char generic_lds[];
     const int lane = threadIdx.x;
     const bool rgba = opt.format == SVOX_FORMAT_RGBA;
-    const int bd = rgba ? 1 : opt.basis_dim;
+    const int bd = (rgba ? 1 : opt.basis_dim) | 1;                          // row length, odd
     T* const sh_basis = (T*)generic_lds;                                    // [lane * bd + i]
     T* const sh_go = sh_basis + kMarchThreads * bd;                         // [c * 64 + lane]: grad_out of the ray
     T* const sh_factor = sh_go + kMarchThreads * out_dim;                   // [c * 64 + lane]: tmp2 of the sample
@@ -1160,7 +1176,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_generic_kernel(
             precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
 #pragma unroll
             for (int i = 0; i < SVOX_MAX_BASIS_DIM; ++i)
-                if (i < bd) sh_basis[lane * bd + i] = basis[i];
+                if (i < opt.basis_dim) sh_basis[lane * bd + i] = basis[i];
         }
         for (int j = 0; j < out_dim; ++j) sh_go[j * kMarchThreads + lane] = grad_out[slot * out_dim + j];
     }
@@ -2220,7 +2236,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_generic_kernel(TreeDev<
     extern __shared__ __align__(16) unsigned char generic_lds[];
     const int lane = threadIdx.x;
     const bool rgba = opt.format == SVOX_FORMAT_RGBA;
-    const int bd = rgba ? 1 : opt.basis_dim;
+    const int bd = (rgba ? 1 : opt.basis_dim) | 1;                          // row length, odd
     T* const sh_basis = (T*)generic_lds;                                    // [lane * bd + i]
     T* const sh_resid = sh_basis + kMarchThreads * bd;                      // [c * 64 + lane]: residual of the ray
     T* const sh_factor = sh_resid + kMarchThreads * out_dim;                // [c * 64 + lane]: grad_ci of the sample
@@ -2243,7 +2259,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_generic_kernel(TreeDev<
         precalc_basis<T>(opt.format, opt.basis_dim, tr.extra, tr.extra_cols, vdir, basis);
 #pragma unroll
         for (int i = 0; i < SVOX_MAX_BASIS_DIM; ++i)
-            if (i < bd) sh_basis[lane * bd + i] = basis[i];
+            if (i < opt.basis_dim) sh_basis[lane * bd + i] = basis[i];
     }
     wave_lds_sync();
     const T* const my_basis = sh_basis + lane * bd;

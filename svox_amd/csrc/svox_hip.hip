@@ -450,8 +450,10 @@ void launch_forward(const SvoxTreeSpec* tree, const Source& src, const SvoxRende
             return;
         }
     }
+    const int basis_rows = opt->format == SVOX_FORMAT_RGBA ? 1 : opt->basis_dim;
     hipLaunchKernelGGL((render_forward_generic_kernel<T, Source>), dim3(blocks_for(items, kMarchThreads)),
-                       dim3(kMarchThreads), 0, stream, make_tree<T>(tree), src, *opt, out_dim, (T*)out);
+                       dim3(kMarchThreads), generic_forward_lds_bytes<T>(basis_rows, out_dim), stream,
+                       make_tree<T>(tree), src, *opt, out_dim, (T*)out);
 }
 
 constexpr int64_t kChunkBytes = (int64_t)kChunkFloat2 * 8;   // 384: 15 records and a link
