@@ -220,7 +220,10 @@ __global__ __launch_bounds__(256) void mark_leaves_kernel(const T* __restrict__ 
     const int32_t c = child[i];
     int32_t m = c;
     if (c == 0) {
-        T sigma = data[i * K + (K - 1)];
+        // read past the caches' keep-list: a density is 4 bytes of a line nobody asks for again soon, and 0.7 GB of
+        // such lines would push the child table and the marks out of L2 ahead of the render that follows
+        // (8 poses of 800x800: marking 0.141 -> 0.129 ms, the render call as a whole 0.811 -> 0.790 ms)
+        T sigma = __builtin_nontemporal_load(&data[i * K + (K - 1)]);
         if (softplus) sigma = softplus_m1(sigma);
         m = sigma > thresh ? 0 : SVOX_EMPTY_LEAF;
     }
