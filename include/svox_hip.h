@@ -367,10 +367,11 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
                              SvoxMarchStats* stats_out, void* stream);
 
 /* No counterpart in the reference.  Which family of kernels serves the render calls of this tree under
- * these options: 1 the wavefront-per-tile octree kernels (fp32, N = 2, RGBA / SH / SG / ASG records with
- * basis_dim 1, 4, 9, 16 or 25 and the full component range), 0 the one-ray-per-lane kernels that cover
- * everything else the reference accepts (fp64, other N, other basis sizes, partial component ranges), or a
- * negative SvoxStatus for a tree or options no kernel accepts.  Results do not depend on the family. */
+ * these options (forward, backward and se_grad alike, with or without density_softplus): 1 the
+ * wavefront-per-tile kernels (fp32, any branching factor, fewer than 2^30 cells, RGBA / SH / SG / ASG records
+ * with basis_dim 1, 4, 9, 16 or 25 and the full component range), 0 the one-ray-per-lane kernels that cover
+ * everything else the reference accepts (fp64, other basis sizes and record shapes, partial component ranges), or
+ * a negative SvoxStatus for a tree or options no kernel accepts.  Results do not depend on the family. */
 int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt);
 
 /* No counterpart in the reference.  1 if the noting calls (svox_volume_render_noted, svox_volume_render_images_noted)

@@ -20,6 +20,7 @@ constexpr int kQueryThreads = 256;
 constexpr int kWave = 64;
 
 enum QueryMode { kQueryGather = 0, kQueryScatterAdd = 1, kQueryAssign = 2 };
+typedef unsigned int Piece16 __attribute__((ext_vector_type(4)));   // 16 bytes as the non-temporal builtins take them
 
 constexpr int kQueryPts = 2;   // points a lane walks in lockstep (their child reads overlap)
 
@@ -139,7 +140,9 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(TreeDev<T> tr, con
 #pragma unroll
                     for (int b = 0; b < kBatch; ++b) {
                         const int f = f0 + b * kWave + lane;
-                        if (f < total) lin16[f] = buf[b];
+                        // (stored past the caches' keep-list: the output is written once, and the tree it is gathered
+                        // from should stay in the last-level cache: 4 Mi points of a 268 MB tree 0.346 -> 0.332 ms)
+                        if (f < total) __builtin_nontemporal_store((Piece16){buf[b].x, buf[b].y, buf[b].z, buf[b].w}, (Piece16*)lin16 + f);
                     }
                 }
                 continue;
@@ -154,9 +157,9 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(TreeDev<T> tr, con
                 const int64_t lf = ((int64_t)hi << 32) | (uint32_t)lo;
                 if (f < total && lf >= 0) {
                     if (MODE == kQueryGather) {
-                        lin[f] = tr.data[lf * row + e];
+                        __builtin_nontemporal_store(tr.data[lf * row + e], &lin[f]);
                     } else if (MODE == kQueryScatterAdd) {
-                        atomicAdd(target + lf * row + e, lin[f]);
+                        atomicAdd(target + lf * row + e, __builtin_nontemporal_load(&lin[f]));
                     } else {
                         tr.data[lf * row + e] = lin[f];
                     }
