@@ -113,6 +113,19 @@ def test_every_image_path_against_the_oracle(gpu, oracle_mod, case):
                     check_grad(f"{tag}: marching se_grad hessian", got[2], want_se[2])
             finally:
                 C.set_debug_flags(0)
+    # the one-ray-per-lane kernels on the same pictures (debug flag 1): forward, gradient and se_grad
+    C.set_debug_flags(1)
+    try:
+        if not np.array_equal(C.volume_render_images(plain, cam, opt).cpu().numpy(), want):
+            failures.append("generic: picture differs")
+        check_grad("generic: gradient", C.volume_render_images_backward(plain, cam, opt, go.to(gpu), workspace=False), want_g)
+        got = C.se_grad_persp(plain, cam1, opt, ref.to(gpu), workspace=False)
+        if not np.array_equal(got[0].cpu().numpy(), want_se[0]):
+            failures.append("generic: se_grad colour differs")
+        check_grad("generic: se_grad gradient", got[1], want_se[1])
+        check_grad("generic: se_grad hessian", got[2], want_se[2])
+    finally:
+        C.set_debug_flags(0)
     assert not failures, f"case {case} {p}: " + "; ".join(failures)
 
 

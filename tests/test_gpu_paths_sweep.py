@@ -99,6 +99,10 @@ def test_every_render_path_against_the_exact_sum_oracle(gpu, oracle_mod, case):
     combos += list(itertools.product((4, 8), ((plain, "plain"), (marked, "marked")), ("fwd", "noted", "se")))
     combos += list(itertools.product((0, 2, 4, 8), ((decided, "decided"),), ("fwd",)))
     combos += list(itertools.product((0,), ((decided, "decided"),), ("bwd", "noted", "se")))
+    # the one-ray-per-lane kernels (what fp64 trees, partial component ranges and the other record shapes run on),
+    # forced onto the same fp32 cases: forward, the gradient kernel and se_grad, whose wavefronts add the records
+    # of a step together
+    combos += list(itertools.product((1,), ((plain, "plain"),), ("fwd", "bwd_nows", "se_nows")))
     for flags, (spec, spec_name), name in combos:
         tag = f"{name}/flags{flags}/{spec_name}"
         C.set_debug_flags(flags)
