@@ -700,7 +700,7 @@ def main():
         generic["note"] = ("fp32 SH, SG and ASG records of 1, 4, 9, 16 or 25 basis functions run on the wavefront-per-tile kernels, "
                            "for any branching factor and with or without density_softplus "
                            "(`..._generic_kernel_ms`: the same call forced onto the one-ray-per-lane kernels, which "
-                           "serve fp64, partial component ranges and the other record shapes)")
+                           "serve fp64 and the other record shapes)")
         del sgtree
         gtree64 = gtree.double()
         g64cam = _make_camera_spec(poses[0].double().contiguous(), W, H, fx, fx)

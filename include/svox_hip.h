@@ -369,8 +369,8 @@ int svox_volume_render_stats(const SvoxTreeSpec* tree, const SvoxRaysSpec* rays,
 /* No counterpart in the reference.  Which family of kernels serves the render calls of this tree under
  * these options (forward, backward and se_grad alike, with or without density_softplus): 1 the
  * wavefront-per-tile kernels (fp32, any branching factor, fewer than 2^30 cells, RGBA / SH / SG / ASG records
- * with basis_dim 1, 4, 9, 16 or 25 and the full component range), 0 the one-ray-per-lane kernels that cover
- * everything else the reference accepts (fp64, other basis sizes and record shapes, partial component ranges), or
+ * with basis_dim 1, 4, 9, 16 or 25, any range of components), 0 the one-ray-per-lane kernels that cover
+ * everything else the reference accepts (fp64, other basis sizes and record shapes), or
  * a negative SvoxStatus for a tree or options no kernel accepts.  Results do not depend on the family. */
 int svox_octree_kernels_serve(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt);
 

@@ -750,9 +750,9 @@ def volume_render_stats(tree, rays_or_cam, opt):
 
 
 def octree_kernels_serve(tree, opt):
-    """True where the wavefront-per-tile octree kernels serve the render calls of `tree` under `opt` (forward,
-    backward, se_grad, with or without density_softplus), False where the one-ray-per-lane kernels do (fp64,
-    N != 2, other basis sizes, partial component ranges)."""
+    """True where the wavefront-per-tile kernels serve the render calls of `tree` under `opt` (forward, backward,
+    se_grad, with or without density_softplus, any branching factor, any range of components), False where the
+    one-ray-per-lane kernels do (fp64, other basis sizes and record shapes)."""
     spec = _pack_tree(tree)
     copt = opt._pack()
     rc = _abi.load_library().svox_octree_kernels_serve(ctypes.byref(spec), ctypes.byref(copt))

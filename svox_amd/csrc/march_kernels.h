@@ -415,14 +415,34 @@ struct Lobes {
     int cols;
     int format;
 };
-// The basis of one ray (maybe_precalc_basis, rt_kernel.cu:111-187) for the policy's format.
+// A launch that renders only the components [min_comp, max_comp] of the basis (rt_kernel.cu:286-288: the loops over
+// the coefficients run over that range) runs on the kernels that keep a ray's basis as a row in LDS (the lobe
+// policy, whatever the format: its rows are made by precalc_basis, which knows spherical harmonics too), with the
+// row zero outside the range: the full-length colour sums then add 0 * coefficient = 0 for the terms the reference
+// leaves out, which leaves the running sum as it is -- the same bits for every finite coefficient (a coefficient
+// that is infinite or NaN outside the range would show here and not in the reference) -- and the gradient terms
+// of those components are zeros added to zeros.
+template <int D>
+__device__ __forceinline__ bool partial_range(const SvoxRenderOptions& opt) {
+    return opt.min_comp > 0 || opt.max_comp < D - 1;   // (uniform: the same for every lane of the launch)
+}
+template <int D>
+__device__ __forceinline__ void keep_range(const SvoxRenderOptions& opt, float* x) {
+#pragma unroll
+    for (int i = 0; i < D; ++i) x[i] = (i >= opt.min_comp && i <= opt.max_comp) ? x[i] : 0.0f;
+}
+
+// The basis of one ray (maybe_precalc_basis, rt_kernel.cu:111-187) for the policy's format, zero outside the
+// launch's component range.
 template <class P>
-__device__ __forceinline__ void policy_basis(const Lobes& lobes, const float* vdir, float* out) {
+__device__ __forceinline__ void policy_basis(const Lobes& lobes, const SvoxRenderOptions& opt, const float* vdir,
+                                             float* out) {
     if constexpr (P::kFormat == SVOX_FORMAT_SH) {
         sh_basis<float>(P::kBasis, vdir, out);
     } else {
         precalc_basis<float>(lobes.format, P::kBasis, lobes.table, lobes.cols, vdir, out);
     }
+    if (partial_range<P::kBasis>(opt)) keep_range<P::kBasis>(opt, out);
 }
 
 // atomicMax of the reference (common.cuh:152-172): compare-and-swap loop around fmaxf
@@ -511,28 +531,6 @@ __device__ void trace_generic(const TreeDev<T>& tr, const SvoxRenderOptions& opt
     if (!stopped)
         for (int j = 0; j < out_dim; ++j) acc[j * S] = fma_(light, (T)opt.background_brightness, acc[j * S]);
     for (int j = 0; j < out_dim; ++j) out[j] = acc[j * S];
-}
-
-// colour of one leaf record for the octree flavour: 3 sigmoids of basis . coefficients.
-// `basis` is read with stride `kStride` (1: a register array, 64: this lane's column of an LDS array
-// laid out [coefficient][lane], which 64 lanes read without bank conflicts).
-template <class P, int kStride>
-__device__ __forceinline__ void leaf_colour(const float* __restrict__ rec, const float* basis, float* s) {
-    if constexpr (P::kFormat == SVOX_FORMAT_RGBA) {
-#pragma unroll
-        for (int c = 0; c < 3; ++c) s[c] = sigmoid_(rec[c]);
-    } else {
-        float b[P::kBasis];
-#pragma unroll
-        for (int i = 0; i < P::kBasis; ++i) b[i] = basis[i * kStride];
-#pragma unroll
-        for (int c = 0; c < 3; ++c) {
-            float tmp = 0.0f;
-#pragma unroll
-            for (int i = 0; i < P::kBasis; ++i) tmp = fma_(b[i], rec[c * P::kBasis + i], tmp);
-            s[c] = sigmoid_(tmp);
-        }
-    }
 }
 
 // number of set bits of `mask` below this lane
@@ -1000,7 +998,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_forward_kernel(TreeDev<f
                 sh.vdir[lane * 3 + 2] = vdir[2];
             } else if constexpr (P::kForwardRows) {
                 float basis[D];
-                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, vdir, basis);
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, opt, vdir, basis);
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
@@ -1721,7 +1719,7 @@ __global__ __launch_bounds__(kSplitThreads) void render_forward_split_kernel(Tre
             } else if constexpr (P::kForwardRows) {
                 if (active) {
                     float basis[D];
-                    policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, vdir, basis);
+                    policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, opt, vdir, basis);
 #pragma unroll
                     for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
                 }
@@ -1948,7 +1946,7 @@ __global__ __launch_bounds__(kMarchThreads) void render_backward_kernel(TreeDev<
             }
             if constexpr (P::kFormat != SVOX_FORMAT_RGBA) {
                 float basis[D];
-                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, vdir, basis);
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, opt, vdir, basis);
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
@@ -2111,7 +2109,7 @@ __global__ __launch_bounds__(kMarchThreads) __attribute__((amdgpu_waves_per_eu(3
             float vdir[3];
             src.view_dir(ray, vdir);
             float basis[D];
-            policy_basis<P>(lobes, vdir, basis);
+            policy_basis<P>(lobes, opt, vdir, basis);
 #pragma unroll
             for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
         }
@@ -2445,7 +2443,7 @@ __global__ __launch_bounds__(kMarchThreads) void se_grad_kernel(TreeDev<float> t
         if (setup_ray(r, origin, dir, scaling)) {
             if constexpr (P::kFormat != SVOX_FORMAT_RGBA) {
                 float basis[D];
-                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, vdir, basis);
+                policy_basis<P>(Lobes{tr.extra, tr.extra_cols, opt.format}, opt, vdir, basis);
 #pragma unroll
                 for (int i = 0; i < D; ++i) sh.basis[lane * D + i] = basis[i];
             }
@@ -2677,7 +2675,7 @@ __global__ __launch_bounds__(kMarchThreads) void replay_se_grad_kernel(Source sr
             float vdir[3];
             src.view_dir(ray, vdir);
             float basis[D];
-            policy_basis<P>(lobes, vdir, basis);
+            policy_basis<P>(lobes, opt, vdir, basis);
 #pragma unroll
             for (int i = 0; i < D; ++i) basis_rows[lane * D + i] = basis[i];
         }

@@ -229,7 +229,12 @@ int fast_basis(const SvoxTreeSpec* tree, const SvoxRenderOptions* opt) {
     if (opt->format != SVOX_FORMAT_SH && opt->format != SVOX_FORMAT_SG && opt->format != SVOX_FORMAT_ASG) return -1;
     const int D = opt->basis_dim;
     if (D != 1 && D != 4 && D != 9 && D != 16 && D != 25) return -1;
-    if (tree->data_dim != 3 * D + 1 || opt->min_comp != 0 || opt->max_comp != D - 1) return -1;
+    if (tree->data_dim != 3 * D + 1 || opt->min_comp < 0 || opt->max_comp > D - 1) return -1;
+    // A range of components narrower than the basis runs on the kernels that keep a ray's basis as a row in LDS (the
+    // lobe policy: its rows come from precalc_basis, for spherical harmonics too), the row zero outside the range;
+    // min_comp > max_comp is the reference's empty range, mid grey.
+    const bool partial = opt->min_comp > 0 || opt->max_comp < D - 1;
+    if (opt->format == SVOX_FORMAT_SH && partial) return kLobeKernels + D;
     if (opt->format != SVOX_FORMAT_SH) {
         // lobes: the table must be there, [lambda, mu] per spherical gaussian (rt_kernel.cu:133-139),
         // [lambda_x, lambda_y, three axes] per anisotropic one (rt_kernel.cu:120-131)

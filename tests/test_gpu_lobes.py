@@ -86,15 +86,16 @@ def test_lobes_on_the_octree_kernels(gpu, oracle_mod, kind, n_lobes):
 
 
 def test_which_kernels_serve_which_trees(gpu):
-    """The octree kernels take fp32 octrees with RGBA, SH, SG or ASG records of 1, 4, 9, 16 or 25 basis
-    functions and the full component range; everything else goes to the one-ray-per-lane kernels."""
+    """The wavefront-per-tile kernels take fp32 trees with RGBA, SH, SG or ASG records of 1, 4, 9, 16 or 25 basis
+    functions, for any range of components; everything else goes to the one-ray-per-lane kernels."""
     def serve(tree, **kw):
         dev = on_gpu(tree, gpu)
         return C.octree_kernels_serve(dev._spec(), options(tree, **kw))
     assert serve(synth.dense_tree(2, "RGBA", seed=1))
     assert serve(synth.dense_tree(2, "SH9", seed=1))
     assert serve(synth.dense_tree(2, "SH9", seed=1), density_softplus=True)
-    assert not serve(synth.dense_tree(2, "SH9", seed=1), min_comp=1, max_comp=3)
+    assert serve(synth.dense_tree(2, "SH9", seed=1), min_comp=1, max_comp=3)
+    assert serve(synth.dense_tree(2, "SH9", seed=1), min_comp=2, max_comp=1)         # the empty range: mid grey
     assert not serve(synth.dense_tree(2, "SH4", seed=1, dtype=torch.float64))
     assert serve(lobe_tree(9, seed=2, depth=4))
     assert not serve(lobe_tree(5, seed=2, depth=4))                       # no kernel built for five lobes

@@ -164,16 +164,85 @@ def test_generic_options_double_and_lobes(gpu, oracle_mod):
     for name, tree, kw, dt in cases:
         r = svox.Rays(rays.origins.to(dt), rays.dirs.to(dt), rays.viewdirs.to(dt))
         opt = options(tree, step_size=2e-3, **kw)
-        out, ref, stats, ref_stats, dev, ot = render_both(gpu, oracle_mod, tree, r, opt)
-        if "softplus" in name:
-            assert np.abs(out - ref).max() <= 1e-5, name    # logf comes from two math libraries
+        for generic in (0, 1):       # the kernels the library picks, then the one-ray-per-lane kernels for every case
+            out, ref, stats, ref_stats, dev, ot = render_both(gpu, oracle_mod, tree, r, opt, generic)
+            if "softplus" in name:
+                assert np.abs(out - ref).max() <= 1e-5, name    # logf comes from two math libraries
+            else:
+                assert np.array_equal(out, ref), (name, generic)
+            go = torch.randn(out.shape, generator=torch.Generator().manual_seed(1), dtype=dt)
+            ref_grad = oracle_mod.volume_render_backward(ot, r.origins, r.dirs, r.viewdirs, opt, go)
+            C.set_debug_flags(generic)
+            try:
+                grad = C.volume_render_backward(dev._spec(), rays_spec(r, gpu), opt, go.to(gpu))
+            finally:
+                C.set_debug_flags(0)
+            err, ok = grad_close(grad.cpu().numpy(), ref_grad, what=f"{name} generic {generic}")
+            assert ok, (name, generic, err)
+
+
+@pytest.mark.parametrize("fmt,lo,hi", [("SH9", 1, 3), ("SH9", 2, 1), ("SH16", 4, 15), ("SH4", 0, 0), ("SG9", 2, 6),
+                                       ("ASG4", 1, 2)])
+def test_component_ranges_on_the_wavefront_kernels(gpu, oracle_mod, fmt, lo, hi):
+    """A range of basis components (rt_kernel.cu:286-288; min_comp > max_comp renders mid grey) on the wavefront-per-tile
+    kernels: every call -- forward on one and two wavefronts per tile, noted forward and replay, marching backward with
+    and without a workspace, se_grad from notes and marching, an image and its gradient -- against the oracle."""
+    g = torch.Generator().manual_seed(21)
+    if fmt.startswith("SH"):
+        tree = synth.shell_tree(depth=5, n_spheres=4, data_format=fmt, seed=4, sigma_range=(5.0, 80.0))
+    else:
+        n = int(fmt[-1])
+        if fmt.startswith("SG"):
+            extra = torch.cat([torch.rand(n, 1, generator=g) * 4 + 0.5, synth.unit_vectors(n, g)], dim=1)
         else:
-            assert np.array_equal(out, ref), name
-        go = torch.randn(out.shape, generator=torch.Generator().manual_seed(1), dtype=dt)
-        ref_grad = oracle_mod.volume_render_backward(ot, r.origins, r.dirs, r.viewdirs, opt, go)
-        grad = C.volume_render_backward(dev._spec(), rays_spec(r, gpu), opt, go.to(gpu))
-        err, ok = grad_close(grad.cpu().numpy(), ref_grad)
-        assert ok, (name, err)
+            frames = torch.linalg.qr(torch.randn(n, 3, 3, generator=g))[0].reshape(n, 9)
+            extra = torch.cat([torch.rand(n, 2, generator=g) * 3, frames], 1)
+        tree = svox.N3Tree(data_format=fmt, init_refine=3, extra_data=extra)
+        tree.data.data.normal_(0, 0.7, generator=g)
+        tree.data.data[..., -1] = tree.data.data[..., -1].abs() * 6 * (torch.rand(tree.child.shape, generator=g) < 0.6)
+    rays = synth.sphere_rays(1200, seed=13)
+    opt = options(tree, step_size=2e-3, min_comp=lo, max_comp=hi)
+    ot = oracle_mod.Tree.from_n3tree(tree)
+    dev = on_gpu(tree, gpu)
+    assert C.octree_kernels_serve(dev._spec(), opt) == 1
+    rs = rays_spec(rays, gpu)
+    want = oracle_mod.volume_render(ot, rays.origins, rays.dirs, rays.viewdirs, opt)
+    go = torch.randn(1200, 3, generator=g) * 1e-2
+    want_g = oracle_mod.volume_render_backward(ot, rays.origins, rays.dirs, rays.viewdirs, opt, go)
+    ref = torch.rand(1200, 3, generator=g)
+    want_se = oracle_mod.se_grad(ot, rays.origins, rays.dirs, rays.viewdirs, ref, opt, n_threads=8)
+    for flags in (0, 2, 4, 8):
+        C.set_debug_flags(flags)
+        try:
+            assert np.array_equal(C.volume_render(dev._spec(), rs, opt).cpu().numpy(), want), flags
+            out, notes = C.volume_render_noted(dev._spec(), rs, opt)
+            assert notes is not None and np.array_equal(out.cpu().numpy(), want), flags
+            err, ok = grad_close(C.volume_render_backward_noted(dev._spec(), rs, opt, go.to(gpu), notes).cpu().numpy(),
+                                 want_g, what=f"range notes flags {flags}")
+            assert ok, (flags, err)
+            for workspace in (True, False):
+                err, ok = grad_close(C.volume_render_backward(dev._spec(), rs, opt, go.to(gpu),
+                                                              workspace=workspace).cpu().numpy(), want_g,
+                                     what=f"range backward flags {flags} workspace {workspace}")
+                assert ok, (flags, workspace, err)
+                got = C.se_grad(dev._spec(), rs, ref.to(gpu), opt, workspace=workspace)
+                assert np.array_equal(got[0].cpu().numpy(), want_se[0]), (flags, workspace)
+                for what, x, w in zip(("gradient", "hessian"), got[1:], want_se[1:3]):
+                    err, ok = grad_close(x.cpu().numpy(), w, what=f"range se_grad {what} flags {flags}")
+                    assert ok, (flags, workspace, what, err)
+        finally:
+            C.set_debug_flags(0)
+    # one picture and its gradient through the image kernels
+    W, H, fx = 48, 40, 60.0
+    c2w = synth.orbit_poses(1, seed=3, radius=2.5)[0]
+    want_img = oracle_mod.volume_render_image(ot, c2w, fx, fx, W, H, opt)
+    cam = cam_spec(c2w.to(gpu), W, H, fx)
+    assert np.array_equal(C.volume_render_image(dev._spec(), cam, opt).cpu().numpy(), want_img)
+    go_img = torch.randn(H, W, 3, generator=g) * 1e-2
+    want_gi = oracle_mod.volume_render_image_backward(ot, c2w, fx, fx, W, H, opt, go_img)
+    err, ok = grad_close(C.volume_render_image_backward(dev._spec(), cam, opt, go_img.to(gpu)).cpu().numpy(), want_gi,
+                         what="range image gradient")
+    assert ok, err
 
 
 def irregular_tree(N, fmt, seed, rounds=3):
@@ -1113,8 +1182,8 @@ def test_gradient_gate_without_order_slack(gpu, oracle_mod, fmt):
 
 
 def test_notes_are_kept_only_where_they_are_taken(gpu):
-    """A renderer whose tree or options the noting kernels do not serve (fp64 records, a partial component range, a
-    negative sigma_thresh) runs the plain forward pass: no workspace is allocated, the autograd context keeps nothing, and
+    """A renderer whose tree or options the noting kernels do not serve (fp64 records, a negative sigma_thresh) runs
+    the plain forward pass: no workspace is allocated, the autograd context keeps nothing, and
     the notes budget never looks at a counter nobody wrote."""
     from svox_amd import renderer as R
     rays = synth.sphere_rays(500, seed=1)
@@ -1133,7 +1202,7 @@ def test_notes_are_kept_only_where_they_are_taken(gpu):
         t3.data.data.normal_()
         t3.data.data[..., -1].abs_()
         cases.append((svox.VolumeRenderer(t3, step_size=1e-2), True))         # (N = 3 runs on the same kernels)
-        cases.append((svox.VolumeRenderer(t3, step_size=1e-2, max_comp=2), False))
+        cases.append((svox.VolumeRenderer(t3, step_size=1e-2, max_comp=2), True))     # (and so does a range of components)
         t64 = on_gpu(synth.dense_tree(2, "SH4", seed=1, sigma="lognormal", dtype=torch.float64), gpu)
         cases.append((svox.VolumeRenderer(t64, step_size=1e-2), False))
         t2 = on_gpu(synth.dense_tree(3, "SH4", seed=0, sigma="lognormal"), gpu)
